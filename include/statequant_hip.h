@@ -1,0 +1,146 @@
+/* C ABI of libsqhip.so: the packed recurrent-state decode step on one MI355X (gfx950).
+ *
+ * Every entry point takes plain device pointers, element strides and sizes; nothing here allocates, frees, retains
+ * a pointer or synchronizes.  Work is enqueued on the HIP stream passed as `stream` (a hipStream_t; NULL = the null
+ * stream), so calls are safe under HIP graph capture.  Return value: 0 on success, otherwise a negative SQ_E_* code
+ * (sq_strerror() names it; sq_last_error() gives the detail of the last failure on the calling thread).
+ *
+ * The entry points replace the Triton launch sites of the reference (paths relative to
+ * /root/reference/src/statequant/kernels/):
+ *   sq_gdn_step     _fused_triton.py:48 `_fused_step`, launched from fold.py:400-408 (lockstep) and
+ *                   slots.py:178-187 (slot-addressed)
+ *   sq_kda_step     _kda_triton.py:38 `_kda_step`, launched from kda.py:192-205
+ *   sq_mamba2_step  _mamba2_triton.py:48 `_m2_step`, launched from mamba2.py:223-241
+ * The argument convention is the reference's (_fold_triton.py:30-36): every per-sequence tensor comes as a base
+ * pointer plus its per-sequence stride IN ELEMENTS of that tensor's type; batch row b works on sequence idx[b]
+ * (idx == NULL: sequence b); rows with idx[b] <= 0 are padding: their output row is zeroed, nothing else is touched.
+ */
+#ifndef STATEQUANT_HIP_H
+#define STATEQUANT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SQ_ABI_VERSION 1
+
+enum { SQ_F32 = 0, SQ_BF16 = 1, SQ_F16 = 2 };                /* dtype codes of float tensors */
+
+enum {
+    SQ_OK = 0,
+    SQ_E_ARG = -1,          /* a null pointer, bad stride / alignment or inconsistent sizes */
+    SQ_E_UNSUPPORTED = -2,  /* a (bits, axis, group, d_k, d_v, m, buffer) combination no kernel is built for */
+    SQ_E_LAUNCH = -3        /* the HIP runtime refused the launch (sq_last_error() holds hipGetErrorString) */
+};
+
+/* The stored state and decode buffer of a set of sequences (slots.py:9-22 for the field meanings and shapes).
+ * S     codes: int8 [hv, dv, dk] (bits 8) or uint8 [hv, dv, dk/2] (bits 4, byte j = (c[2j]+8) | (c[2j+1]+8) << 4)
+ * SC    fp16 scales [hv, dv, ceil(dk/group)] (key-axis groups)
+ * KB    buffered keys [hk, m, dk], int8 (buffer_bits 8) or bf16 (16);  KBS fp16 [hk, m] (int8 buffer only)
+ * UB    buffered delta values [hv, m, dv], int8 or bf16;               UBS fp16 [hv, m] (int8 buffer only)
+ * GB    fp32 cumulative log decay of each buffered token: [hv, m] (GDN, Mamba2) or [hv, m, dk] (KDA)
+ * GCUR  fp32 running log decay since the last fold: [hv] or [hv, dk] (KDA)
+ * NPTR  int32 buffer fill counter, one copy per value head: element h of a sequence belongs to head h */
+typedef struct sq_state {
+    void* S;        int64_t sS;
+    void* SC;       int64_t sSC;
+    void* KB;       int64_t sKB;
+    void* KBS;      int64_t sKBS;
+    void* UB;       int64_t sUB;
+    void* UBS;      int64_t sUBS;
+    float* GB;      int64_t sGB;
+    float* GCUR;    int64_t sGC;
+    int32_t* NPTR;  int64_t sN;
+} sq_state;
+
+/* Layer geometry and storage format (fold.py:91-104 `packed_format`, slots.py:53-74). */
+typedef struct sq_layout {
+    int32_t bits;         /* 4 or 8 */
+    int32_t axis_k;       /* 1: scale groups along d_k (the only axis built so far) */
+    int32_t group;        /* scale group length, a power of two */
+    int32_t buffer_bits;  /* 8 (int8 + fp16 scale per vector) or 16 (bf16) */
+    int32_t m;            /* buffer length, a power of two */
+    int32_t hv, hk;       /* value heads, key heads (groups); hv % hk == 0 */
+    int32_t dk, dv;       /* head dims */
+} sq_layout;
+
+/* One Gated DeltaNet decode token per batch row (fold.py:381-408, slots.py:124-187).
+ * q, k   [rows, hk, dk] (qk_per_key_head = 1) or [rows, hv, dk] (0), raw; l2-normalised in the kernel
+ * v      [rows, hv, dv];  out [rows, hv, dv] contiguous
+ * gate = 0: g, beta [rows, hv] (log decay, sigmoided beta)
+ * gate = 1: a, b [rows, hv], A_log, dt_bias [hv]: g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b)
+ * Row strides (s_*) are in elements; inner dims are contiguous. */
+typedef struct sq_gdn_args {
+    sq_state st;
+    sq_layout lay;
+    int32_t rows;
+    const int32_t* idx;
+    const void* q;      int64_t s_q;     int32_t q_dtype;
+    const void* k;      int64_t s_k;     int32_t k_dtype;
+    const void* v;      int64_t s_v;     int32_t v_dtype;
+    int32_t qk_per_key_head;
+    int32_t gate;
+    const void* g;      int64_t s_g;     int32_t g_dtype;
+    const void* beta;   int64_t s_beta;  int32_t beta_dtype;
+    const void* a;      int64_t s_a;     int32_t a_dtype;
+    const void* b;      int64_t s_b;     int32_t b_dtype;
+    const void* A_log;  int32_t A_log_dtype;
+    const void* dt_bias; int32_t dt_bias_dtype;
+    void* out;          int32_t out_dtype;
+    float scale;
+} sq_gdn_args;
+
+/* One KDA decode token per batch row (kda.py:192-205, 330-347): per-key-channel log decay g [rows, hv, dk];
+ * hk == hv.  q, k [rows, hv, dk], v [rows, hv, dv], beta [rows, hv], out [rows, hv, dv] with row stride s_out. */
+typedef struct sq_kda_args {
+    sq_state st;
+    sq_layout lay;
+    int32_t rows;
+    const int32_t* idx;
+    const void* q;      int64_t s_q;     int32_t q_dtype;
+    const void* k;      int64_t s_k;     int32_t k_dtype;
+    const void* v;      int64_t s_v;     int32_t v_dtype;
+    const void* g;      int64_t s_g;     int32_t g_dtype;
+    const void* beta;   int64_t s_beta;  int32_t beta_dtype;
+    void* out;          int64_t s_out;   int32_t out_dtype;
+    float scale;
+} sq_kda_args;
+
+/* One Mamba2 / SSD decode token per batch row (mamba2.py:223-241, 377-396).
+ * x [rows, hv, dv], dt [rows, hv] raw, B / C [rows, hk, dk] (hk = groups), A [hv], D / dt_bias [hv] or NULL,
+ * out [rows, hv, dv] with row stride s_out.  dt <- dt + dt_bias; softplus (threshold 20) if dt_softplus;
+ * clamped to [dt_min, dt_max] if dt_clamp. */
+typedef struct sq_mamba2_args {
+    sq_state st;
+    sq_layout lay;
+    int32_t rows;
+    const int32_t* idx;
+    const void* x;      int64_t s_x;     int32_t x_dtype;
+    const void* dt;     int64_t s_dt;    int32_t dt_dtype;
+    const void* B;      int64_t s_B;     int32_t B_dtype;
+    const void* C;      int64_t s_C;     int32_t C_dtype;
+    const void* A;      int32_t A_dtype;
+    const void* D;      int32_t D_dtype;
+    const void* dt_bias; int32_t dt_bias_dtype;
+    int32_t dt_softplus;
+    int32_t dt_clamp;   float dt_min, dt_max;
+    void* out;          int64_t s_out;   int32_t out_dtype;
+} sq_mamba2_args;
+
+int sq_abi_version(void);
+const char* sq_strerror(int code);
+const char* sq_last_error(void);
+
+/* 1 if a kernel is built for this layout (family: 0 GDN, 1 KDA, 2 Mamba2), else 0. Pure host code. */
+int sq_supported(int family, const sq_layout* lay);
+
+int sq_gdn_step(const sq_gdn_args* args, void* stream);
+int sq_kda_step(const sq_kda_args* args, void* stream);
+int sq_mamba2_step(const sq_mamba2_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STATEQUANT_HIP_H */

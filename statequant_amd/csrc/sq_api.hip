@@ -1,0 +1,218 @@
+// extern "C" surface of libsqhip.so (declared in include/statequant_hip.h): argument validation, translation of the
+// public structs into kernel parameter blocks, error reporting.  No allocation, no synchronization.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/statequant_hip.h"
+#include "sq_params.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool pow2(int n) { return n > 0 && (n & (n - 1)) == 0; }
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+bool dtype_ok(int d) { return d == SQ_F32 || d == SQ_BF16 || d == SQ_F16; }
+
+// Geometry / format checks shared by the three families; fills the LayoutKey part of a parameter block.
+int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
+    if (L.bits != 4 && L.bits != 8) return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4 or 8, got %d", who, L.bits);
+    if (!L.axis_k) return fail(SQ_E_UNSUPPORTED, "%s: value-axis scale groups are not built", who);
+    if (!pow2(L.group)) return fail(SQ_E_ARG, "%s: group %d is not a power of two", who, L.group);
+    if (L.buffer_bits != 8 && L.buffer_bits != 16)
+        return fail(SQ_E_ARG, "%s: buffer_bits must be 8 or 16, got %d", who, L.buffer_bits);
+    if (!pow2(L.m) || L.m > 32) return fail(SQ_E_ARG, "%s: m must be a power of two <= 32, got %d", who, L.m);
+    if (L.hv <= 0 || L.hk <= 0 || L.hv % L.hk) return fail(SQ_E_ARG, "%s: hv %d, hk %d", who, L.hv, L.hk);
+    if (L.dk <= 0 || L.dv <= 0 || (L.dk & 1)) return fail(SQ_E_ARG, "%s: dk %d, dv %d", who, L.dk, L.dv);
+    key->bits = L.bits;
+    key->group = L.group;
+    key->qbuf = L.buffer_bits == 8;
+    key->m = L.m;
+    key->hv = L.hv;
+    key->hk = L.hk;
+    key->dk = L.dk;
+    key->dv = L.dv;
+    return SQ_OK;
+}
+
+// Pointers, strides and alignment of the stored state.  The kernels read a lane's piece of a code row with one
+// 128-bit (int8) or 64-bit (int4) load and a piece of a buffered int8 key with one 128-bit load.
+int check_state(const sq_state& s, const sq_layout& L, const char* who, sq::StatePtrs* st) {
+    if (!s.S || !s.SC || !s.KB || !s.UB || !s.GB || !s.GCUR || !s.NPTR)
+        return fail(SQ_E_ARG, "%s: null state pointer", who);
+    if (L.buffer_bits == 8 && (!s.KBS || !s.UBS)) return fail(SQ_E_ARG, "%s: int8 buffer without scales", who);
+    const size_t row_align = L.bits == 8 ? 16 : 8;
+    if (!aligned(s.S, row_align) || (s.sS % int64_t(row_align)))
+        return fail(SQ_E_ARG, "%s: codes must be %zu-byte aligned (base and per-sequence stride)", who, row_align);
+    if (L.buffer_bits == 8 && (!aligned(s.KB, 16) || (s.sKB % 16)))
+        return fail(SQ_E_ARG, "%s: int8 key buffer must be 16-byte aligned (base and per-sequence stride)", who);
+    if (!aligned(s.SC, 2) || !aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
+        return fail(SQ_E_ARG, "%s: misaligned scale / decay / counter pointer", who);
+    st->S = static_cast<uint8_t*>(s.S);         st->sS = s.sS;
+    st->SC = static_cast<uint16_t*>(s.SC);      st->sSC = s.sSC;
+    st->KB = static_cast<uint8_t*>(s.KB);       st->sKB = s.sKB;
+    st->KBS = static_cast<uint16_t*>(s.KBS);    st->sKBS = s.sKBS;
+    st->UB = static_cast<uint8_t*>(s.UB);       st->sUB = s.sUB;
+    st->UBS = static_cast<uint16_t*>(s.UBS);    st->sUBS = s.sUBS;
+    st->GB = s.GB;                              st->sGB = s.sGB;
+    st->GCUR = s.GCUR;                          st->sGC = s.sGC;
+    st->NPTR = s.NPTR;                          st->sN = s.sN;
+    return SQ_OK;
+}
+
+int finish(int rc, const char* who, const sq_layout& L) {
+    if (rc == 0) return SQ_OK;
+    if (rc == -1)
+        return fail(SQ_E_UNSUPPORTED, "%s: no kernel built for int%d group %d, d_k %d, d_v %d, m %d, buffer_bits %d",
+                    who, L.bits, L.group, L.dk, L.dv, L.m, L.buffer_bits);
+    return fail(SQ_E_LAUNCH, "%s: %s", who, hipGetErrorString(hipError_t(rc)));
+}
+
+#define SQ_TRY(expr)              \
+    do {                          \
+        const int rc_ = (expr);   \
+        if (rc_ != SQ_OK) return rc_; \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int sq_abi_version(void) { return SQ_ABI_VERSION; }
+
+const char* sq_strerror(int code) {
+    switch (code) {
+        case SQ_OK: return "ok";
+        case SQ_E_ARG: return "invalid argument";
+        case SQ_E_UNSUPPORTED: return "unsupported layout";
+        case SQ_E_LAUNCH: return "kernel launch failed";
+        default: return "unknown error";
+    }
+}
+
+const char* sq_last_error(void) { return g_err; }
+
+int sq_supported(int family, const sq_layout* lay) {
+    if (!lay) return 0;
+    sq::LayoutKey key;
+    if (check_layout(*lay, "sq_supported", &key) != SQ_OK) return 0;
+    if (family == 0) {
+        sq::GdnParams p{};
+        static_cast<sq::LayoutKey&>(p) = key;
+        return sq::dispatch_gdn(p, nullptr, false) == 0;
+    }
+    if (family == 1) {
+        sq::KdaParams p{};
+        static_cast<sq::LayoutKey&>(p) = key;
+        return sq::dispatch_kda(p, nullptr, false) == 0;
+    }
+    if (family == 2) {
+        sq::Mamba2Params p{};
+        static_cast<sq::LayoutKey&>(p) = key;
+        return sq::dispatch_mamba2(p, nullptr, false) == 0;
+    }
+    return 0;
+}
+
+int sq_gdn_step(const sq_gdn_args* a, void* stream) {
+    const char* who = "sq_gdn_step";
+    if (!a) return fail(SQ_E_ARG, "%s: null args", who);
+    sq::GdnParams p{};
+    SQ_TRY(check_layout(a->lay, who, &p));
+    if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
+    if (a->rows == 0) return SQ_OK;
+    SQ_TRY(check_state(a->st, a->lay, who, &p.st));
+    if (!a->q || !a->k || !a->v || !a->out) return fail(SQ_E_ARG, "%s: null q / k / v / out", who);
+    if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->out_dtype))
+        return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    if (a->gate) {
+        if (!a->a || !a->b || !a->A_log || !a->dt_bias) return fail(SQ_E_ARG, "%s: gate without a / b / A_log / dt_bias", who);
+        if (!dtype_ok(a->a_dtype) || !dtype_ok(a->b_dtype) || !dtype_ok(a->A_log_dtype) || !dtype_ok(a->dt_bias_dtype))
+            return fail(SQ_E_ARG, "%s: bad gate dtype code", who);
+    } else {
+        if (!a->g || !a->beta) return fail(SQ_E_ARG, "%s: neither g / beta nor a gate", who);
+        if (!dtype_ok(a->g_dtype) || !dtype_ok(a->beta_dtype)) return fail(SQ_E_ARG, "%s: bad g / beta dtype code", who);
+    }
+    p.rows = a->rows;
+    p.idx = a->idx;
+    p.q = a->q; p.s_q = a->s_q; p.q_dt = a->q_dtype;
+    p.k = a->k; p.s_k = a->s_k; p.k_dt = a->k_dtype;
+    p.v = a->v; p.s_v = a->s_v; p.v_dt = a->v_dtype;
+    p.qk_per_key_head = a->qk_per_key_head != 0;
+    p.gate = a->gate != 0;
+    p.g = a->g; p.s_g = a->s_g; p.g_dt = a->g_dtype;
+    p.beta = a->beta; p.s_beta = a->s_beta; p.beta_dt = a->beta_dtype;
+    p.a = a->a; p.s_a = a->s_a; p.a_dt = a->a_dtype;
+    p.bt = a->b; p.s_bt = a->s_b; p.bt_dt = a->b_dtype;
+    p.A_log = a->A_log; p.A_log_dt = a->A_log_dtype;
+    p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    p.out = a->out; p.out_dt = a->out_dtype;
+    p.scale = a->scale;
+    return finish(sq::dispatch_gdn(p, static_cast<hipStream_t>(stream), true), who, a->lay);
+}
+
+int sq_kda_step(const sq_kda_args* a, void* stream) {
+    const char* who = "sq_kda_step";
+    if (!a) return fail(SQ_E_ARG, "%s: null args", who);
+    sq::KdaParams p{};
+    SQ_TRY(check_layout(a->lay, who, &p));
+    if (a->lay.hk != a->lay.hv) return fail(SQ_E_ARG, "%s: KDA has no grouped keys (hk %d != hv %d)", who, a->lay.hk, a->lay.hv);
+    if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
+    if (a->rows == 0) return SQ_OK;
+    SQ_TRY(check_state(a->st, a->lay, who, &p.st));
+    if (!a->q || !a->k || !a->v || !a->g || !a->beta || !a->out) return fail(SQ_E_ARG, "%s: null input / output", who);
+    if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->g_dtype) ||
+        !dtype_ok(a->beta_dtype) || !dtype_ok(a->out_dtype))
+        return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    p.rows = a->rows;
+    p.idx = a->idx;
+    p.q = a->q; p.s_q = a->s_q; p.q_dt = a->q_dtype;
+    p.k = a->k; p.s_k = a->s_k; p.k_dt = a->k_dtype;
+    p.v = a->v; p.s_v = a->s_v; p.v_dt = a->v_dtype;
+    p.g = a->g; p.s_g = a->s_g; p.g_dt = a->g_dtype;
+    p.beta = a->beta; p.s_beta = a->s_beta; p.beta_dt = a->beta_dtype;
+    p.out = a->out; p.s_out = a->s_out; p.out_dt = a->out_dtype;
+    p.scale = a->scale;
+    return finish(sq::dispatch_kda(p, static_cast<hipStream_t>(stream), true), who, a->lay);
+}
+
+int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
+    const char* who = "sq_mamba2_step";
+    if (!a) return fail(SQ_E_ARG, "%s: null args", who);
+    sq::Mamba2Params p{};
+    SQ_TRY(check_layout(a->lay, who, &p));
+    if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
+    if (a->rows == 0) return SQ_OK;
+    SQ_TRY(check_state(a->st, a->lay, who, &p.st));
+    if (!a->x || !a->dt || !a->B || !a->C || !a->A || !a->out) return fail(SQ_E_ARG, "%s: null input / output", who);
+    if (!dtype_ok(a->x_dtype) || !dtype_ok(a->dt_dtype) || !dtype_ok(a->B_dtype) || !dtype_ok(a->C_dtype) ||
+        !dtype_ok(a->A_dtype) || !dtype_ok(a->out_dtype) || (a->D && !dtype_ok(a->D_dtype)) ||
+        (a->dt_bias && !dtype_ok(a->dt_bias_dtype)))
+        return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    p.rows = a->rows;
+    p.idx = a->idx;
+    p.x = a->x; p.s_x = a->s_x; p.x_dt = a->x_dtype;
+    p.dt = a->dt; p.s_dt = a->s_dt; p.dt_dt = a->dt_dtype;
+    p.B = a->B; p.s_B = a->s_B; p.B_dt = a->B_dtype;
+    p.C = a->C; p.s_C = a->s_C; p.C_dt = a->C_dtype;
+    p.A = a->A; p.A_dt = a->A_dtype;
+    p.D = a->D; p.D_dt = a->D_dtype;
+    p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    p.dt_softplus = a->dt_softplus != 0;
+    p.dt_clamp = a->dt_clamp != 0;
+    p.dt_min = a->dt_min; p.dt_max = a->dt_max;
+    p.out = a->out; p.s_out = a->s_out; p.out_dt = a->out_dtype;
+    return finish(sq::dispatch_mamba2(p, static_cast<hipStream_t>(stream), true), who, a->lay);
+}
+
+}  // extern "C"

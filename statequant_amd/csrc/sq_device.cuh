@@ -1,0 +1,201 @@
+// Device-side building blocks of the packed-state decode step for gfx950 (wave64).
+//
+// One wavefront owns one (sequence, value head) tile of the stored state: DV rows of DK codes, value-major.  A row is
+// split into 16-column pieces, one per lane, so a lane's piece of an int8 row is one 128-bit load (int4: 64 bits) and
+// the lanes of a wavefront read whole, consecutive rows.  Everything below is written for that decomposition.
+//
+// Arithmetic follows the reference's device kernels: fp32 throughout, explicit fma where the reference uses one,
+// IEEE division / sqrt, round-half-to-even, payloads rounded against the fp16-rounded scale
+// (/root/reference/src/statequant/kernels/_fold_triton.py:38-62).  The translation unit must be compiled with
+// -ffp-contract=off so that no other multiply-add is contracted.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sq {
+
+constexpr int WAVE = 64;
+constexpr int CPL = 16;                       // state columns per lane
+constexpr float FP16_TINY = 5.960464477539063e-08f;   // 2^-24: floor of a stored fp16 scale
+
+enum DType : int { F32 = 0, BF16 = 1, F16 = 2 };
+
+__host__ __device__ constexpr int pow2_ceil(int n) { int p = 1; while (p < n) p <<= 1; return p; }
+__host__ __device__ constexpr int round_up(int n, int k) { return (n + k - 1) / k * k; }
+__host__ __device__ constexpr int ilog2(int n) { int l = 0; while ((1 << l) < n) ++l; return l; }
+
+// ---------------------------------------------------------------------------------------------------------------
+// bit casts and narrow float formats
+// ---------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return as_f32(uint32_t(h) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {      // round to nearest even, quiet NaNs (as torch)
+    uint32_t u = as_u32(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return uint16_t(u >> 16);
+}
+__device__ __forceinline__ float f16_to_f32(uint16_t h) { return float(__builtin_bit_cast(_Float16, h)); }
+__device__ __forceinline__ uint16_t f32_to_f16(float f) { return __builtin_bit_cast(uint16_t, _Float16(f)); }
+
+// A scalar of a float tensor of run-time dtype (inputs come as fp32, bf16 or fp16).
+__device__ __forceinline__ float load_f(const void* p, int dt, int64_t i) {
+    if (dt == F32) return reinterpret_cast<const float*>(p)[i];
+    const uint16_t h = reinterpret_cast<const uint16_t*>(p)[i];
+    return dt == BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+__device__ __forceinline__ void store_f(void* p, int dt, int64_t i, float v) {
+    if (dt == F32) reinterpret_cast<float*>(p)[i] = v;
+    else reinterpret_cast<uint16_t*>(p)[i] = dt == BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// rounding (reference: _fold_triton.py:52-62, _fused_triton.py:471-501)
+// ---------------------------------------------------------------------------------------------------------------
+// Quantizer scale: max(amax, 1e-8) / qmax -> fp16 (nearest even, subnormals kept) -> fp32, floored at 2^-24.
+__device__ __forceinline__ float fp16_scale(float amax, float qmax) {
+    float s = fmaxf(amax, 1e-8f) / qmax;
+    s = float(_Float16(s));
+    return fmaxf(s, FP16_TINY);
+}
+
+// Buffer entry: clamp(rint(x / scale), +-127) as a float.
+__device__ __forceinline__ float round_buf(float x, float scale) {
+    return fminf(fmaxf(rintf(x / scale), -127.0f), 127.0f);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// cross-lane movement.  DPP controls: quad_perm = 8-bit selector, 0x141 row_half_mirror, 0x140 row_mirror.
+// ---------------------------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return as_f32(uint32_t(__builtin_amdgcn_update_dpp(0, int(as_u32(v)), CTRL, 0xF, 0xF, true)));
+}
+constexpr int DPP_XOR1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int DPP_HMIRROR = 0x141;    // lane i <-> 7 - i within each 8 lanes
+constexpr int DPP_MIRROR = 0x140;     // lane i <-> 15 - i within each 16 lanes
+
+// The value of the partner lane at butterfly level LVL (0: xor 1, 1: xor 2, 2: other half of 8, 3: other half of 16).
+// Levels 2 and 3 pair lane i with its mirror image, which is a valid butterfly partner once the lower levels have
+// made all lanes of the smaller block equal.
+template <int LVL>
+__device__ __forceinline__ float partner(float v) {
+    if constexpr (LVL == 0) return dpp<DPP_XOR1>(v);
+    else if constexpr (LVL == 1) return dpp<DPP_XOR2>(v);
+    else if constexpr (LVL == 2) return dpp<DPP_HMIRROR>(v);
+    else return dpp<DPP_MIRROR>(v);
+}
+
+// Sum / max over aligned blocks of N lanes (N a power of two <= 16); every lane of the block gets the result.
+template <int N>
+__device__ __forceinline__ float block_sum(float v) {
+    if constexpr (N >= 2) v = v + partner<0>(v);
+    if constexpr (N >= 4) v = v + partner<1>(v);
+    if constexpr (N >= 8) v = v + partner<2>(v);
+    if constexpr (N >= 16) v = v + partner<3>(v);
+    return v;
+}
+template <int N>
+__device__ __forceinline__ float block_max(float v) {
+    if constexpr (N >= 2) v = fmaxf(v, partner<0>(v));
+    if constexpr (N >= 4) v = fmaxf(v, partner<1>(v));
+    if constexpr (N >= 8) v = fmaxf(v, partner<2>(v));
+    if constexpr (N >= 16) v = fmaxf(v, partner<3>(v));
+    return v;
+}
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+    return as_f32(uint32_t(__builtin_amdgcn_readlane(int(as_u32(v)), lane)));
+}
+// Over the whole wavefront; the result is wave-uniform.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = block_sum<16>(v);
+    return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = block_max<16>(v);
+    return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// a lane's 16 codes of one row
+// ---------------------------------------------------------------------------------------------------------------
+template <int BITS> struct RawRow;
+template <> struct RawRow<8> { uint4 v; };      // 16 int8
+template <> struct RawRow<4> { uint2 v; };      // 16 nibbles: byte j = (c[2j] + 8) | (c[2j+1] + 8) << 4
+
+template <int BITS>
+__device__ __forceinline__ RawRow<BITS> load_row(const uint8_t* p) {
+    RawRow<BITS> r;
+    if constexpr (BITS == 8) r.v = *reinterpret_cast<const uint4*>(p);
+    else r.v = *reinterpret_cast<const uint2*>(p);
+    return r;
+}
+template <int BITS>
+__device__ __forceinline__ RawRow<BITS> zero_row() {
+    RawRow<BITS> r;
+    if constexpr (BITS == 8) r.v = make_uint4(0, 0, 0, 0);
+    else r.v = make_uint2(0x88888888u, 0x88888888u);      // nibble 8 = code 0
+    return r;
+}
+__device__ __forceinline__ float s8_to_f(uint32_t w, int byte) { return float(int32_t(w << (24 - 8 * byte)) >> 24); }
+
+template <int BITS>
+__device__ __forceinline__ void decode_row(const RawRow<BITS>& r, float (&c)[CPL]) {
+    if constexpr (BITS == 8) {
+        const uint32_t w[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) c[4 * d + b] = s8_to_f(w[d], b);
+    } else {
+        const uint32_t w[2] = {r.v.x, r.v.y};
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) c[8 * d + nb] = float(int32_t((w[d] >> (4 * nb)) & 0xFu) - 8);
+    }
+}
+
+// Integral floats in [-qmax, qmax] -> a lane's stored row.
+template <int BITS>
+__device__ __forceinline__ RawRow<BITS> encode_row(const float (&c)[CPL]) {
+    RawRow<BITS> r;
+    if constexpr (BITS == 8) {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            w[d] = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) w[d] |= (uint32_t(int32_t(c[4 * d + b])) & 0xFFu) << (8 * b);
+        }
+        r.v = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        uint32_t w[2];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            w[d] = 0;
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) w[d] |= (uint32_t(int32_t(c[8 * d + nb]) + 8) & 0xFu) << (4 * nb);
+        }
+        r.v = make_uint2(w[0], w[1]);
+    }
+    return r;
+}
+template <int BITS>
+__device__ __forceinline__ void store_row(uint8_t* p, const RawRow<BITS>& r) {
+    if constexpr (BITS == 8) *reinterpret_cast<uint4*>(p) = r.v;
+    else *reinterpret_cast<uint2*>(p) = r.v;
+}
+
+// Workgroup id -> tile id.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs; this makes every XCD walk
+// a contiguous range of tiles, so the tiles of one sequence (shared key buffer, neighbouring counters) meet in one L2.
+__device__ __forceinline__ int xcd_tile(int wg, int n) {
+    constexpr int XCDS = 8;
+    if (n % XCDS) return wg;
+    return (wg % XCDS) * (n / XCDS) + wg / XCDS;
+}
+
+}  // namespace sq

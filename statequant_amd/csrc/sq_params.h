@@ -1,0 +1,76 @@
+// Kernel-side argument blocks (typed, validated copies of the public structs in include/statequant_hip.h) and the
+// per-family dispatchers that map a layout onto a compiled kernel instance.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sq {
+
+struct StatePtrs {
+    uint8_t* S;      int64_t sS;     // bytes of codes per sequence step (int8: elements = bytes; int4: packed bytes)
+    uint16_t* SC;    int64_t sSC;
+    uint8_t* KB;     int64_t sKB;    // strides of KB / UB in ELEMENTS (int8 or bf16)
+    uint16_t* KBS;   int64_t sKBS;
+    uint8_t* UB;     int64_t sUB;
+    uint16_t* UBS;   int64_t sUBS;
+    float* GB;       int64_t sGB;
+    float* GCUR;     int64_t sGC;
+    int32_t* NPTR;   int64_t sN;
+};
+
+struct LayoutKey {
+    int bits, group, qbuf, m, hv, hk, dk, dv;
+};
+
+struct GdnParams : LayoutKey {
+    StatePtrs st;
+    int rows;
+    const int32_t* idx;
+    const void *q, *k, *v;
+    int64_t s_q, s_k, s_v;
+    int q_dt, k_dt, v_dt;
+    int qk_per_key_head, gate;
+    const void *g, *beta;
+    int64_t s_g, s_beta;
+    int g_dt, beta_dt;
+    const void *a, *bt, *A_log, *dt_bias;
+    int64_t s_a, s_bt;
+    int a_dt, bt_dt, A_log_dt, dt_bias_dt;
+    void* out;
+    int out_dt;
+    float scale;
+};
+
+struct KdaParams : LayoutKey {
+    StatePtrs st;
+    int rows;
+    const int32_t* idx;
+    const void *q, *k, *v, *g, *beta;
+    int64_t s_q, s_k, s_v, s_g, s_beta;
+    int q_dt, k_dt, v_dt, g_dt, beta_dt;
+    void* out;
+    int64_t s_out;
+    int out_dt;
+    float scale;
+};
+
+struct Mamba2Params : LayoutKey {
+    StatePtrs st;
+    int rows;
+    const int32_t* idx;
+    const void *x, *dt, *B, *C, *A, *D, *dt_bias;
+    int64_t s_x, s_dt, s_B, s_C;
+    int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
+    int dt_softplus, dt_clamp;
+    float dt_min, dt_max;
+    void* out;
+    int64_t s_out;
+    int out_dt;
+};
+
+// hipError_t of the launch (0 = enqueued), or -1 if no kernel is compiled for the layout.  run = false: probe only.
+int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
+int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
+int dispatch_mamba2(const Mamba2Params& p, hipStream_t stream, bool run);
+
+}  // namespace sq

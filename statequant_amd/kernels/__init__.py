@@ -1,0 +1,17 @@
+"""Packed (real-storage) decode path on HIP kernels: int4 / int8 recurrent state with a delta-value decode buffer.
+
+    from statequant_amd.kernels import PackedGDNState, SlotLayout, pack, unpack
+
+Same names as the reference's ``statequant.kernels`` (``/root/reference/src/statequant/kernels/__init__.py:10-18``).
+``pack`` / ``unpack`` are torch; ``PackedGDNState`` (sequences in lockstep), ``SlotLayout.step`` (slot-addressed
+sequences: the serving layout), ``PackedMamba2State`` / ``Mamba2SlotLayout`` and ``PackedKDAState`` /
+``KDASlotLayout`` call the HIP kernels in ``libsqhip.so`` and need an MI355X.
+"""
+from .fold import PackedGDNState, check_dims, pack, pack_vk, packed_format, unpack, unpack_vk
+from .kda import KDASlotLayout, PackedKDAState, kda_recurrence
+from .mamba2 import Mamba2SlotLayout, PackedMamba2State, mamba2_recurrence
+from .slots import SlotLayout
+
+__all__ = ['PackedGDNState', 'SlotLayout', 'pack', 'unpack', 'pack_vk', 'unpack_vk', 'packed_format', 'check_dims',
+           'PackedMamba2State', 'Mamba2SlotLayout', 'mamba2_recurrence',
+           'PackedKDAState', 'KDASlotLayout', 'kda_recurrence']

@@ -1,0 +1,146 @@
+"""ctypes binding of libsqhip.so (the C ABI declared in ``include/statequant_hip.h``).
+
+The library is built in-tree by ``python -m statequant_amd.csrc.build`` and must be present: there is no fallback
+path.  ``lib()`` raises ``RuntimeError`` when it is missing, so a decode step can never silently run anywhere but in
+the HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG, 'libsqhip.so')
+ABI_VERSION = 1
+
+F32, BF16, F16 = 0, 1, 2
+_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+FAMILY = {'gdn': 0, 'kda': 1, 'mamba2': 2}
+
+SYMBOLS = ('sq_abi_version', 'sq_strerror', 'sq_last_error', 'sq_supported', 'sq_gdn_step', 'sq_kda_step',
+           'sq_mamba2_step')
+
+_vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
+
+
+class SqState(C.Structure):
+    _fields_ = [('S', _vp), ('sS', _i64), ('SC', _vp), ('sSC', _i64), ('KB', _vp), ('sKB', _i64),
+                ('KBS', _vp), ('sKBS', _i64), ('UB', _vp), ('sUB', _i64), ('UBS', _vp), ('sUBS', _i64),
+                ('GB', _vp), ('sGB', _i64), ('GCUR', _vp), ('sGC', _i64), ('NPTR', _vp), ('sN', _i64)]
+
+
+class SqLayout(C.Structure):
+    _fields_ = [('bits', _i32), ('axis_k', _i32), ('group', _i32), ('buffer_bits', _i32), ('m', _i32),
+                ('hv', _i32), ('hk', _i32), ('dk', _i32), ('dv', _i32)]
+
+
+class SqGdnArgs(C.Structure):
+    _fields_ = [('st', SqState), ('lay', SqLayout), ('rows', _i32), ('idx', _vp),
+                ('q', _vp), ('s_q', _i64), ('q_dtype', _i32),
+                ('k', _vp), ('s_k', _i64), ('k_dtype', _i32),
+                ('v', _vp), ('s_v', _i64), ('v_dtype', _i32),
+                ('qk_per_key_head', _i32), ('gate', _i32),
+                ('g', _vp), ('s_g', _i64), ('g_dtype', _i32),
+                ('beta', _vp), ('s_beta', _i64), ('beta_dtype', _i32),
+                ('a', _vp), ('s_a', _i64), ('a_dtype', _i32),
+                ('b', _vp), ('s_b', _i64), ('b_dtype', _i32),
+                ('A_log', _vp), ('A_log_dtype', _i32),
+                ('dt_bias', _vp), ('dt_bias_dtype', _i32),
+                ('out', _vp), ('out_dtype', _i32), ('scale', _f32)]
+
+
+class SqKdaArgs(C.Structure):
+    _fields_ = [('st', SqState), ('lay', SqLayout), ('rows', _i32), ('idx', _vp),
+                ('q', _vp), ('s_q', _i64), ('q_dtype', _i32),
+                ('k', _vp), ('s_k', _i64), ('k_dtype', _i32),
+                ('v', _vp), ('s_v', _i64), ('v_dtype', _i32),
+                ('g', _vp), ('s_g', _i64), ('g_dtype', _i32),
+                ('beta', _vp), ('s_beta', _i64), ('beta_dtype', _i32),
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('scale', _f32)]
+
+
+class SqMamba2Args(C.Structure):
+    _fields_ = [('st', SqState), ('lay', SqLayout), ('rows', _i32), ('idx', _vp),
+                ('x', _vp), ('s_x', _i64), ('x_dtype', _i32),
+                ('dt', _vp), ('s_dt', _i64), ('dt_dtype', _i32),
+                ('B', _vp), ('s_B', _i64), ('B_dtype', _i32),
+                ('C', _vp), ('s_C', _i64), ('C_dtype', _i32),
+                ('A', _vp), ('A_dtype', _i32), ('D', _vp), ('D_dtype', _i32),
+                ('dt_bias', _vp), ('dt_bias_dtype', _i32),
+                ('dt_softplus', _i32), ('dt_clamp', _i32), ('dt_min', _f32), ('dt_max', _f32),
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built or does not match this binding."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f'{LIB_PATH} is missing: build it with `python -m statequant_amd.csrc.build` '
+                               '(the packed decode step has no fallback path)')
+        L = C.CDLL(LIB_PATH)
+        L.sq_abi_version.restype = C.c_int
+        L.sq_strerror.restype = C.c_char_p
+        L.sq_strerror.argtypes = [C.c_int]
+        L.sq_last_error.restype = C.c_char_p
+        L.sq_supported.restype = C.c_int
+        L.sq_supported.argtypes = [C.c_int, C.POINTER(SqLayout)]
+        for name, T in (('sq_gdn_step', SqGdnArgs), ('sq_kda_step', SqKdaArgs), ('sq_mamba2_step', SqMamba2Args)):
+            f = getattr(L, name)
+            f.restype = C.c_int
+            f.argtypes = [C.POINTER(T), C.c_void_p]
+        if L.sq_abi_version() != ABI_VERSION:
+            raise RuntimeError(f'{LIB_PATH}: ABI version {L.sq_abi_version()}, this package expects {ABI_VERSION}')
+        _lib = L
+    return _lib
+
+
+def dtype_code(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f'float tensor of dtype fp32 / bf16 / fp16 expected, got {t.dtype}') from None
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def make_layout(st):
+    """``SqLayout`` from a layout / state object with the reference's attribute names (bits, axk, group, ...)."""
+    return SqLayout(bits=st.bits, axis_k=int(st.axk), group=st.group, buffer_bits=st.buffer_bits, m=st.m,
+                    hv=st.HV, hk=st.HK, dk=st.DK, dv=st.DV)
+
+
+def supported(family, st):
+    lay = make_layout(st)
+    return bool(lib().sq_supported(FAMILY[family], C.byref(lay)))
+
+
+def make_state(T, strides, nptr_stride):
+    """``SqState`` from the nine state tensors (dict) and their per-sequence strides in elements."""
+    sS, sSC, sKB, sKBS, sUB, sUBS, sGB, sGC = strides
+    return SqState(S=ptr(T['S']), sS=sS, SC=ptr(T['SC']), sSC=sSC, KB=ptr(T['KB']), sKB=sKB,
+                   KBS=ptr(T['KBS']), sKBS=sKBS, UB=ptr(T['UB']), sUB=sUB, UBS=ptr(T['UBS']), sUBS=sUBS,
+                   GB=ptr(T['GB']), sGB=sGB, GCUR=ptr(T['GCUR']), sGC=sGC, NPTR=ptr(T['NPTR']), sN=nptr_stride)
+
+
+def current_stream(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def check(rc):
+    if rc != 0:
+        L = lib()
+        raise RuntimeError(f'libsqhip: {L.sq_strerror(rc).decode()}: {L.sq_last_error().decode()}')
+
+
+def require_gpu(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(f'{what}: the packed decode step runs on the GPU only (HIP kernels, no fallback); '
+                           f'got a tensor on {t.device}')

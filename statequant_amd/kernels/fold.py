@@ -1,0 +1,266 @@
+"""Packed recurrent-state storage for Gated DeltaNet and the lockstep decode step, on HIP kernels.
+
+Mirrors the host API of the reference's ``statequant/kernels/fold.py`` (``/root/reference/src/statequant/kernels/
+fold.py``): ``packed_format``, ``pack`` / ``unpack`` / ``pack_vk`` / ``unpack_vk``, ``check_dims``, ``use_fused`` and
+``PackedGDNState`` keep their names, arguments and tensor layouts; the Triton launches (fold.py:400-424) are replaced
+by one call into ``libsqhip.so`` (``sq_gdn_step``).
+
+The decode algebra (fold.py:1-19): the stored state S_0 is kept rounded and rewritten only every ``m`` tokens; the
+tokens in between sit in a buffer of (cumulative log decay G_i, normalised key k_i, delta value u_i); a step reads the
+stored codes once and the buffer once; a full buffer is folded into the state, which is re-rounded on the device.
+
+Layouts: states enter and leave as [BH, d_k, d_v]; they are stored value-major, [BH, d_v, d_k].
+"""
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+
+import torch
+
+from ..quantizer import FloatCast, Quantizer
+from . import _hip
+
+_FP16_MIN = 2.0 ** -24
+
+
+def pow2(n):
+    """Smallest power of two >= n."""
+    return 1 << max(0, (int(n) - 1).bit_length())
+
+
+def packed_format(fmt):
+    """The format a packed store holds: ``fmt`` with fp16 scales, or None for the bf16 control (fold.py:91-104).
+
+    Accepts a symmetric round-to-nearest ``Quantizer`` (4 or 8 bits, axis 'k' or 'v', no rotation, 16-bit scales) or
+    'bf16' / ``FloatCast('bf16')`` / None.  Any object with the Quantizer's attributes is taken (duck typing), so
+    formats built with the reference's own class pass through."""
+    if fmt is None or fmt == 'bf16':
+        return None
+    if isinstance(fmt, FloatCast) or type(fmt).__name__ == 'FloatCast':
+        if fmt.dtype == 'bf16' and not fmt.stochastic:
+            return None
+    need = ('bits', 'axis', 'group', 'affine', 'rotation', 'rounding', 'scale_bits')
+    assert all(hasattr(fmt, a) for a in need), f'packed storage needs a Quantizer or bf16, got {fmt!r}'
+    assert fmt.bits in (4, 8) and fmt.axis in ('k', 'v'), (fmt.bits, fmt.axis)
+    assert not fmt.affine and fmt.rotation is None and fmt.rounding == 'rtn' and fmt.scale_bits == 16, \
+        'packed storage implements symmetric RTN with 16-bit scales and no rotation'
+    assert fmt.group % 2 == 0
+    if isinstance(fmt, Quantizer):
+        return dataclasses.replace(fmt, scale_dtype='fp16')
+    return Quantizer(fmt.bits, fmt.axis, fmt.group, scale_dtype='fp16')
+
+
+def check_dims(fmt, dk, dv):
+    """Head dims and groups a packed GDN store accepts (fold.py:63-76)."""
+    assert dk >= 16 and dk % 2 == 0, f'd_k must be even and >= 16, got {dk}'
+    assert dv % 32 == 0, f'd_v must be a multiple of 32, got {dv}'
+    if fmt is not None:
+        g = fmt.group
+        assert g >= 2 and g & (g - 1) == 0, f'group {g} must be a power of two'
+        if fmt.axis == 'k':
+            assert g <= pow2(dk) and pow2(dk) // g <= 8, f'key group {g} on d_k {dk}: 1 .. 8 groups'
+        else:
+            assert dv % g == 0, f'value group {g} must divide d_v {dv}'
+
+
+def use_fused(fused, bh, axis_v=False):
+    """Kept for call compatibility (fold.py:79-85).  There is a single HIP step, always one launch."""
+    return True
+
+
+def _bits(fmt):
+    return 16 if fmt is None else fmt.bits
+
+
+def _scale_of(amax, qmax):
+    """absmax -> stored scale: max(amax, 1e-8) / qmax, to fp16 and back, floored at 2^-24 (quantizer.py:159-164)."""
+    return (amax.clamp_min(1e-8) / qmax).to(torch.float16).float().clamp_min(_FP16_MIN)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# storage format (torch; the reference's pack / unpack are torch too, fold.py:111-173)
+# ---------------------------------------------------------------------------------------------------------------
+def pack_vk(x, fmt):
+    """Value-major state [BH, d_v, d_k] (or [..., d_v, d_k]) -> (codes, scales) (fold.py:123-147).
+
+    codes   int8 [BH, d_v, d_k]; 4 bit: uint8 [BH, d_v, d_k/2], byte j = (c[2j] + 8) | (c[2j+1] + 8) << 4;
+            bf16 state: bf16 [BH, d_v, d_k]
+    scales  fp16; axis 'k': [BH, d_v, ceil(d_k/group)] (a ragged last group has its own scale);
+            axis 'v': [BH, d_v/group, d_k]; bf16 state: a [1] tensor of ones
+    """
+    fmt = packed_format(fmt)
+    x = x.float().reshape(-1, x.shape[-2], x.shape[-1])
+    n, dv, dk = x.shape
+    if fmt is None:
+        return x.to(torch.bfloat16).contiguous(), torch.ones(1, device=x.device, dtype=torch.float16)
+    g = fmt.group
+    qmax = float(2 ** (fmt.bits - 1) - 1)
+    if fmt.axis == 'k':
+        ng = -(-dk // g)
+        xg = torch.nn.functional.pad(x, (0, ng * g - dk)).view(n, dv, ng, g)       # zero pad: same absmax
+        sc = _scale_of(xg.abs().amax(3, keepdim=True), qmax)
+        q = torch.round(xg / sc).clamp_(-qmax, qmax).view(n, dv, ng * g)[:, :, :dk]
+        sc = sc.view(n, dv, ng)
+    else:
+        assert dv % g == 0, f'value group {g} must divide d_v {dv}'
+        xg = x.view(n, dv // g, g, dk)
+        sc = _scale_of(xg.abs().amax(2, keepdim=True), qmax)
+        q = torch.round(xg / sc).clamp_(-qmax, qmax).view(n, dv, dk)
+        sc = sc.view(n, dv // g, dk)
+    q = q.to(torch.int8)
+    if fmt.bits == 4:
+        nib = (q + 8).to(torch.uint8)
+        q = nib[:, :, 0::2] | (nib[:, :, 1::2] << 4)
+    return q.contiguous(), sc.to(torch.float16).contiguous()
+
+
+def unpack_vk(codes, scales, fmt, d_k):
+    """Inverse of ``pack_vk``: -> fp32 [BH, d_v, d_k] (fold.py:155-173)."""
+    fmt = packed_format(fmt)
+    if fmt is None:
+        return codes.float()
+    n, dv = codes.shape[:2]
+    if fmt.bits == 4:
+        b = codes.to(torch.int16)
+        x = torch.stack(((b & 15) - 8, ((b >> 4) & 15) - 8), dim=-1).view(n, dv, -1)[:, :, :d_k].float()
+    else:
+        x = codes.float()
+    sc = scales.float()
+    g = fmt.group
+    if fmt.axis == 'k':
+        return x * sc.repeat_interleave(g, dim=2)[:, :, :d_k]
+    return (x.view(n, dv // g, g, d_k) * sc[:, :, None, :]).view(n, dv, d_k)
+
+
+def pack(S, fmt):
+    """[BH, d_k, d_v] (or [B, H, d_k, d_v]) float -> (codes, scales) of the value-major store (fold.py:111-120)."""
+    x = S.float().reshape(-1, S.shape[-2], S.shape[-1]).transpose(1, 2).contiguous()
+    return pack_vk(x, fmt)
+
+
+def unpack(codes, scales, fmt, d_k):
+    """Inverse of ``pack``: -> fp32 [BH, d_k, d_v] (fold.py:150-152)."""
+    return unpack_vk(codes, scales, fmt, d_k).transpose(1, 2).contiguous()
+
+
+def _flat(S):
+    return S.float().reshape(-1, S.shape[-2], S.shape[-1]).contiguous()
+
+
+def _require_kernel(family, st):
+    """Fail at construction, with the reason, when no HIP kernel exists for a layout."""
+    if st.fmt is None:
+        raise NotImplementedError('the unquantized bf16 / fp32 state control is not built for the HIP step yet')
+    if not st.axk:
+        raise NotImplementedError('value-axis scale groups (axis="v") are not built for the HIP step yet')
+    if not _hip.supported(family, st):
+        raise NotImplementedError(
+            f'no HIP kernel instance for {family}: int{st.bits} group {st.group}, d_k {st.DK}, d_v {st.DV}, '
+            f'm {st.m}, buffer_bits {st.buffer_bits} (see statequant_amd/csrc/build.py: CASES)')
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# lockstep state
+# ---------------------------------------------------------------------------------------------------------------
+class PackedGDNState:
+    """One layer's packed recurrent state and decode buffer for B sequences stepped in lockstep (fold.py:280-424).
+
+    S            [BH, d_k, d_v] (or [B, H, d_k, d_v]) float state to start from
+    fmt          ``Quantizer(4 or 8, 'k', group)``; scales are stored fp16
+    m            buffer length (power of two); the state is folded and re-rounded every m steps
+    hv, hk       value / key heads per sequence (hv % hk == 0); BH = B * hv
+    buffer_bits  8 (int8 + one fp16 absmax scale per vector) or 16 (bf16)
+    out_dtype    dtype of the output
+    The remaining keyword arguments of the reference (block sizes, warps, ``fused``) are accepted and ignored.
+
+    ``step(q, k, v, g, beta, scale)``: q, k raw [BH, d_k] or per key head [B * hk, d_k]; v [BH, d_v]; g (log decay)
+    and beta [BH].  Returns the output buffer [BH, d_v] (the same tensor every step).  Every tensor is allocated
+    once and updated in place, and the step is one kernel launch on the current stream, so it can be graph-captured.
+    """
+
+    def __init__(self, S, fmt, m=8, hv=None, hk=None, buffer_bits=8, out_dtype=torch.bfloat16,
+                 block_v=None, warps=None, fused=None, fused_warps=None):
+        S = _flat(S)
+        _hip.require_gpu(S, 'PackedGDNState')
+        BH, DK, DV = S.shape
+        dev = S.device
+        self.BH, self.DK, self.DV, self.m = BH, DK, DV, m
+        self.fmt = packed_format(fmt)
+        self.bits = _bits(self.fmt)
+        self.HV = hv or BH
+        self.HK = hk or self.HV
+        assert self.HV % self.HK == 0 and BH % self.HV == 0, (BH, self.HV, self.HK)
+        self.gqa, self.B = self.HV // self.HK, BH // self.HV
+        assert m >= 1 and m & (m - 1) == 0, 'm must be a power of two'
+        check_dims(self.fmt, DK, DV)
+        assert buffer_bits in (8, 16)
+        self.buffer_bits, self.qbuf = buffer_bits, buffer_bits == 8
+        self.axk = self.fmt is not None and self.fmt.axis == 'k'
+        self.group = self.fmt.group if self.fmt is not None else 32
+        self.fused = True
+        _require_kernel('gdn', self)
+
+        codes, scales = pack(S, self.fmt)
+        self.codes, self.scales = codes.clone(), scales.clone()
+        bdt = torch.int8 if self.qbuf else torch.bfloat16
+        z = lambda *shape, dtype: torch.zeros(*shape, device=dev, dtype=dtype)      # noqa: E731
+        self.KB = z(self.B * self.HK, m, DK, dtype=bdt)
+        self.UB = z(BH, m, DV, dtype=bdt)
+        self.KBS = z(self.B * self.HK, m, dtype=torch.float16)
+        self.UBS = z(BH, m, dtype=torch.float16)
+        self.GB = z(BH, m, dtype=torch.float32)
+        self.GCUR = z(BH, dtype=torch.float32)
+        self.NPTR = z(self.B, self.HV, dtype=torch.int32)          # one counter copy per (sequence, value head)
+        self.O = z(BH, DV, dtype=out_dtype)
+        HV, HK = self.HV, self.HK
+        self._T = dict(S=self.codes, SC=self.scales, KB=self.KB, KBS=self.KBS, UB=self.UB, UBS=self.UBS, GB=self.GB,
+                       GCUR=self.GCUR, NPTR=self.NPTR)
+        # per-sequence strides of the lockstep layout: contiguous sequences
+        self._strides = (HV * self.codes[0].numel(), HV * self.scales[0].numel(), HK * m * DK, HK * m,
+                         HV * m * DV, HV * m, HV * m, HV)
+        self._lay = _hip.make_layout(self)
+
+    @torch.no_grad()
+    def load(self, S):
+        """Replace the state in place and empty the buffer."""
+        c, sc = pack(_flat(S), self.fmt)
+        self.codes.copy_(c)
+        self.scales.copy_(sc)
+        for t in (self.KB, self.UB, self.KBS, self.UBS, self.GB, self.GCUR, self.NPTR):
+            t.zero_()
+
+    def dequantize(self):
+        """The stored state S_0 (without the buffered tokens) as fp32 [BH, d_k, d_v]."""
+        return unpack(self.codes, self.scales, self.fmt, self.DK)
+
+    @property
+    def n(self):
+        return int(self.NPTR.reshape(-1)[0])
+
+    def stored_bytes(self):
+        """Resident bytes: state payload + scales, the buffer, the decays (fold.py:371-378)."""
+        nb = lambda t: t.numel() * t.element_size()          # noqa: E731
+        per = dict(state=nb(self.codes) + nb(self.scales),
+                   buffer=nb(self.KB) + nb(self.UB) + ((nb(self.KBS) + nb(self.UBS)) if self.qbuf else 0),
+                   decay=nb(self.GB) + nb(self.GCUR) + nb(self.NPTR))
+        per['total'] = sum(per.values())
+        return per
+
+    def step(self, q, k, v, g, beta, scale):
+        BH, HV, HK = self.BH, self.HV, self.HK
+        per_key = q.shape[0] != BH
+        if per_key:
+            assert q.shape[0] == self.B * HK and k.shape[0] == self.B * HK
+        for t in (q, k, v, g, beta):
+            assert t.is_contiguous()
+        sqk = (HK if per_key else HV) * self.DK
+        a = _hip.SqGdnArgs(
+            st=_hip.make_state(self._T, self._strides, HV), lay=self._lay, rows=self.B, idx=None,
+            q=q.data_ptr(), s_q=sqk, q_dtype=_hip.dtype_code(q), k=k.data_ptr(), s_k=sqk, k_dtype=_hip.dtype_code(k),
+            v=v.data_ptr(), s_v=HV * self.DV, v_dtype=_hip.dtype_code(v), qk_per_key_head=int(per_key), gate=0,
+            g=g.data_ptr(), s_g=HV, g_dtype=_hip.dtype_code(g),
+            beta=beta.data_ptr(), s_beta=HV, beta_dtype=_hip.dtype_code(beta),
+            out=self.O.data_ptr(), out_dtype=_hip.dtype_code(self.O), scale=float(scale))
+        _hip.check(_hip.lib().sq_gdn_step(ctypes.byref(a), _hip.current_stream(self.O.device)))
+        return self.O

@@ -1,0 +1,201 @@
+"""Writes the golden vectors under tests/golden/ by running the REFERENCE's own torch classes on seeded inputs.
+
+Runs only where the reference checkout is mounted (default /root/reference; override with SQ_REFERENCE); the tests
+never import the reference, they only load the .pt files written here (plain tensors, ``weights_only=True``).
+
+    python tests/golden/make_golden.py
+
+What is recorded (CPU, fp32, torch.manual_seed per case):
+  pack_*.pt      pack / pack_vk / unpack on the reference tests' edge cases (all-zero groups, 1e-6-scaled states, a
+                 ragged last key group), `_round_buf`, `Quantizer(..., scale_dtype='fp16').fake`
+  gdn_*.pt       ReferenceGDNState: per step the inputs, the output, the entries appended to the buffer, and at
+                 every fold the unrounded folded state, the codes and the scales
+  kda_*.pt       ReferenceKDAState, likewise;   m2_*.pt  ReferenceMamba2State, likewise
+  slots_*.pt     SlotLayout / KDASlotLayout / Mamba2SlotLayout: field tables, `write` then `read` on a blob with a
+                 partly filled buffer
+"""
+import os
+import sys
+
+import torch
+
+REF = os.environ.get('SQ_REFERENCE', '/root/reference')
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(REF, 'src'))
+
+import statequant as sq  # noqa: E402
+from statequant.kernels import (KDASlotLayout, Mamba2SlotLayout, ReferenceGDNState, ReferenceKDAState,  # noqa: E402
+                                ReferenceMamba2State, SlotLayout, pack, pack_vk, unpack, unpack_vk)
+from statequant.kernels.fold import _round_buf  # noqa: E402
+
+torch.set_num_threads(1)                 # one thread: reduction order independent of the host's core count
+
+
+def save(name, obj):
+    path = os.path.join(HERE, name)
+    torch.save(obj, path)
+    print(f'{name}: {os.path.getsize(path) / 1024:.0f} KiB')
+
+
+def fmt_of(t):
+    return sq.Quantizer(*t)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def golden_pack():
+    torch.manual_seed(0)
+    S = torch.randn(3, 64, 32) * torch.rand(3, 64, 1) * 3          # [BH, d_k, d_v]
+    S[0, :32, :] = 0                                                # all-zero key groups
+    S[1] *= 1e-6                                                    # scales in the fp16 subnormal range
+    out = {'S': S, 'cases': []}
+    for bits in (4, 8):
+        for axis, group in (('k', 32), ('k', 64), ('v', 16), ('v', 32)):
+            q = sq.Quantizer(bits, axis, group)
+            c, s = pack(S, q)
+            out['cases'].append(dict(fmt=(bits, axis, group), codes=c, scales=s, deq=unpack(c, s, q, 64),
+                                     fake=sq.Quantizer(bits, axis, group, scale_dtype='fp16').fake(S)))
+    # ragged last key group: d_k = 96, group 64 (value-major input)
+    X = torch.randn(2, 32, 96)
+    rag = []
+    for bits in (4, 8):
+        q = sq.Quantizer(bits, 'k', 64)
+        c, s = pack_vk(X, q)
+        rag.append(dict(fmt=(bits, 'k', 64), codes=c, scales=s, deq=unpack_vk(c, s, q, 96)))
+    out['ragged_X'], out['ragged'] = X, rag
+    cb, sb = pack(S, 'bf16')
+    out['bf16_codes'], out['bf16_deq'] = cb, unpack(cb, sb, 'bf16', 64)
+    v = torch.randn(5, 64) * torch.tensor([1., 1e-3, 50., 1e-7, 0.])[:, None]
+    out['rb_in'], out['rb8'], out['rb16'] = v, _round_buf(v, 8), _round_buf(v, 16)
+    save('pack.pt', out)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def run_gdn(name, fmt, B, HV, HK, DK, DV, m, bb, T, seed, S0_scale=0.5, per_key=True, v_head_scale=False):
+    torch.manual_seed(seed)
+    BH = B * HV
+    S0 = torch.randn(BH, DK, DV) * S0_scale if S0_scale else torch.zeros(BH, DK, DV)
+    ref = ReferenceGDNState(S0, fmt_of(fmt) if fmt != 'bf16' else 'bf16', m=m, hv=HV, hk=HK, buffer_bits=bb)
+    rec = dict(family='gdn', fmt=fmt, B=B, HV=HV, HK=HK, DK=DK, DV=DV, m=m, buffer_bits=bb, scale=DK ** -0.5,
+               S0=S0, codes0=ref.codes.clone(), scales0=ref.scales.clone(), steps=[])
+    vs = torch.exp(torch.empty(HV).uniform_(-2.302585, 2.302585)) if v_head_scale else torch.ones(HV)
+    for t in range(T):
+        nq = B * HK if per_key else BH
+        q, k = torch.randn(nq, DK), torch.randn(nq, DK)
+        v = torch.randn(BH, DV) * vs.repeat(B)[:, None]
+        g = -torch.nn.functional.softplus(torch.randn(BH))
+        beta = torch.sigmoid(torch.randn(BH))
+        n = ref.n
+        o = ref.step(q, k, v, g, beta, DK ** -0.5)
+        st = dict(q=q, k=k, v=v, g=g, beta=beta, o=o.clone(), n=n, U=ref.U[:, n].clone(), K=ref.K[:, n].clone(),
+                  G=ref.G[:, n].clone())
+        if ref.n == 0:                                              # folded in this step
+            st.update(S_raw=ref.S_raw.clone(), codes=ref.codes.clone(), scales=ref.scales.clone())
+        rec['steps'].append(st)
+    save(name, rec)
+
+
+def run_kda(name, fmt, B, H, DK, DV, m, bb, T, seed):
+    torch.manual_seed(seed)
+    BH = B * H
+    S0 = torch.randn(BH, DV, DK) * 0.5
+    ref = ReferenceKDAState(S0, fmt_of(fmt), m=m, hv=H, buffer_bits=bb)
+    rec = dict(family='kda', fmt=fmt, B=B, HV=H, HK=H, DK=DK, DV=DV, m=m, buffer_bits=bb, S0=S0,
+               codes0=ref.codes.clone(), scales0=ref.scales.clone(), steps=[])
+    for t in range(T):
+        q, k, v = torch.randn(BH, DK), torch.randn(BH, DK), torch.randn(BH, DV)
+        g = -torch.nn.functional.softplus(torch.randn(BH, DK))
+        beta = torch.sigmoid(torch.randn(BH))
+        n = ref.n
+        o = ref.step(q, k, v, g, beta)
+        st = dict(q=q, k=k, v=v, g=g, beta=beta, o=o.clone(), n=n, U=ref.U[:, n].clone(), K=ref.K[:, n].clone(),
+                  G=ref.G[:, n].clone())
+        if ref.n == 0:
+            st.update(S_raw=ref.S_raw.clone(), codes=ref.codes.clone(), scales=ref.scales.clone())
+        rec['steps'].append(st)
+    save(name, rec)
+
+
+def run_m2(name, fmt, B, H, G, DK, DV, m, bb, T, seed):
+    torch.manual_seed(seed)
+    BH = B * H
+    S0 = torch.randn(BH, DV, DK) * 0.5
+    ref = ReferenceMamba2State(S0, fmt_of(fmt), m=m, hv=H, hk=G, buffer_bits=bb)
+    A = -torch.exp(torch.rand(H) * 2)
+    D = torch.randn(H)
+    dt_bias = torch.randn(H) * 0.1
+    rec = dict(family='mamba2', fmt=fmt, B=B, HV=H, HK=G, DK=DK, DV=DV, m=m, buffer_bits=bb, S0=S0, A=A, D=D,
+               dt_bias=dt_bias, codes0=ref.codes.clone(), scales0=ref.scales.clone(), steps=[])
+    for t in range(T):
+        x = torch.randn(B, H, DV)
+        dt = torch.randn(B, H) * 0.5 - 2
+        Bm, C = torch.randn(B, G, DK), torch.randn(B, G, DK)
+        n = ref.n
+        y = ref.step(x, dt, Bm, C, A, D, dt_bias, True, (0., float('inf')))
+        st = dict(x=x, dt=dt, B=Bm, C=C, o=y.clone(), n=n, U=ref.U[:, n].clone(), K=ref.K[:, n].clone(),
+                  G=ref.G[:, n].clone())
+        if ref.n == 0:
+            st.update(S_raw=ref.S_raw.clone(), codes=ref.codes.clone(), scales=ref.scales.clone())
+        rec['steps'].append(st)
+    save(name, rec)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def golden_slots():
+    out = {'tables': []}
+    for fam, cls, args in (
+            ('gdn', SlotLayout, dict(fmt=(4, 'k', 64), hv=32, hk=16, dk=128, dv=128, m=8, buffer_bits=8)),
+            ('gdn', SlotLayout, dict(fmt=(8, 'k', 32), hv=32, hk=16, dk=128, dv=128, m=8, buffer_bits=8)),
+            ('gdn', SlotLayout, dict(fmt=(8, 'k', 128), hv=32, hk=16, dk=128, dv=128, m=8, buffer_bits=16)),
+            ('gdn', SlotLayout, dict(fmt=(4, 'k', 64), hv=30, hk=30, dk=96, dv=192, m=8, buffer_bits=8)),
+            ('gdn', SlotLayout, dict(fmt='bf16', hv=4, hk=2, dk=64, dv=64, m=4, buffer_bits=16)),
+            ('gdn', SlotLayout, dict(fmt='fp32', hv=4, hk=2, dk=64, dv=64, m=4, buffer_bits=8)),
+            ('gdn', SlotLayout, dict(fmt=(4, 'v', 32), hv=4, hk=2, dk=128, dv=128, m=8, buffer_bits=8)),
+            ('kda', KDASlotLayout, dict(fmt=(4, 'k', 32), hv=32, dk=128, dv=128, m=8, buffer_bits=8)),
+            ('kda', KDASlotLayout, dict(fmt=(4, 'k', 64), hv=16, dk=128, dv=128, m=8, buffer_bits=8)),
+            ('mamba2', Mamba2SlotLayout, dict(fmt=(8, 'k', 128), hv=128, hk=8, dk=128, dv=64, m=8, buffer_bits=8)),
+            ('mamba2', Mamba2SlotLayout, dict(fmt=(8, 'k', 32), hv=112, hk=8, dk=128, dv=64, m=8, buffer_bits=8))):
+        kw = dict(args)
+        f = kw.pop('fmt')
+        lay = cls(fmt_of(f) if isinstance(f, tuple) else f, **kw)
+        out['tables'].append(dict(family=fam, args=args, nbytes=lay.nbytes,
+                                  fields={n: (o, str(dt), tuple(sh), nb) for n, (o, dt, sh, nb) in lay.fields.items()}))
+    # write -> partly filled buffer -> read, for the three families (small shapes)
+    torch.manual_seed(7)
+    rw = []
+    for fam, cls, kw, f in (('gdn', SlotLayout, dict(hv=4, hk=2, dk=64, dv=32, m=4, buffer_bits=8), (4, 'k', 32)),
+                            ('mamba2', Mamba2SlotLayout, dict(hv=4, hk=2, dk=32, dv=32, m=4, buffer_bits=16), (8, 'k', 32)),
+                            ('kda', KDASlotLayout, dict(hv=2, dk=32, dv=32, m=4, buffer_bits=8), (8, 'k', 32))):
+        lay = cls(fmt_of(f), **kw)
+        blob = torch.randint(0, 256, (5, lay.nbytes), dtype=torch.uint8)
+        V = lay.views(blob)
+        idx = torch.tensor([3, 1])
+        S = torch.randn(2, kw['hv'], kw['dv'], kw['dk'])
+        lay.write(V, idx, S)
+        after_write = blob.clone()
+        # a buffer with n = 2 live entries: finite decays, finite scales; dead entries stay random bytes
+        V['NPTR'][idx] = 2
+        V['GCUR'][idx] = -torch.rand_like(V['GCUR'][idx])
+        V['GB'][idx] = -torch.rand_like(V['GB'][idx]) * 0.5
+        if 'KBS' in V:
+            V['KBS'][idx] = (torch.rand_like(V['KBS'][idx].float()) * 0.01).half()
+            V['UBS'][idx] = (torch.rand_like(V['UBS'][idx].float()) * 0.01).half()
+        else:
+            V['KB'][idx] = torch.randn(V['KB'][idx].shape).to(torch.bfloat16)
+            V['UB'][idx] = torch.randn(V['UB'][idx].shape).to(torch.bfloat16)
+        rw.append(dict(family=fam, fmt=f, args=kw, idx=idx, S=S, after_write=after_write, blob=blob.clone(),
+                       read=lay.read(V, idx)))
+    out['rw'] = rw
+    save('slots.pt', out)
+
+
+if __name__ == '__main__':
+    golden_pack()
+    # config-1 shape (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start) in a 24-step excerpt
+    run_gdn('gdn_c1.pt', (8, 'k', 64), 4, 4, 2, 64, 64, 8, 16, 24, seed=1, S0_scale=0.0)
+    run_gdn('gdn_int4.pt', (4, 'k', 32), 2, 4, 2, 64, 64, 4, 8, 14, seed=2, v_head_scale=True)
+    run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 32, 1, 8, 4, seed=3, per_key=False)
+    run_kda('kda_int4.pt', (4, 'k', 32), 2, 3, 64, 64, 4, 8, 10, seed=4)
+    run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 32, 2, 16, 6, seed=5)
+    run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 32, 4, 8, 10, seed=6)
+    run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 64, 32, 2, 16, 6, seed=7)
+    golden_slots()
