@@ -1,0 +1,226 @@
+"""Benchmark of the packed-state decode step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn-int8-g128 | gdn-int8-g32 | gdn-int4-g64 | ...]
+
+Headline workload (default): Gated DeltaNet decode at the Qwen3.5-4B shape -- 32 value / 16 key heads, d_k = d_v = 128,
+256 slots, int8 state with one fp16 scale per (head, value row), int8 decode buffer of m = 8 tokens, bf16 q / k / v,
+g and beta given -- on 24 independent layer blobs stepped back to back (3.6 GB of state, so no layer's state survives
+in the 256 MiB Infinity Cache until its next step).  A "step" is one decode token through all 24 layers = 24 launches
+of the fused step kernel through the C ABI (``SlotLayout.step`` -> ``sq_gdn_step``).  All slots start from a zero
+state and advance in lockstep, so one step in m folds and re-quantizes every state tile (the reference's benchmark does
+the same: benchmarks/decode_state.py:41-66 there times graphs of m steps = one fold).
+
+Timing: W untimed warm-up steps, then exactly K steps between ``torch.cuda.synchronize()`` calls on the wall clock
+(``ms_per_step``), with HIP events on the launch stream around the same region.  The steps are replayed from a HIP
+graph of m steps (m x 24 kernel nodes) when K and W are multiples of m, otherwise launched eagerly.
+
+Prints ONE JSON line.  ``value`` = microseconds per layer per decode step (lower is better).  ``roofline`` prices the
+step kernel against HBM: achieved = algorithmic state bytes per launch / average launch duration, where the
+algorithmic bytes are (codes + scales) x (1 + 1/m) per slot (read every step, rewritten once per m steps) x slots.
+``cpu_baseline`` times the CPU oracle (a torch restatement of the reference's own CPU path) on this box's host cores
+on a bounded sample of the same workload; it is a reported baseline, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (family, bits, group, hv, hk, dk, dv, slots, layers)
+    'gdn-int8-g128': ('gdn', 8, 128, 32, 16, 128, 128, 256, 24),
+    'gdn-int8-g32': ('gdn', 8, 32, 32, 16, 128, 128, 256, 24),
+    'gdn-int4-g64': ('gdn', 4, 64, 32, 16, 128, 128, 256, 24),
+    'gdn-int4-g32': ('gdn', 4, 32, 32, 16, 128, 128, 256, 24),
+    'mamba2-int8-g128': ('mamba2', 8, 128, 128, 8, 128, 64, 128, 24),
+    'kda-int4-g32': ('kda', 4, 32, 32, 32, 128, 128, 256, 24),
+}
+
+# HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
+# over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
+MEASURED_TRAFFIC = {}
+
+
+def state_bytes_per_slot(bits, group, hv, dk, dv, m):
+    codes = hv * dv * dk * bits // 8
+    scales = hv * dv * (-(-dk // group)) * 2
+    return (codes + scales) * (1 + 1 / m)
+
+
+def build(workload, m, device):
+    import statequant_amd as sq
+    from statequant_amd.kernels import KDASlotLayout, Mamba2SlotLayout, SlotLayout
+    fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[workload]
+    fmt = sq.Quantizer(bits, 'k', group)
+    if fam == 'gdn':
+        lay = SlotLayout(fmt, hv, hk, dk, dv, m=m, buffer_bits=8)
+    elif fam == 'kda':
+        lay = KDASlotLayout(fmt, hv, dk, dv, m=m, buffer_bits=8)
+    else:
+        lay = Mamba2SlotLayout(fmt, hv, hk, dk, dv, m=m, buffer_bits=8)
+    blobs = [lay.alloc(slots + 1, device) for _ in range(layers)]            # slot 0 is the engine's null slot
+    views = [lay.views(b) for b in blobs]
+    gen = torch.Generator(device='cpu').manual_seed(0)
+    idx = (torch.randperm(slots, generator=gen) + 1).to(torch.int32).to(device)
+    return fam, lay, views, idx
+
+
+def make_inputs(fam, lay, slots, layers, m, device, seed=1):
+    """Synthetic inputs of one fold period: a distinct set per (step in period, layer), in the configs' distributions."""
+    gen = torch.Generator(device=device).manual_seed(seed)
+    r = lambda *s: torch.randn(*s, device=device, generator=gen)          # noqa: E731
+    hv, hk, dk, dv = lay.HV, lay.HK, lay.DK, lay.DV
+    out = []
+    for _ in range(m * layers):
+        if fam == 'gdn':
+            out.append(dict(q=r(slots, hk, dk).bfloat16(), k=r(slots, hk, dk).bfloat16(), v=r(slots, hv, dv).bfloat16(),
+                            g=-torch.nn.functional.softplus(r(slots, hv)), beta=torch.sigmoid(r(slots, hv))))
+        elif fam == 'kda':
+            out.append(dict(q=r(slots, hv, dk).bfloat16(), k=r(slots, hv, dk).bfloat16(), v=r(slots, hv, dv).bfloat16(),
+                            g=-torch.nn.functional.softplus(r(slots, hv, dk)), beta=torch.sigmoid(r(slots, hv))))
+        else:
+            out.append(dict(x=r(slots, hv, dv).bfloat16(), dt=r(slots, hv) * 0.5 - 2, B=r(slots, hk, dk).bfloat16(),
+                            C=r(slots, hk, dk).bfloat16()))
+    extra = {}
+    if fam == 'mamba2':
+        extra = dict(A=-torch.exp(torch.rand(hv, device=device, generator=gen) * 2), D=r(hv), dt_bias=r(hv) * 0.1)
+    return out, extra
+
+
+def launch(fam, lay, views, idx, inp, extra, out):
+    if fam == 'gdn':
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'])
+    elif fam == 'kda':
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out)
+    else:
+        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'])
+
+
+def cpu_baseline(workload, m, budget_s=20.0):
+    """The CPU oracle on a bounded sample of the workload: one layer, all slots, one fold period (m steps incl. the
+    fold), repeated while the budget lasts.  Returns the JSON object."""
+    from oracle import states as ST
+    fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[workload]
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(0)
+    r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
+    S0 = r(slots * hv, dv, dk) * 0.1
+    fmt = (bits, 'k', group)
+    if fam == 'gdn':
+        st = ST.GDNOracle(S0, fmt, m=m, hv=hv, hk=hk, buffer_bits=8)
+    elif fam == 'kda':
+        st = ST.KDAOracle(S0, fmt, m=m, hv=hv, buffer_bits=8)
+    else:
+        st = ST.Mamba2Oracle(S0, fmt, m=m, hv=hv, hk=hk, buffer_bits=8)
+        A, D, dtb = -torch.exp(torch.rand(hv, generator=gen) * 2), r(hv), r(hv) * 0.1
+    steps, t_total = 0, 0.0
+    while t_total < budget_s and steps < 4 * m:
+        for _ in range(m):
+            if fam == 'gdn':
+                args = (r(slots * hk, dk).bfloat16(), r(slots * hk, dk).bfloat16(), r(slots * hv, dv).bfloat16(),
+                        -torch.nn.functional.softplus(r(slots * hv)), torch.sigmoid(r(slots * hv)), dk ** -0.5)
+            elif fam == 'kda':
+                args = (r(slots * hv, dk).bfloat16(), r(slots * hv, dk).bfloat16(), r(slots * hv, dv).bfloat16(),
+                        -torch.nn.functional.softplus(r(slots * hv, dk)), torch.sigmoid(r(slots * hv)))
+            else:
+                args = (r(slots, hv, dv).bfloat16(), r(slots, hv) * 0.5 - 2, r(slots, hk, dk).bfloat16(),
+                        r(slots, hk, dk).bfloat16(), A, D, dtb, True, None)
+            t0 = time.perf_counter()
+            st.step(*args)
+            t_total += time.perf_counter() - t0
+            steps += 1
+    return {'value': round(t_total / steps * 1e6, 1), 'unit': 'us per layer-step', 'cores': cores, 'kind': 'port',
+            'sample': f'{workload}: 1 layer x {slots} slots, {steps} steps ({steps // m} fold periods of m={m}), '
+                      f'torch CPU oracle, {cores} threads'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=1024)
+    ap.add_argument('--warmup', type=int, default=512)
+    ap.add_argument('--workload', default='gdn-int8-g128', choices=list(WORKLOADS))
+    ap.add_argument('--m', type=int, default=8)
+    ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--cpu-budget', type=float, default=20.0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit('bench.py: this build measures one GPU; the decode step has no cross-GPU exchange (slots shard '
+                 'freely), so a multi-GPU figure would be N independent copies of this run. Use --gpus 1.')
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no GPU visible; the packed decode step only runs as HIP kernels')
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    m = a.m
+    fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
+    fam, lay, views, idx = build(a.workload, m, dev)
+    inputs, extra = make_inputs(fam, lay, slots, layers, m, dev)
+    out = torch.empty(slots, hv, dv, device=dev, dtype=torch.bfloat16)
+
+    def period():                                           # m steps x layers launches
+        for s in range(m):
+            for L in range(layers):
+                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out)
+
+    use_graph = not a.no_graph and a.steps % m == 0 and a.warmup % m == 0 and a.steps > 0
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        if use_graph:
+            period()                                        # one eager period first (module load etc.)
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                period()
+            run = lambda n: [graph.replay() for _ in range(n // m)]          # noqa: E731
+            done = m
+        else:
+            def run(n):
+                for s in range(n):
+                    for L in range(layers):
+                        launch(fam, lay, views[L], idx, inputs[(s % m) * layers + L], extra, out)
+            done = 0
+        run(max(a.warmup - done, 0))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        run(a.steps)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ev_ms = e0.elapsed_time(e1)
+    assert torch.isfinite(out.float()).all(), 'non-finite output'
+    n_launch = a.steps * layers
+    us_wall = wall * 1e6 / n_launch
+    us_kernel = ev_ms * 1e3 / n_launch                      # average launch-to-launch duration on the stream
+    alg_bytes = state_bytes_per_slot(bits, group, hv, dk, dv, m) * slots
+    achieved = alg_bytes / (us_kernel * 1e-6) / 1e9
+    res = {
+        'metric': 'us_per_layer_decode_step', 'value': round(us_wall, 3), 'unit': 'us',
+        'n_gpus': 1, 'steps': a.steps, 'warmup': a.warmup, 'ms_per_step': round(wall * 1e3 / a.steps, 5),
+        'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': a.workload, 'family': fam, 'slots': slots, 'layers': layers, 'value_heads': hv,
+                   'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': f'int{bits} key-axis group {group}, fp16 scales',
+                   'buffer': f'int8, m={m}', 'inputs': 'bf16', 'launch': 'hip-graph' if use_graph else 'eager',
+                   'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
+        'hbm_gbs': round(achieved, 1),
+        'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(a.workload),
+                     'kernel_us': round(us_kernel, 3), 'algorithmic_bytes_per_launch': round(alg_bytes)},
+    }
+    if not a.no_cpu_baseline:
+        res['cpu_baseline'] = cpu_baseline(a.workload, m, a.cpu_budget)
+    print(json.dumps(res))
+
+
+if __name__ == '__main__':
+    main()

@@ -74,8 +74,11 @@ def _bits(fmt):
 
 
 def _scale_of(amax, qmax):
-    """absmax -> stored scale: max(amax, 1e-8) / qmax, to fp16 and back, floored at 2^-24 (quantizer.py:159-164)."""
-    return (amax.clamp_min(1e-8) / qmax).to(torch.float16).float().clamp_min(_FP16_MIN)
+    """absmax -> stored scale: max(amax, 1e-8) / qmax, to fp16 and back, floored at 2^-24 (quantizer.py:159-164).
+    The divisor is a device tensor: torch's GPU division by a Python scalar multiplies by the rounded reciprocal,
+    which is not the IEEE quotient the kernels and the CPU path compute."""
+    return (amax.clamp_min(1e-8) / torch.full((), qmax, device=amax.device)).to(torch.float16).float() \
+        .clamp_min(_FP16_MIN)
 
 
 # ---------------------------------------------------------------------------------------------------------------

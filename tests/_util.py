@@ -1,0 +1,83 @@
+"""Shared helpers of the GPU parity tests: seeded inputs in the distributions the benchmark configs name, and the
+kernel <-> oracle hand-over used for per-step comparison.
+
+Protocol (the reference's own, /root/reference/tests/test_kernels.py:83-110): the HIP kernel and the CPU oracle take
+the same token; outputs are compared; the entries the kernel appended to its buffer are compared with the oracle's
+and then ADOPTED by the oracle, and after a fold the kernel's codes and scales likewise, so a rounding flip is counted
+once and never inherited by later steps.
+"""
+import torch
+
+import statequant_amd as sq
+
+
+def quantizer(fmt):
+    return sq.Quantizer(*fmt)
+
+
+def gdn_token(gen, B, HV, HK, DK, DV, dtype=torch.float32, v_scale=None):
+    """q, k ~ N(0,1) per KEY head; v ~ N(0,1); beta = sigmoid(N(0,1)); g = -softplus(N(0,1)) (CPU tensors)."""
+    r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
+    q, k, v = r(B, HK, DK), r(B, HK, DK), r(B, HV, DV)
+    if v_scale is not None:
+        v = v * v_scale[None, :, None]
+    g = -torch.nn.functional.softplus(r(B, HV))
+    beta = torch.sigmoid(r(B, HV))
+    return q.to(dtype), k.to(dtype), v.to(dtype), g, beta
+
+
+def buffer_entry(T, slot, qbuf):
+    """Dequantized (K, U) of buffer slot ``slot`` from a kernel state's tensors (dict with KB, UB, KBS, UBS)."""
+    kb, ub = T['KB'][:, slot].float(), T['UB'][:, slot].float()
+    if qbuf:
+        kb, ub = kb * T['KBS'][:, slot, None].float(), ub * T['UBS'][:, slot, None].float()
+    return kb.cpu(), ub.cpu()
+
+
+class Tally:
+    """Running comparison figures of one kernel-vs-oracle run."""
+
+    def __init__(self):
+        self.worst_o = 0.0
+        self.buf_flips = self.buf_entries = 0
+        self.code_mism = self.code_n = self.scale_mism = 0
+        self.code_far = 0                     # codes differing by more than one step
+        self.worst_raw = 0.0
+        self.worst_deq = 0.0
+        self.folds = 0
+
+    def out(self, o, ref):
+        self.worst_o = max(self.worst_o, ((o - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item())
+
+    def entries(self, got, want):
+        self.buf_flips += (got != want).sum().item()
+        self.buf_entries += want.numel()
+
+    def fold(self, codes, scales, ref, bits):
+        """codes / scales of the kernel (CPU copies) vs the oracle that has just folded the same buffer."""
+        self.folds += 1
+        a, b = unpack_nib(codes, bits), unpack_nib(ref.codes, bits)
+        d = (a.int() - b.int()).abs()
+        self.code_mism += (d != 0).sum().item()
+        self.code_far += (d > 1).sum().item()
+        self.code_n += d.numel()
+        self.scale_mism += (scales != ref.scales).sum().item()
+        from oracle.formats import unpack_vk
+        deq = unpack_vk(codes, scales, ref.fmt, ref.DK)
+        den = ref.S_raw.abs().max().clamp_min(1e-30)
+        self.worst_raw = max(self.worst_raw, ((deq - ref.S_raw).abs().max() / den).item())
+        self.worst_deq = max(self.worst_deq, ((deq - ref.S0).abs().max() / den).item())
+
+    def report(self, tag):
+        return (f'[{tag}] max rel |o - o_oracle| {self.worst_o:.2e}; {self.folds} folds: codes differing '
+                f'{self.code_mism} of {self.code_n} ({100 * self.code_mism / max(self.code_n, 1):.5f}%), by more than '
+                f'1 LSB {self.code_far}, scales differing {self.scale_mism}; max rel |S - S_raw_oracle| '
+                f'{self.worst_raw:.2e}; buffer entries flipped {self.buf_flips} of {self.buf_entries}')
+
+
+def unpack_nib(codes, bits):
+    """Stored codes -> one integer per code (int4 bytes split into their two nibbles)."""
+    if bits == 8:
+        return codes.to(torch.int16)
+    c = codes.to(torch.int16)
+    return torch.stack(((c & 15) - 8, ((c >> 4) & 15) - 8), -1).flatten(-2)

@@ -190,12 +190,12 @@ def golden_slots():
 
 if __name__ == '__main__':
     golden_pack()
-    # config-1 shape (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start) in a 24-step excerpt
-    run_gdn('gdn_c1.pt', (8, 'k', 64), 4, 4, 2, 64, 64, 8, 16, 24, seed=1, S0_scale=0.0)
+    # config-1 shape (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start) in a 17-step excerpt (two folds)
+    run_gdn('gdn_c1.pt', (8, 'k', 64), 4, 4, 2, 64, 64, 8, 16, 17, seed=1, S0_scale=0.0)
     run_gdn('gdn_int4.pt', (4, 'k', 32), 2, 4, 2, 64, 64, 4, 8, 14, seed=2, v_head_scale=True)
-    run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 32, 1, 8, 4, seed=3, per_key=False)
+    run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 64, 1, 8, 4, seed=3, per_key=False)
     run_kda('kda_int4.pt', (4, 'k', 32), 2, 3, 64, 64, 4, 8, 10, seed=4)
-    run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 32, 2, 16, 6, seed=5)
-    run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 32, 4, 8, 10, seed=6)
-    run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 64, 32, 2, 16, 6, seed=7)
+    run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 64, 2, 16, 6, seed=5)
+    run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 64, 4, 8, 10, seed=6)
+    run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 128, 64, 2, 16, 6, seed=7)
     golden_slots()

@@ -1,0 +1,338 @@
+"""Gated DeltaNet HIP step (through the C ABI) against the CPU oracle and the reference's golden vectors.
+
+Mirrors the reference's tests/test_kernels.py (decode vs torch reference), test_slots.py (slot step vs lockstep,
+padding rows, nothing written outside live slots, in-kernel gating, read / write) and test_fused.py's counter checks.
+Tolerances: the task's bar is o and dequantized state within 1e-2 relative, >= 99.9 % identical codes, rest +-1 LSB;
+the asserts below hold the kernel to the much tighter figures the reference demands of its own kernels
+(tests/test_kernels.py:129-134 there): o within 2e-5, <= 1e-4 of codes / buffer entries flipped.
+"""
+import pytest
+import torch
+
+import statequant_amd as sq
+from oracle import states as ST
+from statequant_amd.kernels import PackedGDNState, SlotLayout, pack_vk, unpack_vk
+from tests._util import Tally, buffer_entry, gdn_token, quantizer
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+FORMATS = {'int4-k-g64': (4, 'k', 64), 'int8-k-g32': (8, 'k', 32), 'int8-k-g128': (8, 'k', 128),
+           'int4-k-g32': (4, 'k', 32)}
+
+
+def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.float32, S0_scale=0.5, DV=None):
+    DV = DV or D
+    gen = torch.Generator().manual_seed(seed)
+    S0 = torch.randn(B * HV, DV, D, generator=gen) * S0_scale                    # value-major
+    ker = PackedGDNState(S0.transpose(1, 2).to(DEV), quantizer(fmt), m=m, hv=HV, hk=HK, buffer_bits=bb,
+                         out_dtype=torch.float32)
+    ref = ST.GDNOracle(S0, fmt, m=m, hv=HV, hk=HK, buffer_bits=bb, auto_fold=False)
+    assert torch.equal(ker.codes.cpu(), ref.codes) and torch.equal(ker.scales.cpu(), ref.scales)
+    tal = Tally()
+    scale = D ** -0.5
+    for t in range(T):
+        q, k, v, g, beta = gdn_token(gen, B, HV, HK, D, DV, dtype)
+        slot = ker.n
+        o = ker.step(q.reshape(B * HK, D).to(DEV), k.reshape(B * HK, D).to(DEV), v.reshape(B * HV, DV).to(DEV),
+                     g.reshape(-1).to(DEV), beta.reshape(-1).to(DEV), scale).cpu()
+        r = ref.step(q.reshape(B * HK, D), k.reshape(B * HK, D), v.reshape(B * HV, DV), g.reshape(-1),
+                     beta.reshape(-1), scale)
+        tal.out(o, r)
+        kb, ub = buffer_entry(dict(KB=ker.KB, UB=ker.UB, KBS=ker.KBS, UBS=ker.UBS), slot, bb == 8)
+        tal.entries(kb, ref.K[:, slot])
+        tal.entries(ub, ref.U[:, slot])
+        assert torch.equal(ker.GB[:, slot].cpu(), ref.G[:, slot]), t          # decays: bit-equal
+        ref.K[:, slot], ref.U[:, slot] = kb, ub
+        if ref.n == m:
+            ref.fold()
+        assert ker.n == ref.n
+        if ref.n == 0:
+            assert torch.equal(ker.GCUR.cpu(), torch.zeros(B * HV))
+            codes, scales = ker.codes.cpu(), ker.scales.cpu()
+            tal.fold(codes, scales, ref, fmt[0])
+            ref.adopt(codes, scales)
+        else:
+            assert torch.equal(ker.GCUR.cpu(), ref.gcur)
+        assert torch.equal(ker.NPTR.cpu(), torch.full((B, HV), ref.n, dtype=torch.int32))
+    return tal
+
+
+def check(tal, tag, T, m):
+    print('\n' + tal.report(tag))
+    assert tal.folds == T // m
+    assert tal.worst_o < 2e-5, tal.worst_o
+    assert tal.buf_flips <= max(1, 1e-4 * tal.buf_entries), tal.buf_flips
+    assert tal.code_mism <= max(1, 1e-4 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)
+    assert tal.scale_mism <= max(1, 1e-4 * tal.code_n / 32)
+    assert tal.worst_raw < 0.2
+
+
+@pytest.mark.parametrize('name', list(FORMATS))
+@pytest.mark.parametrize('m', [1, 8, 16])
+@pytest.mark.parametrize('bb', [8, 16])
+def test_decode_vs_oracle(name, m, bb):
+    check(run_decode(FORMATS[name], m, bb), f'{name} m={m} buf{bb}', 40, m)
+
+
+@pytest.mark.parametrize('D,DV,HV,HK,fmt', [(64, 64, 4, 2, (8, 'k', 64)), (64, 64, 4, 4, (4, 'k', 32)),
+                                            (96, 192, 3, 3, (4, 'k', 64)), (96, 192, 2, 1, (8, 'k', 32)),
+                                            (96, 96, 2, 2, (8, 'k', 128))])
+def test_other_head_shapes(D, DV, HV, HK, fmt):
+    """d = 64 (the CPU-reference config's head), OLMo-Hybrid's 96 x 192 with a ragged last key group, 96 x 96."""
+    T, m = 20, 4
+    check(run_decode(fmt, m, 8, B=3, HV=HV, HK=HK, D=D, DV=DV, T=T), f'{D}x{DV} {fmt}', T, m)
+
+
+def test_bf16_inputs_and_output():
+    """bf16 q, k, v (the serving dtype): the kernel upcasts exactly; out_dtype bf16 rounds the fp32 result."""
+    tal = run_decode((8, 'k', 128), 8, 8, dtype=torch.bfloat16, T=16)
+    check(tal, 'bf16 inputs', 16, 8)
+    gen = torch.Generator().manual_seed(5)
+    S0 = torch.randn(8, 128, 128, generator=gen) * 0.5
+    a = PackedGDNState(S0.to(DEV), quantizer((4, 'k', 64)), m=8, hv=4, hk=2, out_dtype=torch.float32)
+    b = PackedGDNState(S0.to(DEV), quantizer((4, 'k', 64)), m=8, hv=4, hk=2, out_dtype=torch.bfloat16)
+    c = PackedGDNState(S0.to(DEV), quantizer((4, 'k', 64)), m=8, hv=4, hk=2, out_dtype=torch.float16)
+    for t in range(10):
+        q, k, v, g, beta = (x.to(DEV) for x in gdn_token(gen, 2, 4, 2, 128, 128, torch.bfloat16))
+        args = (q.reshape(4, 128), k.reshape(4, 128), v.reshape(8, 128), g.reshape(-1), beta.reshape(-1), 128 ** -0.5)
+        oa, ob, oc = a.step(*args), b.step(*args), c.step(*args)
+        assert torch.equal(oa.to(torch.bfloat16), ob) and torch.equal(oa.to(torch.float16), oc)
+    assert torch.equal(a.codes, b.codes) and torch.equal(a.UB, b.UB)
+
+
+def test_q_k_per_value_head_matches_per_key_head():
+    """q, k handed per value head [BH, d_k] (expanded over the GQA group) == per key head [B * hk, d_k]
+    (the reference's tests/test_kernels.py:137-150)."""
+    B, HV, HK, D = 2, 4, 2, 128
+    gen = torch.Generator().manual_seed(3)
+    S0 = torch.randn(B * HV, D, D, generator=gen).to(DEV)
+    a = PackedGDNState(S0, quantizer((4, 'k', 64)), m=8, hv=HV, hk=HK, out_dtype=torch.float32)
+    b = PackedGDNState(S0, quantizer((4, 'k', 64)), m=8, hv=HV, hk=HK, out_dtype=torch.float32)
+    for t in range(10):
+        q, k, v, g, beta = (x.to(DEV) for x in gdn_token(gen, B, HV, HK, D, D))
+        qf = q.repeat_interleave(HV // HK, 1).reshape(B * HV, D).contiguous()
+        kf = k.repeat_interleave(HV // HK, 1).reshape(B * HV, D).contiguous()
+        oa = a.step(qf, kf, v.reshape(B * HV, D), g.reshape(-1), beta.reshape(-1), D ** -0.5).clone()
+        ob = b.step(q.reshape(B * HK, D), k.reshape(B * HK, D), v.reshape(B * HV, D), g.reshape(-1), beta.reshape(-1),
+                    D ** -0.5)
+        assert torch.equal(oa, ob)
+    assert torch.equal(a.codes, b.codes) and torch.equal(a.KB, b.KB)
+
+
+@pytest.mark.parametrize('name', ['gdn_c1.pt', 'gdn_int4.pt', 'gdn_int8_m1.pt'])
+def test_against_reference_golden_vectors(golden, name):
+    """The HIP step replayed on the inputs the reference's own ReferenceGDNState was recorded on: outputs, appended
+    buffer entries, codes and scales after every fold.  The kernel state is re-seeded from the reference's record
+    after each step (its buffer entries) and fold (its codes), so every step is compared on its own."""
+    rec = golden(name)
+    B, HV, HK, DK, DV, m, bb = (rec[k] for k in ('B', 'HV', 'HK', 'DK', 'DV', 'm', 'buffer_bits'))
+    ker = PackedGDNState(rec['S0'].to(DEV), quantizer(rec['fmt']), m=m, hv=HV, hk=HK, buffer_bits=bb,
+                         out_dtype=torch.float32)
+    assert torch.equal(ker.codes.cpu(), rec['codes0']) and torch.equal(ker.scales.cpu(), rec['scales0'])
+    from oracle.formats import round_buf_parts
+    worst, flips, entries, mism, far, ncodes = 0.0, 0, 0, 0, 0, 0
+    for st in rec['steps']:
+        n = st['n']
+        assert ker.n == n
+        dev = lambda x: x.to(DEV).contiguous()      # noqa: E731
+        o = ker.step(dev(st['q']), dev(st['k']), dev(st['v']), dev(st['g']), dev(st['beta']), rec['scale']).cpu()
+        worst = max(worst, ((o - st['o']).abs().max() / st['o'].abs().max().clamp_min(1e-30)).item())
+        kb, ub = buffer_entry(dict(KB=ker.KB, UB=ker.UB, KBS=ker.KBS, UBS=ker.UBS), n, bb == 8)
+        flips += (kb != st['K']).sum().item() + (ub != st['U']).sum().item()
+        entries += kb.numel() + ub.numel()
+        assert torch.equal(ker.GB[:, n].cpu(), st['G'])
+        if 'codes' in st:
+            from tests._util import unpack_nib
+            d = (unpack_nib(ker.codes.cpu(), rec['fmt'][0]).int() - unpack_nib(st['codes'], rec['fmt'][0]).int()).abs()
+            mism += (d != 0).sum().item()
+            far += (d > 1).sum().item()
+            ncodes += d.numel()
+            deq = unpack_vk(ker.codes, ker.scales, quantizer(rec['fmt']), DK).cpu()
+            raw = st['S_raw'].transpose(1, 2)
+            assert ((deq - raw).abs().max() / raw.abs().max()).item() < 0.2
+            ker.codes.copy_(st['codes'])
+            ker.scales.copy_(st['scales'])
+        else:                                       # adopt the reference's entries (int8: as codes + scale)
+            if bb == 8:
+                kc, ks = round_buf_parts(st['K'])
+                uc, us = round_buf_parts(st['U'])
+                ker.KB[:, n].copy_(kc), ker.KBS[:, n].copy_(ks), ker.UB[:, n].copy_(uc), ker.UBS[:, n].copy_(us)
+            else:
+                ker.KB[:, n].copy_(st['K'].to(torch.bfloat16)), ker.UB[:, n].copy_(st['U'].to(torch.bfloat16))
+    print(f'\n[{name}] max rel |o - o_ref| {worst:.2e}; buffer flips {flips}/{entries}; codes differing {mism}/{ncodes}')
+    assert worst < 2e-5
+    assert flips <= max(1, 1e-4 * entries)
+    assert mism <= max(1, 1e-4 * ncodes) and far == 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# slots
+# ---------------------------------------------------------------------------------------------------------------
+HV, HK, D = 4, 2, 128
+
+
+def _setup(fmt, m, bb, n_slots=8, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=bb)
+    # a blob with a slot stride larger than the layout (padded pages) and garbage everywhere else
+    raw = torch.randint(0, 256, (n_slots, lay.nbytes + 4096), dtype=torch.uint8, generator=gen).to(DEV)
+    blob = raw[:, 2048:2048 + lay.nbytes]
+    views = lay.views(blob)
+    slots = [5, 2, 7]
+    S0 = [torch.randn(HV, D, D, generator=gen).to(DEV) * 0.5 for _ in slots]            # [HV, d_k, d_v]
+    refs = [PackedGDNState(s, quantizer(fmt), m=m, hv=HV, hk=HK, buffer_bits=bb, out_dtype=torch.float32)
+            for s in S0]
+    lay.write(views, torch.tensor(slots, device=DEV), torch.stack([s.transpose(-1, -2) for s in S0]))
+    return lay, raw, blob, views, slots, refs
+
+
+@pytest.mark.parametrize('name', ['int4-k-g64', 'int8-k-g32'])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+def test_slot_step_matches_lockstep_per_sequence(name, m, bb):
+    """Slot-addressed step == the lockstep state run per sequence, bit for bit (same kernel, other strides);
+    padding rows give zeros; nothing outside the live slots' blobs is written (reference: tests/test_slots.py:54-109)."""
+    fmt = FORMATS[name]
+    lay, raw, blob, views, slots, refs = _setup(fmt, m, bb)
+    for i, r in enumerate(refs):
+        assert torch.equal(views['S'][slots[i]], r.codes.view(HV, *r.codes.shape[1:]))
+    outside = raw.clone()
+    sched = torch.Generator().manual_seed(1)
+    gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
+    steps = [0] * len(slots)
+    for t in range(30):
+        live = [i for i in torch.randperm(len(slots), generator=sched).tolist()
+                if torch.rand(1, generator=sched).item() < 0.7]
+        rows = live + ['pad0', 'padneg']
+        rows = [rows[j] for j in torch.randperm(len(rows), generator=sched).tolist()]
+        idx = torch.tensor([slots[r] if isinstance(r, int) else (0 if r == 'pad0' else -1) for r in rows],
+                           device=DEV, dtype=torch.int32)
+        Bn = len(rows)
+        q, k = torch.zeros(Bn, HK, D, device=DEV), torch.zeros(Bn, HK, D, device=DEV)
+        v = torch.zeros(Bn, HV, D, device=DEV)
+        g, beta = torch.zeros(Bn, HV, device=DEV), torch.zeros(Bn, HV, device=DEV)
+        want = {}
+        for b, r in enumerate(rows):
+            if not isinstance(r, int):
+                continue
+            tq, tk, tv, tg, tb = (x[0].to(DEV) for x in gdn_token(gens[r], 1, HV, HK, D, D))
+            q[b], k[b], v[b], g[b], beta[b] = tq, tk, tv, tg, tb
+            want[b] = refs[r].step(tq.contiguous(), tk.contiguous(), tv.contiguous(), tg.contiguous(),
+                                   tb.contiguous(), D ** -0.5).clone()
+            steps[r] += 1
+        out = torch.full((Bn, HV, D), 7., device=DEV)
+        lay.step(views, idx, q, k, v, out, D ** -0.5, g=g, beta=beta)
+        for b, r in enumerate(rows):
+            if isinstance(r, int):
+                assert torch.equal(out[b], want[b].view(HV, D)), (t, b)
+                assert views['NPTR'][slots[r], :HV].tolist() == [steps[r] % m] * HV == [refs[r].n] * HV
+                assert torch.equal(views['S'][slots[r]], refs[r].codes.view(HV, *refs[r].codes.shape[1:]))
+                assert torch.equal(views['SC'][slots[r]], refs[r].scales.view(HV, *refs[r].scales.shape[1:]))
+                w = min(steps[r], m)                # buffer slots written so far (the rest: the blob's garbage)
+                assert torch.equal(views['UB'][slots[r]][:, :w], refs[r].UB.view(HV, m, D)[:, :w])
+                assert torch.equal(views['KB'][slots[r]][:, :w], refs[r].KB.view(HK, m, D)[:, :w])
+                assert torch.equal(views['GB'][slots[r]][:, :w], refs[r].GB.view(HV, m)[:, :w])
+                if bb == 8:
+                    assert torch.equal(views['UBS'][slots[r]][:, :w], refs[r].UBS.view(HV, m)[:, :w])
+                    assert torch.equal(views['KBS'][slots[r]][:, :w], refs[r].KBS.view(HK, m)[:, :w])
+                assert torch.equal(views['GCUR'][slots[r]], refs[r].GCUR.view(HV))
+            else:
+                assert torch.equal(out[b], torch.zeros_like(out[b]))
+    keep = torch.ones_like(raw, dtype=torch.bool)
+    for s in slots:
+        keep[s, 2048:2048 + lay.nbytes] = False
+    assert torch.equal(raw[keep], outside[keep])
+
+
+@pytest.mark.parametrize('name', ['int4-k-g64', 'int8-k-g128'])
+def test_read_is_the_state_the_next_step_reads(name):
+    """read() (stored state advanced over the pending buffer) + one textbook fp32 step predicts the kernel's next
+    output (reference: tests/test_slots.py:112-136)."""
+    m = 8
+    lay, raw, blob, views, slots, refs = _setup(FORMATS[name], m, 8)
+    gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
+    idx = torch.tensor(slots, device=DEV, dtype=torch.int32)
+    for t in range(13):
+        toks = [gdn_token(gn, 1, HV, HK, D, D) for gn in gens]
+        q, k, v, g, beta = (torch.cat(x).to(DEV) for x in zip(*toks))
+        out = torch.empty(len(slots), HV, D, device=DEV)
+        if t == 12:
+            S = lay.read(views, idx)
+            qn = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+            kn = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            qx, kx = qn.repeat_interleave(HV // HK, 1), kn.repeat_interleave(HV // HK, 1)
+            a = g.exp()[..., None]
+            u = beta[..., None] * (v - a * torch.einsum('phvk,phk->phv', S, kx))
+            o_pred = a * torch.einsum('phvk,phk->phv', S, qx) + (qx * kx).sum(-1, keepdim=True) * u
+        lay.step(views, idx, q, k, v, out, D ** -0.5, g=g, beta=beta)
+    assert int(views['NPTR'][slots[0], 0]) == 13 % m
+    rel = ((out - o_pred).norm() / o_pred.norm()).item()
+    assert rel < 1e-5, rel
+
+
+def test_write_read_roundtrip_and_reset():
+    fmt = quantizer((4, 'k', 64))
+    lay = SlotLayout(fmt, HV, HK, D, D, m=8)
+    blob = torch.randint(0, 256, (4, lay.nbytes), dtype=torch.uint8).to(DEV)
+    views = lay.views(blob)
+    S = torch.randn(2, HV, D, D, device=DEV)
+    idx = torch.tensor([3, 1], device=DEV)
+    lay.write(views, idx, S)
+    got = lay.read(views, idx)
+    c, s = pack_vk(S.reshape(-1, D, D), fmt)
+    assert torch.equal(got, unpack_vk(c, s, fmt, D).view_as(S))
+    assert views['NPTR'][idx, 0].tolist() == [0, 0] and torch.equal(views['GCUR'][idx], torch.zeros(2, HV, device=DEV))
+
+
+def test_in_kernel_gating():
+    """gate=(a, b, A_log, dt_bias) formed in the kernel == g, beta formed on the host (oracle.gdn_gate), with the
+    bf16 gate inputs vLLM passes (reference: tests/test_slots.py:153-171)."""
+    lay, raw, blob, views, slots, refs = _setup((4, 'k', 64), 8, 8)
+    gen = torch.Generator().manual_seed(3)
+    Bn = len(slots)
+    q, k, v = (torch.randn(Bn, h, D, generator=gen).to(DEV) for h in (HK, HK, HV))
+    a = (torch.randn(Bn, HV, generator=gen) * 3).to(torch.bfloat16)
+    a[0, 0] = 30.0                                                # softplus pass-through above 20
+    bb = torch.randn(Bn, HV, generator=gen).to(torch.bfloat16)
+    A_log = torch.randn(HV, generator=gen) * 0.5
+    dt_bias = torch.randn(HV, generator=gen).to(torch.bfloat16)
+    g, beta = ST.gdn_gate(a, bb, A_log, dt_bias)
+    v2 = lay.views(blob.clone())
+    idx = torch.tensor(slots, device=DEV, dtype=torch.int32)
+    o1, o2 = torch.empty(Bn, HV, D, device=DEV), torch.empty(Bn, HV, D, device=DEV)
+    lay.step(views, idx, q, k, v, o1, D ** -0.5, g=g.to(DEV), beta=beta.to(DEV))
+    lay.step(v2, idx, q, k, v, o2, D ** -0.5, gate=(a.to(DEV), bb.to(DEV), A_log.to(DEV), dt_bias.to(DEV)))
+    assert torch.allclose(o1, o2, rtol=1e-5, atol=1e-6), (o1 - o2).abs().max()
+    assert torch.allclose(views['GB'], v2['GB'], rtol=1e-6, atol=1e-7)
+
+
+def test_strided_inputs_like_the_serving_engine():
+    """q, k, v as column slices of one wider activation (row stride > row length), out contiguous."""
+    lay, raw, blob, views, slots, refs = _setup((8, 'k', 32), 8, 8)
+    gen = torch.Generator().manual_seed(4)
+    Bn = len(slots)
+    wide = torch.randn(Bn, 2 * HK * D + HV * D + 64, generator=gen).to(DEV).to(torch.bfloat16)
+    q = wide[:, :HK * D].view(Bn, HK, D)
+    k = wide[:, HK * D:2 * HK * D].view(Bn, HK, D)
+    v = wide[:, 2 * HK * D:2 * HK * D + HV * D].view(Bn, HV, D)
+    g = -torch.rand(Bn, HV, generator=gen).to(DEV)
+    beta = torch.rand(Bn, HV, generator=gen).to(DEV)
+    v2 = lay.views(blob.clone())
+    idx = torch.tensor(slots, device=DEV, dtype=torch.int32)
+    o1, o2 = torch.empty(Bn, HV, D, device=DEV), torch.empty(Bn, HV, D, device=DEV)
+    lay.step(views, idx, q, k, v, o1, D ** -0.5, g=g, beta=beta)
+    lay.step(v2, idx, q.contiguous(), k.contiguous(), v.contiguous(), o2, D ** -0.5, g=g, beta=beta)
+    assert torch.equal(o1, o2)
+
+
+def test_empty_batch_and_errors():
+    lay = SlotLayout(quantizer((4, 'k', 64)), HV, HK, D, D)
+    blob = lay.alloc(2, DEV)
+    out = torch.zeros(0, HV, D, device=DEV)
+    e = torch.zeros(0, HK, D, device=DEV)
+    assert lay.step(lay.views(blob), torch.zeros(0, dtype=torch.int32, device=DEV), e, e, out, out, 1.0,
+                    g=out, beta=out) is out
+    with pytest.raises(NotImplementedError):                     # value-axis groups: layout yes, HIP step not built
+        SlotLayout(quantizer((4, 'v', 32)), HV, HK, D, D)._layout_struct()
+    with pytest.raises(RuntimeError):                            # CPU tensors never reach a kernel
+        PackedGDNState(torch.zeros(8, D, D), quantizer((4, 'k', 64)), hv=HV, hk=HK)

@@ -1,0 +1,185 @@
+"""Host-side logic that needs no GPU: storage format, per-slot byte layouts against the reference's documented
+totals, the prefill-side read / write on CPU blobs, the C-ABI library's symbols, and loud failure off the GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import statequant_amd as sq
+from oracle import formats as F
+from oracle import slots as OSL
+from statequant_amd.kernels import (KDASlotLayout, Mamba2SlotLayout, PackedGDNState, SlotLayout, _hip, pack, pack_vk,
+                                    packed_format, unpack, unpack_vk)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize('bits', [4, 8])
+@pytest.mark.parametrize('axis', ['k', 'v'])
+@pytest.mark.parametrize('group', [32, 64])
+def test_pack_roundtrip_matches_fake(bits, axis, group):
+    """unpack(pack(S)) == Quantizer(..., scale_dtype='fp16').fake(S) bit for bit, incl. all-zero groups and scales in
+    the fp16 subnormal range (the reference's tests/test_kernels.py:26-49), and == the oracle's pack."""
+    torch.manual_seed(0)
+    S = torch.randn(8, 128, 128) * torch.rand(8, 128, 1) * 3
+    S[0, :, :64] = 0
+    S[1] *= 1e-6
+    q = sq.Quantizer(bits, axis, group)
+    codes, scales = pack(S, q)
+    assert scales.dtype == torch.float16
+    assert codes.dtype == (torch.uint8 if bits == 4 else torch.int8)
+    assert codes.shape == (8, 128, 128 // (2 if bits == 4 else 1))
+    got = unpack(codes, scales, q, 128)
+    assert torch.equal(got, sq.Quantizer(bits, axis, group, scale_dtype='fp16').fake(S))
+    assert torch.equal(packed_format(q).fake(S), got)
+    oc, os_ = F.pack_vk(S.transpose(1, 2).contiguous(), (bits, axis, group))
+    assert torch.equal(codes, oc) and torch.equal(scales, os_)
+    c4, s4 = pack(S.reshape(2, 4, 128, 128), q)
+    assert torch.equal(c4, codes) and torch.equal(s4, scales)
+    # all-zero group: amax 1e-8 / qmax rounds to fp16 zero and is floored at 2^-24; codes 0
+    if axis == 'k':
+        assert (scales[0, :64].float() == 2.0 ** -24).all()          # S[0, :, :64] = 0: value rows 0..63 all zero
+
+
+def test_ragged_key_group_and_bf16():
+    X = torch.randn(3, 32, 96)
+    q = sq.Quantizer(4, 'k', 64)
+    c, s = pack_vk(X, q)
+    assert s.shape == (3, 32, 2) and c.shape == (3, 32, 48)
+    deq = unpack_vk(c, s, q, 96)
+    # a ragged group is quantized on its own: same as quantizing the two column blocks separately
+    a = unpack_vk(*pack_vk(X[..., :64].contiguous(), q), q, 64)
+    b = unpack_vk(*pack_vk(X[..., 64:].contiguous(), sq.Quantizer(4, 'k', 32)), sq.Quantizer(4, 'k', 32), 32)
+    assert torch.equal(deq, torch.cat([a, b], -1))
+    S = torch.randn(4, 64, 64)
+    cb, sb = pack(S, 'bf16')
+    assert torch.equal(unpack(cb, sb, 'bf16', 64), S.to(torch.bfloat16).float())
+
+
+def test_brute_force_per_group_numpy():
+    """pack_vk against a scalar restatement with np.float16 on a tiny input (independent of torch's kernels)."""
+    import numpy as np
+    rng = np.random.default_rng(0)
+    X = (rng.standard_normal((2, 4, 32)) * np.array([1.0, 1e-6])[:, None, None]).astype(np.float32)
+    X[0, 1, :16] = 0
+    for bits, g in ((4, 16), (8, 32)):
+        qmax = 2 ** (bits - 1) - 1
+        codes, scales = pack_vk(torch.from_numpy(X), sq.Quantizer(bits, 'k', g))
+        deq = unpack_vk(codes, scales, sq.Quantizer(bits, 'k', g), 32).numpy()
+        for n in range(2):
+            for r in range(4):
+                for gi in range(32 // g):
+                    blk = X[n, r, gi * g:(gi + 1) * g]
+                    s = np.float32(np.float16(np.float32(max(np.abs(blk).max(), np.float32(1e-8))) / np.float32(qmax)))
+                    s = max(s, np.float32(2.0 ** -24))
+                    want = np.clip(np.rint(blk / s), -qmax, qmax) * s
+                    assert np.array_equal(deq[n, r, gi * g:(gi + 1) * g], want.astype(np.float32))
+
+
+# per-slot bytes the reference documents for real models (docs/vllm.md:116-119, 143-146, 188-191 there)
+DOC_TOTALS = [
+    (SlotLayout, dict(hv=30, hk=30, dk=96, dv=192), {'pace4': 370816, 'int8k': 658816, 'int4v': 382336, 'bf16': 1177216}),
+    (Mamba2SlotLayout, dict(hv=96, hk=8, dk=128, dv=80), {'pace4': 597376, 'int8k': 1119616, 'int4v16': 689536,
+                                                           'bf16': 2041216}),
+    (KDASlotLayout, dict(hv=16, dk=128, dv=128), {'pace4': 246336, 'int8k': 385600, 'int4v': 254528, 'bf16': 631360}),
+]
+PRESETS = {'pace4': sq.Quantizer(4, 'k', 64), 'int8k': sq.Quantizer(8, 'k', 32), 'int4v': sq.Quantizer(4, 'v', 32),
+           'int4v16': sq.Quantizer(4, 'v', 16), 'bf16': 'bf16'}
+
+
+def test_layout_bytes_match_documented_totals():
+    for cls, shape, totals in DOC_TOTALS:
+        for preset, nbytes in totals.items():
+            lay = cls(PRESETS[preset], m=8, buffer_bits=8, **shape)
+            assert lay.nbytes == nbytes, (cls.__name__, preset, lay.nbytes, nbytes)
+            assert lay.nbytes == sum(-(-x // 16) * 16 for x in lay.breakdown().values())
+    # the benchmark layouts: Qwen3.5-4B GDN, 32 value / 16 key heads, 128 x 128
+    want = {(8, 32): 608256, (8, 128): 583680, (4, 64): 329728, (4, 32): 346112}
+    for (bits, g), nbytes in want.items():
+        lay = SlotLayout(sq.Quantizer(bits, 'k', g), 32, 16, 128, 128, m=8, buffer_bits=8)
+        assert lay.nbytes == nbytes
+    lay = SlotLayout(sq.Quantizer(4, 'k', 64), 32, 16, 128, 128, m=8, buffer_bits=8)
+    b = lay.breakdown()                                            # the reference's tests/test_slots.py:210-216
+    assert b['S'] == 32 * 128 * 64 and b['SC'] == 32 * 128 * 2 * 2 and b['KB'] == 16 * 8 * 128 and b['UB'] == 32 * 8 * 128
+    assert KDASlotLayout(sq.Quantizer(4, 'k', 32), 32, 128, 128).nbytes == 509056
+    assert list(lay.fields) == ['GB', 'GCUR', 'NPTR', 'SC', 'KBS', 'UBS', 'S', 'KB', 'UB']
+
+
+@pytest.mark.parametrize('family', ['gdn', 'mamba2', 'kda'])
+def test_layout_read_write_match_oracle(family):
+    """Product layout == oracle layout, field by field; write / read on a CPU blob == the oracle's (torch code)."""
+    fmt = (4, 'k', 32)
+    if family == 'kda':
+        lay = KDASlotLayout(sq.Quantizer(*fmt), 2, 32, 32, m=4, buffer_bits=8)
+        hv, hk = 2, 2
+    else:
+        cls = SlotLayout if family == 'gdn' else Mamba2SlotLayout
+        lay = cls(sq.Quantizer(*fmt), 4, 2, 32, 32, m=4, buffer_bits=8)
+        hv, hk = 4, 2
+    table, nbytes = OSL.layout(family, fmt, hv, hk, 32, 32, 4, 8)
+    assert nbytes == lay.nbytes and table == lay.fields
+    torch.manual_seed(1)
+    blob = torch.randint(0, 256, (5, lay.nbytes), dtype=torch.uint8)
+    blob2 = blob.clone()
+    V, V2 = lay.views(blob), OSL.views(table, blob2)
+    idx = torch.tensor([3, 1])
+    S = torch.randn(2, hv, 32, 32)
+    lay.write(V, idx, S)
+    OSL.write(V2, idx, S, fmt, hv, 32, 32)
+    assert torch.equal(blob, blob2)
+    for W in (V, V2):
+        W['NPTR'][idx] = 2
+        W['GCUR'][idx] = -0.3
+        W['GB'][idx] = -0.1
+        W['KBS'][idx] = 0.01
+        W['UBS'][idx] = 0.02
+    got = lay.read(V, idx)
+    want = OSL.read(V2, idx, fmt, hv, hk, 32, 32, 4, per_channel=family == 'kda')
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-7)
+
+
+def test_library_exports_every_declared_symbol():
+    """libsqhip.so loads without a GPU and exports exactly the entry points include/statequant_hip.h declares."""
+    header = open(os.path.join(ROOT, 'include', 'statequant_hip.h')).read()
+    declared = set(re.findall(r'^\s*(?:int|const char\*)\s+(sq_\w+)\s*\(', header, flags=re.M))
+    assert declared == set(_hip.SYMBOLS), declared ^ set(_hip.SYMBOLS)
+    L = _hip.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.sq_abi_version() == 1
+    assert L.sq_strerror(0) == b'ok'
+    lay = _hip.SqLayout(bits=8, axis_k=1, group=128, buffer_bits=8, m=8, hv=32, hk=16, dk=128, dv=128)
+    assert L.sq_supported(0, ctypes.byref(lay)) == 1
+    lay.dv = 100
+    assert L.sq_supported(0, ctypes.byref(lay)) == 0
+    # argument errors are reported before anything touches a device
+    assert L.sq_gdn_step(None, None) == -1 and b'null args' in L.sq_last_error()
+    a = _hip.SqGdnArgs(lay=_hip.SqLayout(bits=5, axis_k=1, group=32, buffer_bits=8, m=8, hv=4, hk=2, dk=64, dv=64))
+    assert L.sq_gdn_step(ctypes.byref(a), None) == -2 and b'bits' in L.sq_last_error()
+
+
+def test_ctypes_structs_match_the_header():
+    """Field order of the ctypes mirrors == the C structs (a reordering would silently shift every pointer)."""
+    header = open(os.path.join(ROOT, 'include', 'statequant_hip.h')).read()
+    for cname, S in (('sq_state', _hip.SqState), ('sq_layout', _hip.SqLayout), ('sq_gdn_args', _hip.SqGdnArgs),
+                     ('sq_kda_args', _hip.SqKdaArgs), ('sq_mamba2_args', _hip.SqMamba2Args)):
+        body = re.search(r'typedef struct %s \{(.*?)\} %s;' % (cname, cname), header, flags=re.S).group(1)
+        body = re.sub(r'/\*.*?\*/', '', body, flags=re.S)
+        names = []
+        for decl in body.split(';'):
+            decl = decl.strip()
+            if decl:
+                for part in decl.split(','):
+                    names.append(re.findall(r'(\w+)\s*$', part.strip())[0])
+        assert names == [f[0] for f in S._fields_], (cname, names)
+
+
+def test_no_fallback_off_the_gpu():
+    """CPU tensors never reach a kernel, and nothing else computes the step instead."""
+    with pytest.raises(RuntimeError, match='GPU only'):
+        PackedGDNState(torch.zeros(8, 64, 64), sq.Quantizer(4, 'k', 32), hv=4, hk=2)
+    lay = SlotLayout(sq.Quantizer(4, 'v', 32), 4, 2, 128, 128)
+    with pytest.raises(NotImplementedError):
+        lay._layout_struct()

@@ -1,0 +1,231 @@
+"""Mamba2 / SSD HIP step (through the C ABI) against the CPU oracle and the reference's golden vectors.
+
+Mirrors the reference's tests/test_mamba2.py: decode vs the torch reference with per-step re-sync, slot step vs
+lockstep with padding rows, read() predicting the next output, dt options (bias, softplus, clamp, D).
+"""
+import pytest
+import torch
+
+from oracle import states as ST
+from statequant_amd.kernels import Mamba2SlotLayout, PackedMamba2State, mamba2_recurrence, unpack_vk
+from tests._util import Tally, buffer_entry, quantizer, unpack_nib
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def m2_token(gen, B, H, G, DK, DV, dtype=torch.float32):
+    """x ~ N(0,1); B, C ~ N(0,1) per group; raw dt ~ N(-2, 0.5) (softplus in the kernel)."""
+    r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
+    return r(B, H, DV).to(dtype), r(B, H) * 0.5 - 2, r(B, G, DK).to(dtype), r(B, G, DK).to(dtype)
+
+
+def params(gen, H):
+    A = -torch.exp(torch.rand(H, generator=gen) * 2)
+    return A, torch.randn(H, generator=gen), torch.randn(H, generator=gen) * 0.1
+
+
+def run_decode(fmt, m, bb, B=2, H=8, G=2, DK=128, DV=64, T=24, seed=1, dtype=torch.float32, use_D=True, use_bias=True,
+               softplus=True, limit=(0., float('inf'))):
+    gen = torch.Generator().manual_seed(seed)
+    S0 = torch.randn(B * H, DV, DK, generator=gen) * 0.5
+    A, D, dtb = params(gen, H)
+    D = D if use_D else None
+    dtb = dtb if use_bias else None
+    ker = PackedMamba2State(S0.to(DEV), quantizer(fmt), m=m, hv=H, hk=G, buffer_bits=bb, out_dtype=torch.float32)
+    ref = ST.Mamba2Oracle(S0, fmt, m=m, hv=H, hk=G, buffer_bits=bb, auto_fold=False)
+    assert torch.equal(ker.codes.cpu(), ref.codes) and torch.equal(ker.scales.cpu(), ref.scales)
+    tal = Tally()
+    dv = lambda t: None if t is None else t.to(DEV)        # noqa: E731
+    for t in range(T):
+        x, dt, Bm, C = m2_token(gen, B, H, G, DK, DV, dtype)
+        slot = ker.n
+        y = ker.step(dv(x), dv(dt), dv(Bm), dv(C), dv(A), dv(D), dv(dtb), softplus, limit).cpu().reshape(B * H, DV)
+        r = ref.step(x, dt, Bm, C, A, D, dtb, softplus, limit)
+        tal.out(y, r)
+        kb, ub = buffer_entry(ker.T, slot, bb == 8)
+        tal.entries(kb, ref.K[:, slot])
+        tal.entries(ub, ref.U[:, slot])
+        # the decay goes through softplus (log, exp): the device's and the host's libm may differ in the last bit,
+        # so compare to a few ulps and let the oracle continue from the kernel's value
+        gk = ker.GB[:, slot].cpu()
+        assert torch.allclose(gk, ref.G[:, slot], rtol=1e-6, atol=1e-7), t
+        ref.G[:, slot] = gk
+        ref.gcur = gk.clone()
+        ref.K[:, slot], ref.U[:, slot] = kb, ub
+        if ref.n == m:
+            ref.fold()
+        assert ker.n == ref.n
+        if ref.n == 0:
+            codes, scales = ker.codes.cpu(), ker.scales.cpu()
+            tal.fold(codes, scales, ref, fmt[0])
+            ref.adopt(codes, scales)
+        assert torch.equal(ker.NPTR.cpu(), torch.full((B, H), ref.n, dtype=torch.int32))
+    return tal
+
+
+def check(tal, tag, T, m):
+    print('\n' + tal.report(tag))
+    assert tal.folds == T // m
+    assert tal.worst_o < 2e-5, tal.worst_o
+    assert tal.buf_flips <= max(1, 1e-4 * tal.buf_entries), tal.buf_flips
+    assert tal.code_mism <= max(1, 1e-4 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)
+    assert tal.worst_raw < 0.2
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 8)])
+def test_decode_vs_oracle(fmt, m, bb):
+    T = 32 if m == 16 else 24
+    check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
+
+
+@pytest.mark.parametrize('DK,DV,H,G', [(128, 128, 4, 1), (64, 64, 4, 4)])
+def test_other_head_shapes(DK, DV, H, G):
+    check(run_decode((8, 'k', 64), 4, 8, B=3, H=H, G=G, DK=DK, DV=DV, T=12), f'mamba2 {DK}x{DV}', 12, 4)
+
+
+def test_dt_options_and_bf16_inputs():
+    """No D, no dt_bias, dt given pre-activated (dt_softplus=False), a dt clamp; bf16 x / B / C."""
+    check(run_decode((8, 'k', 128), 4, 8, T=8, use_D=False, use_bias=False), 'no D, no bias', 8, 4)
+    check(run_decode((8, 'k', 128), 4, 8, T=8, limit=(0.05, 0.2)), 'dt clamp', 8, 4)
+    check(run_decode((4, 'k', 64), 4, 8, T=8, dtype=torch.bfloat16), 'bf16 inputs', 8, 4)
+    # pre-activated dt: same result as activating in the kernel
+    gen = torch.Generator().manual_seed(2)
+    B, H, G, DK, DV = 2, 8, 2, 128, 64
+    S0 = torch.randn(B * H, DV, DK, generator=gen).to(DEV)
+    A, D, dtb = (t.to(DEV) for t in params(gen, H))
+    a = PackedMamba2State(S0, quantizer((8, 'k', 128)), m=4, hv=H, hk=G, out_dtype=torch.float32)
+    b = PackedMamba2State(S0, quantizer((8, 'k', 128)), m=4, hv=H, hk=G, out_dtype=torch.float32)
+    for t in range(6):
+        x, dt, Bm, C = (t_.to(DEV) for t_ in m2_token(gen, B, H, G, DK, DV))
+        act, _ = ST.mamba2_gate(dt.cpu(), A.cpu(), dtb.cpu(), True, None)
+        ya = a.step(x, dt, Bm, C, A, D, dtb, True, None).clone()
+        yb = b.step(x, act.to(DEV), Bm, C, A, D, None, False, None)
+        assert torch.allclose(ya, yb, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize('name', ['m2_int8.pt', 'm2_int4_bf16buf.pt'])
+def test_against_reference_golden_vectors(golden, name):
+    rec = golden(name)
+    B, H, G, DK, DV, m, bb = (rec[k] for k in ('B', 'HV', 'HK', 'DK', 'DV', 'm', 'buffer_bits'))
+    ker = PackedMamba2State(rec['S0'].to(DEV), quantizer(rec['fmt']), m=m, hv=H, hk=G, buffer_bits=bb,
+                            out_dtype=torch.float32)
+    assert torch.equal(ker.codes.cpu(), rec['codes0']) and torch.equal(ker.scales.cpu(), rec['scales0'])
+    from oracle.formats import round_buf_parts
+    A, D, dtb = (rec[k].to(DEV) for k in ('A', 'D', 'dt_bias'))
+    worst, flips, entries, mism, far, ncodes = 0.0, 0, 0, 0, 0, 0
+    for st in rec['steps']:
+        n = st['n']
+        assert ker.n == n
+        y = ker.step(st['x'].to(DEV), st['dt'].to(DEV), st['B'].to(DEV), st['C'].to(DEV), A, D, dtb, True,
+                     (0., float('inf'))).cpu().reshape(B * H, DV)
+        worst = max(worst, ((y - st['o']).abs().max() / st['o'].abs().max()).item())
+        kb, ub = buffer_entry(ker.T, n, bb == 8)
+        flips += (kb != st['K']).sum().item() + (ub != st['U']).sum().item()
+        entries += kb.numel() + ub.numel()
+        assert torch.allclose(ker.GB[:, n].cpu(), st['G'], rtol=1e-6, atol=1e-7)     # softplus: see run_decode
+        ker.GB[:, n].copy_(st['G'])
+        if 'codes' not in st:
+            ker.GCUR.copy_(st['G'])
+        if 'codes' in st:
+            d = (unpack_nib(ker.codes.cpu(), rec['fmt'][0]).int() - unpack_nib(st['codes'], rec['fmt'][0]).int()).abs()
+            mism += (d != 0).sum().item()
+            far += (d > 1).sum().item()
+            ncodes += d.numel()
+            ker.codes.copy_(st['codes'])
+            ker.scales.copy_(st['scales'])
+        elif bb == 8:
+            kc, ks = round_buf_parts(st['K'])
+            uc, us = round_buf_parts(st['U'])
+            ker.KB[:, n].copy_(kc), ker.KBS[:, n].copy_(ks), ker.UB[:, n].copy_(uc), ker.UBS[:, n].copy_(us)
+        else:
+            ker.KB[:, n].copy_(st['K'].to(torch.bfloat16)), ker.UB[:, n].copy_(st['U'].to(torch.bfloat16))
+    print(f'\n[{name}] max rel |y - y_ref| {worst:.2e}; buffer flips {flips}/{entries}; codes differing {mism}/{ncodes}')
+    assert worst < 2e-5 and flips <= max(1, 1e-4 * entries) and mism <= max(1, 1e-4 * ncodes) and far == 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+H, G, DK, DV = 8, 2, 128, 64
+
+
+def _setup(fmt, m, bb, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    lay = Mamba2SlotLayout(quantizer(fmt), H, G, DK, DV, m=m, buffer_bits=bb)
+    raw = torch.randint(0, 256, (8, lay.nbytes + 4096), dtype=torch.uint8, generator=gen).to(DEV)
+    blob = raw[:, 2048:2048 + lay.nbytes]
+    views = lay.views(blob)
+    slots = [5, 2, 7]
+    S0 = [torch.randn(H, DV, DK, generator=gen).to(DEV) * 0.5 for _ in slots]
+    refs = [PackedMamba2State(s, quantizer(fmt), m=m, hv=H, hk=G, buffer_bits=bb, out_dtype=torch.float32)
+            for s in S0]
+    lay.write(views, torch.tensor(slots, device=DEV), torch.stack(S0))
+    A, D, dtb = (t.to(DEV) for t in params(gen, H))
+    return lay, raw, blob, views, slots, refs, (A, D, dtb)
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (2, 16)])
+def test_slot_step_matches_lockstep_per_sequence(fmt, m, bb):
+    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup(fmt, m, bb)
+    outside = raw.clone()
+    sched = torch.Generator().manual_seed(1)
+    gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
+    steps = [0] * len(slots)
+    for t in range(20):
+        live = [i for i in torch.randperm(len(slots), generator=sched).tolist()
+                if torch.rand(1, generator=sched).item() < 0.7]
+        rows = live + ['pad0', 'padneg']
+        rows = [rows[j] for j in torch.randperm(len(rows), generator=sched).tolist()]
+        idx = torch.tensor([slots[r] if isinstance(r, int) else (0 if r == 'pad0' else -1) for r in rows],
+                           device=DEV, dtype=torch.int32)
+        Bn = len(rows)
+        x, dt = torch.zeros(Bn, H, DV, device=DEV), torch.zeros(Bn, H, device=DEV)
+        Bm, C = torch.zeros(Bn, G, DK, device=DEV), torch.zeros(Bn, G, DK, device=DEV)
+        want = {}
+        for b, r in enumerate(rows):
+            if not isinstance(r, int):
+                continue
+            tx, tdt, tB, tC = (z[0].to(DEV) for z in m2_token(gens[r], 1, H, G, DK, DV))
+            x[b], dt[b], Bm[b], C[b] = tx, tdt, tB, tC
+            want[b] = refs[r].step(tx, tdt, tB, tC, A, D, dtb, True, (0., float('inf'))).clone()
+            steps[r] += 1
+        out = torch.full((Bn, H, DV), 7., device=DEV)
+        lay.step(views, idx, x, dt, Bm, C, out, A, D, dtb)
+        for b, r in enumerate(rows):
+            if isinstance(r, int):
+                assert torch.equal(out[b], want[b].view(H, DV)), (t, b)
+                assert views['NPTR'][slots[r], :H].tolist() == [steps[r] % m] * H
+                assert torch.equal(views['S'][slots[r]], refs[r].codes.view(H, *refs[r].codes.shape[1:]))
+                assert torch.equal(views['SC'][slots[r]], refs[r].scales.view(H, *refs[r].scales.shape[1:]))
+            else:
+                assert torch.equal(out[b], torch.zeros_like(out[b]))
+    keep = torch.ones_like(raw, dtype=torch.bool)
+    for s in slots:
+        keep[s, 2048:2048 + lay.nbytes] = False
+    assert torch.equal(raw[keep], outside[keep])
+
+
+def test_read_is_the_state_the_next_step_reads():
+    """read() + one textbook fp32 Mamba2 step == the kernel's next output (reference: tests/test_mamba2.py:273-300)."""
+    m = 8
+    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup((8, 'k', 32), m, 8)
+    gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
+    idx = torch.tensor(slots, device=DEV, dtype=torch.int32)
+    for t in range(13):
+        toks = [m2_token(gn, 1, H, G, DK, DV) for gn in gens]
+        x, dt, Bm, C = (torch.cat(z).to(DEV) for z in zip(*toks))
+        out = torch.empty(len(slots), H, DV, device=DEV)
+        if t == 12:
+            S = lay.read(views, idx)
+            y_pred = mamba2_recurrence(S, x, dt, Bm, C, A, D, dtb, True, None)
+        lay.step(views, idx, x, dt, Bm, C, out, A, D, dtb)
+    rel = ((out - y_pred).norm() / y_pred.norm()).item()
+    assert rel < 1e-5, rel
+    # write(read()) == pack(unpack())
+    S = lay.read(views, idx)
+    lay.write(views, idx, S)
+    got = lay.read(views, idx)
+    from statequant_amd.kernels import pack_vk
+    c, s = pack_vk(S.reshape(-1, DV, DK), quantizer((8, 'k', 32)))
+    assert torch.equal(got, unpack_vk(c, s, quantizer((8, 'k', 32)), DK).view_as(S))
