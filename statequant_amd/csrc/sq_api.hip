@@ -150,12 +150,17 @@ int sq_gdn_step(const sq_gdn_args* a, void* stream) {
     p.v = a->v; p.s_v = a->s_v; p.v_dt = a->v_dtype;
     p.qk_per_key_head = a->qk_per_key_head != 0;
     p.gate = a->gate != 0;
-    p.g = a->g; p.s_g = a->s_g; p.g_dt = a->g_dtype;
-    p.beta = a->beta; p.s_beta = a->s_beta; p.beta_dt = a->beta_dtype;
-    p.a = a->a; p.s_a = a->s_a; p.a_dt = a->a_dtype;
-    p.bt = a->b; p.s_bt = a->s_b; p.bt_dt = a->b_dtype;
-    p.A_log = a->A_log; p.A_log_dt = a->A_log_dtype;
-    p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    if (p.gate) {
+        p.a = a->a; p.s_a = a->s_a; p.a_dt = a->a_dtype;
+        p.bt = a->b; p.s_bt = a->s_b; p.bt_dt = a->b_dtype;
+        p.A_log = a->A_log; p.A_log_dt = a->A_log_dtype;
+        p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    } else {                  // the kernel reads the same four operands either way: g, beta, and g twice as dummies
+        p.a = a->g; p.s_a = a->s_g; p.a_dt = a->g_dtype;
+        p.bt = a->beta; p.s_bt = a->s_beta; p.bt_dt = a->beta_dtype;
+        p.A_log = a->g; p.A_log_dt = a->g_dtype;
+        p.dt_bias = a->g; p.dt_bias_dt = a->g_dtype;
+    }
     p.out = a->out; p.out_dt = a->out_dtype;
     p.scale = a->scale;
     return finish(sq::dispatch_gdn(p, static_cast<hipStream_t>(stream), true), who, a->lay);
@@ -170,6 +175,8 @@ int sq_kda_step(const sq_kda_args* a, void* stream) {
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;
     SQ_TRY(check_state(a->st, a->lay, who, &p.st));
+    if (!aligned(a->st.GB, 16) || (a->st.sGB % 4))
+        return fail(SQ_E_ARG, "%s: GB must be 16-byte aligned (base and per-sequence stride)", who);
     if (!a->q || !a->k || !a->v || !a->g || !a->beta || !a->out) return fail(SQ_E_ARG, "%s: null input / output", who);
     if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->g_dtype) ||
         !dtype_ok(a->beta_dtype) || !dtype_ok(a->out_dtype))
@@ -206,8 +213,12 @@ int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
     p.B = a->B; p.s_B = a->s_B; p.B_dt = a->B_dtype;
     p.C = a->C; p.s_C = a->s_C; p.C_dt = a->C_dtype;
     p.A = a->A; p.A_dt = a->A_dtype;
-    p.D = a->D; p.D_dt = a->D_dtype;
-    p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    p.has_D = a->D != nullptr;
+    p.has_dt_bias = a->dt_bias != nullptr;
+    p.D = p.has_D ? a->D : a->A;
+    p.D_dt = p.has_D ? a->D_dtype : a->A_dtype;
+    p.dt_bias = p.has_dt_bias ? a->dt_bias : a->A;
+    p.dt_bias_dt = p.has_dt_bias ? a->dt_bias_dtype : a->A_dtype;
     p.dt_softplus = a->dt_softplus != 0;
     p.dt_clamp = a->dt_clamp != 0;
     p.dt_min = a->dt_min; p.dt_max = a->dt_max;

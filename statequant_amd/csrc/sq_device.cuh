@@ -40,12 +40,25 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {      // round to near
 __device__ __forceinline__ float f16_to_f32(uint16_t h) { return float(__builtin_bit_cast(_Float16, h)); }
 __device__ __forceinline__ uint16_t f32_to_f16(float f) { return __builtin_bit_cast(uint16_t, _Float16(f)); }
 
-// A scalar of a float tensor of run-time dtype (inputs come as fp32, bf16 or fp16).
-__device__ __forceinline__ float load_f(const void* p, int dt, int64_t i) {
-    if (dt == F32) return reinterpret_cast<const float*>(p)[i];
-    const uint16_t h = reinterpret_cast<const uint16_t*>(p)[i];
-    return dt == BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+// A scalar of a float tensor of run-time dtype (inputs come as fp32, bf16 or fp16), in two steps so that a kernel can
+// issue all its loads first and convert later: a conversion right behind a load, inside the dtype branch, makes
+// the compiler wait for memory in every branch and serializes the loads.
+__device__ __forceinline__ uint32_t load_raw(const void* p, int dt, int64_t i) {
+    if (dt == F32) return reinterpret_cast<const uint32_t*>(p)[i];
+    return reinterpret_cast<const uint16_t*>(p)[i];
 }
+// The same for a wave-uniform address (a per-head scalar).  The offset is laundered through a vector register so
+// that the load stays a vector load: as a scalar load its result would have to be moved into a VGPR right away, and
+// the wait for that move also waits for every vector load issued before it.
+__device__ __forceinline__ uint32_t load_raw_uniform(const void* p, int dt, int64_t i) {
+    int32_t z = 0;
+    asm volatile("" : "+v"(z));
+    return load_raw(p, dt, i + z);
+}
+__device__ __forceinline__ float raw_to_f(uint32_t r, int dt) {
+    return dt == F32 ? as_f32(r) : dt == BF16 ? bf16_to_f32(uint16_t(r)) : f16_to_f32(uint16_t(r));
+}
+__device__ __forceinline__ float load_f(const void* p, int dt, int64_t i) { return raw_to_f(load_raw(p, dt, i), dt); }
 __device__ __forceinline__ void store_f(void* p, int dt, int64_t i, float v) {
     if (dt == F32) reinterpret_cast<float*>(p)[i] = v;
     else reinterpret_cast<uint16_t*>(p)[i] = dt == BF16 ? f32_to_bf16(v) : f32_to_f16(v);

@@ -10,6 +10,8 @@
 //   fold     buffer full: S = a_m S0 + sum_i (a_m/a_i) u_i k_i^T from the codes still in registers (no second read
 //            of the state), re-quantized in place
 //   advance  running decay and this head's copy of the counter
+// Every load the step needs is issued before the first use of any of them (small operands first, then the state
+// tile), so a wavefront pays one memory round trip after the slot index, not one per operand.
 #pragma once
 #include "sq_tile.cuh"
 #include "sq_params.h"
@@ -32,6 +34,7 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
     const int hk = h / gqa;
     const int m = p.m;
     constexpr int DK = T::DK, DV = T::DV;
+    constexpr int KT = KeyBuf<T>::KT;
 
     const int64_t seq = p.idx ? int64_t(p.idx[b]) : int64_t(b);
     const int64_t obase = (int64_t(b) * p.hv + h) * DV;
@@ -40,58 +43,76 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
         return;
     }
 
-    // ---- the state tile and everything else that only depends on the slot: issue the loads first ----
+    // ---- addresses ----
     uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
     uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
-    RawRow<T::BITS> raw[T::RPL];
-    load_tile<T>(Sh, l, raw);
-    float sc[T::RPL];
-    load_scales<T>(SCh, l, sc);
-
     constexpr int BE = T::QBUF ? 1 : 2;                           // bytes per buffer element
-    uint8_t* KBh = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * BE;
-    uint8_t* UBh = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * BE;
-    uint16_t* KBSh = p.st.KBS + seq * p.st.sKBS + int64_t(hk) * m;
-    uint16_t* UBSh = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
+    BufAddr<T> buf;
+    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * BE;
+    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * BE;
+    buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(hk) * m;
+    buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
     float* gcp = p.st.GCUR + seq * p.st.sGC + h;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
+    const int jown = own_first<T>(l);
+    const int hq = p.qk_per_key_head ? hk : h;
+    const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
 
+    // ---- issue every load: counters, buffer, inputs, then the state tile ----
     const int n = *np & (m - 1);
     const float gcur = *gcp;
-    const bool full = n == m - 1;
-
-    // per-slot scalars: lane i holds slot i's
-    float ubs_l = 1.0f;
-    if (T::QBUF && l.lane < m) ubs_l = f16_to_f32(UBSh[l.lane]);
-
-    // delta values of the rows this lane will own, all slots (dead slots are discarded below, never multiplied)
-    const int jown = own_first<T>(l);
-    float ub[T::MMAX][T::NOWN];
+    const int lm = l.lane < m ? l.lane : m - 1;
+    uint16_t ubs_raw = 0;
+    if constexpr (T::QBUF) ubs_raw = buf.UBS[lm];
+    const float gb_lane = GBh[lm];                                // lane i: slot i's cumulative decay
+    int32_t ub[T::MMAX][T::NOWN];
+    load_ub<T>(buf.UB, m, l, jown, ub);
+    KeyBuf<T> kbuf;
+    load_keybuf<T>(buf, m, l, kbuf);
+    float gb[KT];
 #pragma unroll
-    for (int i = 0; i < T::MMAX; ++i)
-#pragma unroll
-        for (int t = 0; t < T::NOWN; ++t) {
-            const int r = row_of<T>(l, jown + t);
-            float x = 0.0f;
-            if (i < m && jown + t < T::RPL) {
-                if constexpr (T::QBUF) x = float(reinterpret_cast<const int8_t*>(UBh)[i * DV + r]);
-                else x = bf16_to_f32(reinterpret_cast<const uint16_t*>(UBh)[i * DV + r]);
-            }
-            ub[i][t] = x;
-        }
-
-    // ---- prep: q, k (fla's l2 normalisation), gates ----
-    const int hq = p.qk_per_key_head ? hk : h;
-    float qe[T::NE], ke[T::NE], kxe[T::NE];
-    float ssq = 0.0f, ssk = 0.0f;
+    for (int t = 0; t < KT; ++t) { const int i = l.rg + T::RG * t; gb[t] = GBh[i < m ? i : m - 1]; }
+    uint32_t qr[T::NE], kr_[T::NE], kxr[T::NE];
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
-        const int e = l.lane + WAVE * t;
-        qe[t] = e < DK ? load_f(p.q, p.q_dt, int64_t(b) * p.s_q + int64_t(hq) * DK + e) : 0.0f;
-        ke[t] = e < DK ? load_f(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hq) * DK + e) : 0.0f;
+        int e = l.lane + WAVE * t;
+        e = e < DK ? e : DK - 1;
+        qr[t] = load_raw(p.q, p.q_dt, int64_t(b) * p.s_q + int64_t(hq) * DK + e);
+        kr_[t] = load_raw(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hq) * DK + e);
+        kxr[t] = own_key ? load_raw(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hk * gqa) * DK + e) : 0u;
+    }
+    // gate: a, b [rows, hv], A_log, dt_bias [hv];  no gate: the same four slots carry g, beta and two dummies
+    // (the C ABI points them at g), so the loads need no branch
+    const uint32_t g0 = load_raw_uniform(p.a, p.a_dt, int64_t(b) * p.s_a + h);
+    const uint32_t g1 = load_raw_uniform(p.bt, p.bt_dt, int64_t(b) * p.s_bt + h);
+    const uint32_t g2 = load_raw_uniform(p.A_log, p.A_log_dt, h);
+    const uint32_t g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);
+    uint32_t vr[T::NOWN];
+#pragma unroll
+    for (int t = 0; t < T::NOWN; ++t) {
+        int r = row_of<T>(l, jown + t);
+        r = r < DV ? r : DV - 1;
+        vr[t] = load_raw(p.v, p.v_dt, int64_t(b) * p.s_v + int64_t(h) * DV + r);
+    }
+    RawRow<T::BITS> raw[T::RPL];
+    load_tile<T>(Sh, l, raw);
+    uint16_t scr[T::RPL];
+    load_scales<T>(SCh, l, scr);
+
+    // ---- prep: q, k (fla's l2 normalisation), gates ----
+    const bool full = n == m - 1;
+    float qe[T::NE], ke[T::NE], kxe[T::NE];
+    float ssq = 0.0f, ssk = 0.0f, ssx = 0.0f;
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) {
+        const bool in = l.lane + WAVE * t < DK;
+        qe[t] = in ? raw_to_f(qr[t], p.q_dt) : 0.0f;
+        ke[t] = in ? raw_to_f(kr_[t], p.k_dt) : 0.0f;
+        kxe[t] = in ? raw_to_f(kxr[t], p.k_dt) : 0.0f;
         ssq = __builtin_fmaf(qe[t], qe[t], ssq);
         ssk = __builtin_fmaf(ke[t], ke[t], ssk);
+        ssx = __builtin_fmaf(kxe[t], kxe[t], ssx);
     }
     const float nq = sqrtf(wave_sum(ssq) + 1e-6f);
     const float nk = sqrtf(wave_sum(ssk) + 1e-6f);
@@ -100,97 +121,46 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
     for (int t = 0; t < T::NE; ++t) {
         qe[t] = qe[t] / nq * p.scale;
         ke[t] = ke[t] / nk;
-        kxe[t] = ke[t];
         kqp = __builtin_fmaf(ke[t], qe[t], kqp);
         const int e = l.lane + WAVE * t;
         if (e < T::LPRP * CPL) { lds_q[kpos<T>(e)] = qe[t]; lds_kn[kpos<T>(e)] = ke[t]; }
     }
     const float kq = wave_sum(kqp);
-    if (!p.qk_per_key_head && gqa > 1) {                          // the buffered key is the group's first head's
-        float ss = 0.0f;
-#pragma unroll
-        for (int t = 0; t < T::NE; ++t) {
-            const int e = l.lane + WAVE * t;
-            kxe[t] = e < DK ? load_f(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hk * gqa) * DK + e) : 0.0f;
-            ss = __builtin_fmaf(kxe[t], kxe[t], ss);
-        }
-        const float nx = sqrtf(wave_sum(ss) + 1e-6f);
+    if (own_key) {
+        const float nx = sqrtf(wave_sum(ssx) + 1e-6f);
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) kxe[t] = kxe[t] / nx;
+    } else {
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) kxe[t] = ke[t];
     }
     float g, beta;
     if (p.gate) {
-        const float x = load_f(p.a, p.a_dt, int64_t(b) * p.s_a + h) + load_f(p.dt_bias, p.dt_bias_dt, h);
+        const float x = raw_to_f(g0, p.a_dt) + raw_to_f(g3, p.dt_bias_dt);
         const float sp = x <= 20.0f ? logf(1.0f + expf(x)) : x;
-        g = -expf(load_f(p.A_log, p.A_log_dt, h)) * sp;
-        const float bx = load_f(p.bt, p.bt_dt, int64_t(b) * p.s_bt + h);
-        beta = 1.0f / (1.0f + expf(-bx));
+        g = -expf(raw_to_f(g2, p.A_log_dt)) * sp;
+        beta = 1.0f / (1.0f + expf(-raw_to_f(g1, p.bt_dt)));
     } else {
-        g = load_f(p.g, p.g_dt, int64_t(b) * p.s_g + h);
-        beta = load_f(p.beta, p.beta_dt, int64_t(b) * p.s_beta + h);
+        g = raw_to_f(g0, p.a_dt);
+        beta = raw_to_f(g1, p.bt_dt);
     }
     const float alpha = expf(gcur);
     const float a = expf(g);
     const float gnew = gcur + g;
+    const float ubs_l = T::QBUF ? f16_to_f32(ubs_raw) : 1.0f;
     __syncthreads();
     float x[2][CPL];
     lds_piece<T>(lds_q, l.cg, x[0]);
     lds_piece<T>(lds_kn, l.cg, x[1]);
 
-    // ---- buffer coefficients: the key buffer as a small tile, slot = row group (+ RG per pass) ----
-    float cq[T::MMAX], ck[T::MMAX];
-    {
-        constexpr int KT = (T::MMAX + T::RG - 1) / T::RG;
-        float cq_l[KT], ck_l[KT];
-#pragma unroll
-        for (int t = 0; t < KT; ++t) {
-            const int i = l.rg + T::RG * t;
-            float kb[CPL];
-#pragma unroll
-            for (int c = 0; c < CPL; ++c) kb[c] = 0.0f;
-            float dec = 0.0f;
-            if (i < m) {
-                if (l.cg < T::LPR) {
-                    if constexpr (T::QBUF) {
-                        RawRow<8> rr = load_row<8>(KBh + i * DK + l.cg * CPL);
-                        decode_row<8>(rr, kb);
-                        const float ksc = f16_to_f32(KBSh[i]);
-#pragma unroll
-                        for (int c = 0; c < CPL; ++c) kb[c] = kb[c] * ksc;
-                    } else {
-                        const uint16_t* kp = reinterpret_cast<const uint16_t*>(KBh) + i * DK + l.cg * CPL;
-#pragma unroll
-                        for (int c = 0; c < CPL; ++c) kb[c] = bf16_to_f32(kp[c]);
-                    }
-                }
-                dec = expf(gcur - GBh[i]);
-            }
-            float pq = kb[0] * x[0][0], pk = kb[0] * x[1][0];
-#pragma unroll
-            for (int c = 1; c < CPL; ++c) {
-                pq = __builtin_fmaf(kb[c], x[0][c], pq);
-                pk = __builtin_fmaf(kb[c], x[1][c], pk);
-            }
-            pq = block_sum<T::LPRP>(pq);
-            pk = block_sum<T::LPRP>(pk);
-            const bool alive = i < n;
-            cq_l[t] = alive ? dec * pq : 0.0f;
-            ck_l[t] = alive ? dec * pk : 0.0f;
-            if (full && i < m - 1) {                               // the fold wants the dequantized keys
-                float4* d4 = reinterpret_cast<float4*>(lds_k + i * T::KROW + l.cg * T::KPAD);
-#pragma unroll
-                for (int c = 0; c < CPL / 4; ++c)
-                    d4[c] = make_float4(kb[4 * c], kb[4 * c + 1], kb[4 * c + 2], kb[4 * c + 3]);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < T::MMAX; ++i) {
-            cq[i] = lane_bcast(cq_l[i / T::RG], (i % T::RG) * T::LPRP);
-            ck[i] = lane_bcast(ck_l[i / T::RG], (i % T::RG) * T::LPRP);
-        }
-    }
+    // ---- buffer coefficients ----
+    float c[2][T::MMAX];
+    buffer_coefs<T, 2>(kbuf, gb, gcur, n, m, full, x, l, lds_k, c);
 
     // ---- state pass ----
+    mask_tile<T>(l, raw);
+    float sc[T::RPL];
+    scale_values<T>(scr, l, sc);
     float part[2][T::RPLP];
     tile_dots<T, 2>(raw, x, part);
     float own[2][T::NOWN];
@@ -206,13 +176,13 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
         float sk = alpha * own[1][t];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub[i][t];
+            float uv = ub_value<T>(ub[i][t]);
             if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
-            uv = i < n ? uv : 0.0f;
-            sq = __builtin_fmaf(uv, cq[i], sq);
-            sk = __builtin_fmaf(uv, ck[i], sk);
+            uv = i < n ? uv : 0.0f;                               // dead slots may hold anything: discard
+            sq = __builtin_fmaf(uv, c[0][i], sq);
+            sk = __builtin_fmaf(uv, c[1][i], sk);
         }
-        const float vt = valid ? load_f(p.v, p.v_dt, int64_t(b) * p.s_v + int64_t(h) * DV + r) : 0.0f;
+        const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * __builtin_fmaf(-a, sk, vt);
         const float o = __builtin_fmaf(kq, u[t], a * sq);
         if (valid) store_f(p.out, p.out_dt, obase + r, o);
@@ -222,76 +192,28 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
 
     // ---- append ----
     float us = 1.0f, ks = 1.0f;
-    float ur[T::NOWN];                                             // the delta value as stored (dequantized)
     if constexpr (T::QBUF) {
         us = fp16_scale(wave_max(amax), 127.0f);
         float kmax = 0.0f;
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) kmax = fmaxf(kmax, fabsf(kxe[t]));
         ks = fp16_scale(wave_max(kmax), 127.0f);
-        if (l.lane == 0) UBSh[n] = f32_to_f16(us);
     }
-#pragma unroll
-    for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
-        if constexpr (T::QBUF) {
-            const float c = round_buf(u[t], us);
-            ur[t] = c * us;
-            if (jown + t < T::RPL) reinterpret_cast<int8_t*>(UBh)[n * DV + r] = int8_t(int(c));
-        } else {
-            const uint16_t hb = f32_to_bf16(u[t]);
-            ur[t] = bf16_to_f32(hb);
-            if (jown + t < T::RPL) reinterpret_cast<uint16_t*>(UBh)[n * DV + r] = hb;
-        }
-    }
-    float kr[T::NE];                                               // the key as stored (dequantized)
-    const bool first = (h % gqa) == 0;
-#pragma unroll
-    for (int t = 0; t < T::NE; ++t) {
-        const int e = l.lane + WAVE * t;
-        if constexpr (T::QBUF) {
-            const float c = round_buf(kxe[t], ks);
-            kr[t] = c * ks;
-            if (first && e < DK) reinterpret_cast<int8_t*>(KBh)[n * DK + e] = int8_t(int(c));
-        } else {
-            const uint16_t hb = f32_to_bf16(kxe[t]);
-            kr[t] = bf16_to_f32(hb);
-            if (first && e < DK) reinterpret_cast<uint16_t*>(KBh)[n * DK + e] = hb;
-        }
-    }
-    if (l.lane == 0) {
-        GBh[n] = gnew;
-        if (T::QBUF && first) KBSh[n] = f32_to_f16(ks);
-    }
+    float ur[T::NOWN], kr[T::NE];                                 // value / key as stored, dequantized
+    append_values<T>(u, us, buf, n, l, jown, ur);
+    append_key<T>(kxe, ks, buf, n, (h % gqa) == 0, l, kr);
+    if (l.lane == 0) GBh[n] = gnew;
 
     // ---- fold ----
     if (full) {
-        // decay ratio a_m / a_i per slot (lane i: slot i; the current token's is exp(0) = 1)
-        float decf = 1.0f;
-        if (l.lane < m - 1) decf = expf(gnew - GBh[l.lane]);
-#pragma unroll
-        for (int t = 0; t < T::NOWN; ++t) {
-            const int r = row_of<T>(l, jown + t);
-#pragma unroll
-            for (int i = 0; i < T::MMAX; ++i) {
-                if (i < m) {
-                    float uv = ub[i][t];
-                    if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
-                    if (i == m - 1) uv = ur[t];
-                    lds_u[i * T::UROW + r] = lane_bcast(decf, i) * uv;
-                }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < T::NE; ++t) {
-            const int e = l.lane + WAVE * t;
-            if (e < T::LPRP * CPL) lds_k[(m - 1) * T::KROW + kpos<T>(e)] = e < DK ? kr[t] : 0.0f;
-        }
+        const float decf = l.lane < m - 1 ? expf(gnew - gb_lane) : 1.0f;     // a_m / a_i; the current token's: 1
+        stage_values<T>(ub, ubs_l, decf, ur, m, l, jown, lds_u);
+        stage_key<T>(kr, m - 1, l, lds_k);
         __syncthreads();
         const float alphan = expf(gnew);
         float colmul[CPL];
 #pragma unroll
-        for (int c = 0; c < CPL; ++c) colmul[c] = alphan;
+        for (int k = 0; k < CPL; ++k) colmul[k] = alphan;
         fold_tile<T>(raw, sc, colmul, lds_k, lds_u, m, Sh, SCh, l);
     }
 

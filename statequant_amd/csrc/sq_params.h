@@ -30,9 +30,7 @@ struct GdnParams : LayoutKey {
     int64_t s_q, s_k, s_v;
     int q_dt, k_dt, v_dt;
     int qk_per_key_head, gate;
-    const void *g, *beta;
-    int64_t s_g, s_beta;
-    int g_dt, beta_dt;
+    // gate: a, b, A_log, dt_bias;  no gate: a = g, bt = beta, A_log = dt_bias = g (never used, always readable)
     const void *a, *bt, *A_log, *dt_bias;
     int64_t s_a, s_bt;
     int a_dt, bt_dt, A_log_dt, dt_bias_dt;
@@ -61,7 +59,7 @@ struct Mamba2Params : LayoutKey {
     const void *x, *dt, *B, *C, *A, *D, *dt_bias;
     int64_t s_x, s_dt, s_B, s_C;
     int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
-    int dt_softplus, dt_clamp;
+    int dt_softplus, dt_clamp, has_D, has_dt_bias;      // absent D / dt_bias: pointers alias A (readable, unused)
     float dt_min, dt_max;
     void* out;
     int64_t s_out;

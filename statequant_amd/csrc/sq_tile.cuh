@@ -70,25 +70,46 @@ __device__ __forceinline__ int own_first(const LaneId& l) {
     return off;
 }
 
-// The only read of the stored state: a lane's piece of each of its rows, issued back to back.
+// The only read of the stored state: a lane's piece of each of its rows, issued back to back.  Idle lanes (past
+// d_k) load a live lane's piece instead of branching around the load, and zero it afterwards.
 template <class T>
 __device__ __forceinline__ void load_tile(const uint8_t* head, const LaneId& l, RawRow<T::BITS> (&raw)[T::RPL]) {
-    const bool live = l.cg < T::LPR;
+    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 #pragma unroll
-    for (int j = 0; j < T::RPL; ++j) {
-        if (live) raw[j] = load_row<T::BITS>(head + size_t(row_of<T>(l, j)) * T::ROW_BYTES + l.cg * T::LANE_BYTES);
-        else raw[j] = zero_row<T::BITS>();
+    for (int j = 0; j < T::RPL; ++j)
+        raw[j] = load_row<T::BITS>(head + size_t(row_of<T>(l, j)) * T::ROW_BYTES + cc * T::LANE_BYTES);
+}
+template <class T>
+__device__ __forceinline__ void mask_tile(const LaneId& l, RawRow<T::BITS> (&raw)[T::RPL]) {
+    if constexpr (T::LPR < T::LPRP) {
+        const bool live = l.cg < T::LPR;
+        const RawRow<T::BITS> z = zero_row<T::BITS>();
+#pragma unroll
+        for (int j = 0; j < T::RPL; ++j) {
+            raw[j].v.x = live ? raw[j].v.x : z.v.x;
+            raw[j].v.y = live ? raw[j].v.y : z.v.y;
+            if constexpr (T::BITS == 8) {
+                raw[j].v.z = live ? raw[j].v.z : z.v.z;
+                raw[j].v.w = live ? raw[j].v.w : z.v.w;
+            }
+        }
     }
 }
 
-// The fp16 scale of (row j, this lane's key group) for every row of the lane, as fp32 (0 for idle lanes).
+// The raw fp16 scale of (row j, this lane's key group) for every row of the lane; scale_value() turns it into fp32
+// (0 for lanes whose group lies past d_k).
 template <class T>
-__device__ __forceinline__ void load_scales(const uint16_t* sc_head, const LaneId& l, float (&sc)[T::RPL]) {
-    const int gi = (l.cg * CPL) / T::GROUP;
-    const bool ok = gi < T::NG;
+__device__ __forceinline__ void load_scales(const uint16_t* sc_head, const LaneId& l, uint16_t (&sc)[T::RPL]) {
+    int gi = (l.cg * CPL) / T::GROUP;
+    gi = gi < T::NG ? gi : T::NG - 1;
 #pragma unroll
-    for (int j = 0; j < T::RPL; ++j)
-        sc[j] = ok ? f16_to_f32(sc_head[size_t(row_of<T>(l, j)) * T::NG + gi]) : 0.0f;
+    for (int j = 0; j < T::RPL; ++j) sc[j] = sc_head[size_t(row_of<T>(l, j)) * T::NG + gi];
+}
+template <class T>
+__device__ __forceinline__ void scale_values(const uint16_t (&raw)[T::RPL], const LaneId& l, float (&sc)[T::RPL]) {
+    const bool ok = (l.cg * CPL) / T::GROUP < T::NG;
+#pragma unroll
+    for (int j = 0; j < T::RPL; ++j) sc[j] = ok ? f16_to_f32(raw[j]) : 0.0f;
 }
 
 // A small register vector passed by value, so that selects between its elements stay selects (an array passed by
@@ -167,6 +188,208 @@ __device__ __forceinline__ void lds_piece(const float* vec, int cg, float (&x)[C
     for (int t = 0; t < CPL / 4; ++t) {
         const float4 f = p4[t];
         x[4 * t] = f.x; x[4 * t + 1] = f.y; x[4 * t + 2] = f.z; x[4 * t + 3] = f.w;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// the decode buffer.  All loads below are unconditional (indices clamped into the live range) so that they can be
+// issued back to back ahead of the state tile; dead slots and idle lanes are masked after the fact with selects.
+// ---------------------------------------------------------------------------------------------------------------
+template <class T>
+struct BufAddr {                       // one (sequence, head)'s buffer fields
+    uint8_t* KB;                       // [m][DK] int8 or bf16, of the head's KEY head
+    uint8_t* UB;                       // [m][DV] int8 or bf16
+    uint16_t* KBS;                     // [m] fp16 (int8 buffer)
+    uint16_t* UBS;                     // [m] fp16 (int8 buffer)
+};
+
+// Raw delta values of the rows this lane owns, every slot: ub[i][t] = UB[min(i, m-1)][row t].
+template <class T>
+__device__ __forceinline__ void load_ub(const uint8_t* UB, int m, const LaneId& l, int jown,
+                                        int32_t (&ub)[T::MMAX][T::NOWN]) {
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) {
+        const int ic = i < m ? i : m - 1;
+#pragma unroll
+        for (int t = 0; t < T::NOWN; ++t) {
+            int r = row_of<T>(l, jown + t);
+            r = r < T::DV ? r : T::DV - 1;
+            if constexpr (T::QBUF) ub[i][t] = reinterpret_cast<const int8_t*>(UB)[ic * T::DV + r];
+            else ub[i][t] = reinterpret_cast<const uint16_t*>(UB)[ic * T::DV + r];
+        }
+    }
+}
+template <class T>
+__device__ __forceinline__ float ub_value(int32_t raw) {
+    if constexpr (T::QBUF) return float(raw);
+    else return bf16_to_f32(uint16_t(raw));
+}
+
+// A lane's 16-column piece of one buffered key, raw.
+template <bool QBUF> struct KPiece;
+template <> struct KPiece<true> { uint4 a; };
+template <> struct KPiece<false> { uint4 a, b; };
+
+template <class T>
+__device__ __forceinline__ KPiece<T::QBUF> load_kpiece(const uint8_t* KB, int slot, int m, const LaneId& l) {
+    const int ic = slot < m ? slot : m - 1;
+    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
+    KPiece<T::QBUF> k;
+    if constexpr (T::QBUF) {
+        k.a = *reinterpret_cast<const uint4*>(KB + ic * T::DK + cc * CPL);
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(KB + (ic * T::DK + cc * CPL) * 2);
+        k.a = p[0];
+        k.b = p[1];
+    }
+    return k;
+}
+// -> fp32, times the slot's scale for an int8 buffer; zeros in idle lanes.
+template <class T>
+__device__ __forceinline__ void decode_kpiece(const KPiece<T::QBUF>& k, float scale, const LaneId& l,
+                                              float (&kb)[CPL]) {
+    if constexpr (T::QBUF) {
+        RawRow<8> r;
+        r.v = k.a;
+        decode_row<8>(r, kb);
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) kb[c] = kb[c] * scale;
+    } else {
+        const uint32_t w[8] = {k.a.x, k.a.y, k.a.z, k.a.w, k.b.x, k.b.y, k.b.z, k.b.w};
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            kb[2 * c] = as_f32(w[c] << 16);
+            kb[2 * c + 1] = as_f32(w[c] & 0xFFFF0000u);
+        }
+    }
+    if (l.cg >= T::LPR) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) kb[c] = 0.0f;
+    }
+}
+template <class T>
+__device__ __forceinline__ void stage_kpiece(float* lds_k, int slot, const LaneId& l, const float (&kb)[CPL]) {
+    float4* d4 = reinterpret_cast<float4*>(lds_k + slot * T::KROW + l.cg * T::KPAD);
+#pragma unroll
+    for (int c = 0; c < CPL / 4; ++c) d4[c] = make_float4(kb[4 * c], kb[4 * c + 1], kb[4 * c + 2], kb[4 * c + 3]);
+}
+
+// Passes over the key buffer seen as a small tile: slot = row group + RG x pass.
+template <class T>
+struct KeyBuf {
+    static constexpr int KT = (T::MMAX + T::RG - 1) / T::RG;
+    KPiece<T::QBUF> piece[KT];
+    uint16_t kbs[KT];                  // raw fp16 scale of the lane's slot (int8 buffer)
+};
+template <class T>
+__device__ __forceinline__ void load_keybuf(const BufAddr<T>& a, int m, const LaneId& l, KeyBuf<T>& kb) {
+#pragma unroll
+    for (int t = 0; t < KeyBuf<T>::KT; ++t) {
+        const int i = l.rg + T::RG * t;
+        kb.piece[t] = load_kpiece<T>(a.KB, i, m, l);
+        if constexpr (T::QBUF) kb.kbs[t] = a.KBS[i < m ? i : m - 1];
+        else kb.kbs[t] = 0;
+    }
+}
+
+// Buffer coefficients for scalar decays (GDN, Mamba2): c[v][i] = exp(gcur - G_i) (K_i . x_v) for slots i < n, else 0
+// (reference `_coefs`, _fold_triton.py:260-272).  `gb` = the lane's slots' G (one per pass).  When the buffer is
+// about to be folded the dequantized keys of slots 0 .. m-2 are staged in LDS for the fold.
+template <class T, int NV>
+__device__ __forceinline__ void buffer_coefs(const KeyBuf<T>& kbuf, const float (&gb)[KeyBuf<T>::KT], float gcur,
+                                             int n, int m, bool full, const float (&x)[NV][CPL], const LaneId& l,
+                                             float* lds_k, float (&c)[NV][T::MMAX]) {
+    constexpr int KT = KeyBuf<T>::KT;
+    float cl[NV][KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        const int i = l.rg + T::RG * t;
+        float kb[CPL];
+        decode_kpiece<T>(kbuf.piece[t], f16_to_f32(kbuf.kbs[t]), l, kb);
+        const float dec = expf(gcur - gb[t]);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            float p = kb[0] * x[v][0];
+#pragma unroll
+            for (int k = 1; k < CPL; ++k) p = __builtin_fmaf(kb[k], x[v][k], p);
+            p = block_sum<T::LPRP>(p);
+            cl[v][t] = i < n ? dec * p : 0.0f;
+        }
+        if (full && i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int i = 0; i < T::MMAX; ++i) c[v][i] = lane_bcast(cl[v][i / T::RG], (i % T::RG) * T::LPRP);
+}
+
+// Append the current token's value row: int8 with one absmax scale over the whole row (`us`, stored by lane 0), or
+// bf16.  ur = the value as stored, dequantized (what the fold must use for slot n).
+template <class T>
+__device__ __forceinline__ void append_values(const float (&u)[T::NOWN], float us, const BufAddr<T>& a, int n,
+                                              const LaneId& l, int jown, float (&ur)[T::NOWN]) {
+    if (T::QBUF && l.lane == 0) a.UBS[n] = f32_to_f16(us);
+#pragma unroll
+    for (int t = 0; t < T::NOWN; ++t) {
+        const int r = row_of<T>(l, jown + t);
+        const bool valid = jown + t < T::RPL;
+        if constexpr (T::QBUF) {
+            const float c = round_buf(u[t], us);
+            ur[t] = c * us;
+            if (valid) reinterpret_cast<int8_t*>(a.UB)[n * T::DV + r] = int8_t(int(c));
+        } else {
+            const uint16_t hb = f32_to_bf16(u[t]);
+            ur[t] = bf16_to_f32(hb);
+            if (valid) reinterpret_cast<uint16_t*>(a.UB)[n * T::DV + r] = hb;
+        }
+    }
+}
+// Append the current token's key (element e = lane + 64 t of it sits in kx[t]); `write` = this head stores it.
+template <class T>
+__device__ __forceinline__ void append_key(const float (&kx)[T::NE], float ks, const BufAddr<T>& a, int n, bool write,
+                                           const LaneId& l, float (&kr)[T::NE]) {
+    if (T::QBUF && write && l.lane == 0) a.KBS[n] = f32_to_f16(ks);
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) {
+        const int e = l.lane + WAVE * t;
+        if constexpr (T::QBUF) {
+            const float c = round_buf(kx[t], ks);
+            kr[t] = c * ks;
+            if (write && e < T::DK) reinterpret_cast<int8_t*>(a.KB)[n * T::DK + e] = int8_t(int(c));
+        } else {
+            const uint16_t hb = f32_to_bf16(kx[t]);
+            kr[t] = bf16_to_f32(hb);
+            if (write && e < T::DK) reinterpret_cast<uint16_t*>(a.KB)[n * T::DK + e] = hb;
+        }
+    }
+}
+// Stage the fold's value operand: lds_u[i][row] = f_i x U_i[row] for every slot (slot m-1: the value just appended);
+// f_i = the slot's decay ratio held by lane i of `decf` (KDA passes 1).
+template <class T>
+__device__ __forceinline__ void stage_values(const int32_t (&ub)[T::MMAX][T::NOWN], float ubs_l, float decf,
+                                             const float (&ur)[T::NOWN], int m, const LaneId& l, int jown,
+                                             float* lds_u) {
+#pragma unroll
+    for (int t = 0; t < T::NOWN; ++t) {
+        const int r = row_of<T>(l, jown + t);
+#pragma unroll
+        for (int i = 0; i < T::MMAX; ++i) {
+            if (i < m) {
+                float uv = ub_value<T>(ub[i][t]);
+                if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
+                if (i == m - 1) uv = ur[t];
+                if (jown + t >= T::RPL) uv = 0.0f;
+                lds_u[i * T::UROW + r] = lane_bcast(decf, i) * uv;
+            }
+        }
+    }
+}
+template <class T>
+__device__ __forceinline__ void stage_key(const float (&kr)[T::NE], int slot, const LaneId& l, float* lds_k) {
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) {
+        const int e = l.lane + WAVE * t;
+        if (e < T::LPRP * CPL) lds_k[slot * T::KROW + kpos<T>(e)] = e < T::DK ? kr[t] : 0.0f;
     }
 }
 
