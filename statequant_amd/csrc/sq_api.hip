@@ -56,8 +56,11 @@ int check_state(const sq_state& s, const sq_layout& L, const char* who, sq::Stat
         return fail(SQ_E_ARG, "%s: codes must be %zu-byte aligned (base and per-sequence stride)", who, row_align);
     if (L.buffer_bits == 8 && (!aligned(s.KB, 16) || (s.sKB % 16)))
         return fail(SQ_E_ARG, "%s: int8 key buffer must be 16-byte aligned (base and per-sequence stride)", who);
-    if (!aligned(s.SC, 2) || !aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
-        return fail(SQ_E_ARG, "%s: misaligned scale / decay / counter pointer", who);
+    // scales and buffered values are staged into LDS with 128-bit loads
+    if (!aligned(s.SC, 16) || (s.sSC % 8) || !aligned(s.UB, 16) || ((s.sUB * (L.buffer_bits / 8)) % 16))
+        return fail(SQ_E_ARG, "%s: scales and value buffer must be 16-byte aligned (base and per-sequence stride)", who);
+    if (!aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
+        return fail(SQ_E_ARG, "%s: misaligned decay / counter pointer", who);
     st->S = static_cast<uint8_t*>(s.S);         st->sS = s.sS;
     st->SC = static_cast<uint16_t*>(s.SC);      st->sSC = s.sSC;
     st->KB = static_cast<uint8_t*>(s.KB);       st->sKB = s.sKB;

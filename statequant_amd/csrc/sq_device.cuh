@@ -197,6 +197,45 @@ __device__ __forceinline__ RawRow<BITS> encode_row(const float (&c)[CPL]) {
     }
     return r;
 }
+// Quantize a lane's 16 values of one row against scale 1/r: codes = clamp(rint(a r), +-qmax), packed as stored.
+// a r + 1.5 2^23 (one fma: the exact product, rounded once, half to even, at integer granularity) leaves the code in
+// the low mantissa bits in two's complement; int4 adds its +8 storage bias in the same constant.  The clamp acts on
+// the biased float, the bytes / nibbles are gathered with byte permutes.
+template <int BITS>
+__device__ __forceinline__ RawRow<BITS> quantize_row(const float (&a)[CPL], float r) {
+    constexpr float QMAX = float((1 << (BITS - 1)) - 1);
+    constexpr float MAGIC = 12582912.0f + (BITS == 4 ? 8.0f : 0.0f);
+    uint32_t u[CPL];
+#pragma unroll
+    for (int t = 0; t < CPL; ++t) {
+        const float f = __builtin_fmaf(a[t], r, MAGIC);
+        u[t] = as_u32(__builtin_amdgcn_fmed3f(f, MAGIC - QMAX, MAGIC + QMAX));
+    }
+    RawRow<BITS> o;
+    if constexpr (BITS == 8) {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t lo = __builtin_amdgcn_perm(u[4 * d + 1], u[4 * d], 0x0c0c0400u);
+            const uint32_t hi = __builtin_amdgcn_perm(u[4 * d + 3], u[4 * d + 2], 0x0c0c0400u);
+            w[d] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+        o.v = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {
+        uint32_t w[2];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            const uint32_t* e = u + 8 * d;                       // nibbles 0..7 of the word; each low byte is 1..15
+            const uint32_t ev = __builtin_amdgcn_perm(__builtin_amdgcn_perm(e[6], e[4], 0x0c0c0400u),
+                                                      __builtin_amdgcn_perm(e[2], e[0], 0x0c0c0400u), 0x05040100u);
+            const uint32_t od = __builtin_amdgcn_perm(__builtin_amdgcn_perm(e[7], e[5], 0x0c0c0400u),
+                                                      __builtin_amdgcn_perm(e[3], e[1], 0x0c0c0400u), 0x05040100u);
+            w[d] = ev | (od << 4);
+        }
+        o.v = make_uint2(w[0], w[1]);
+    }
+    return o;
+}
 template <int BITS>
 __device__ __forceinline__ void store_row(uint8_t* p, const RawRow<BITS>& r) {
     if constexpr (BITS == 8) *reinterpret_cast<uint4*>(p) = r.v;

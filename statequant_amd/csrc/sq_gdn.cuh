@@ -3,102 +3,143 @@
 // Replaces the reference's fused Triton step (/root/reference/src/statequant/kernels/_fused_triton.py:48-190) with
 // the same arithmetic per head:
 //   prep     q, k l2-normalised (eps inside the sqrt), the gates, c_q[i] = (a_n/a_i) k_i.q, c_k[i] likewise
-//   state    the stored codes read ONCE into registers; S0 q, S0 k by 16-column pieces + butterfly reduction;
-//            buffer term as a slot-ordered fma chain; u = beta (v - a sk), o = a sq + (k.q) u
+//   state    the stored codes streamed once through a register window; S0 q, S0 k by 16-column pieces + butterfly
+//            reduction; buffer term as a slot-ordered fma chain; u = beta (v - a sk), o = a sq + (k.q) u
 //   append   G_n, the delta value (int8 with one absmax scale over the row, or bf16), the key (first head of a
 //            GQA group only)
-//   fold     buffer full: S = a_m S0 + sum_i (a_m/a_i) u_i k_i^T from the codes still in registers (no second read
-//            of the state), re-quantized in place
+//   fold     buffer full: S = a_m S0 + sum_i (a_m/a_i) u_i k_i^T, re-quantized in place
 //   advance  running decay and this head's copy of the counter
-// Every load the step needs is issued before the first use of any of them (small operands first, then the state
-// tile), so a wavefront pays one memory round trip after the slot index, not one per operand.
+// Every load a tile needs is issued before the first use of any of them (small operands first, then the first
+// block of the state tile), so a wavefront pays one memory round trip after the slot index, not one per operand.
 #pragma once
 #include "sq_tile.cuh"
 #include "sq_params.h"
 
 namespace sq {
 
+// Where one tile's fields live.
 template <class T>
-__global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
-    __shared__ __attribute__((aligned(16))) float lds[T::LDS_FLOATS];
-    float* lds_k = lds;
-    float* lds_u = lds + T::MMAX * T::KROW;
-    float* lds_q = lds_u + T::MMAX * T::UROW;
-    float* lds_kn = lds_q + T::KROW;
-
-    const LaneId l = lane_id<T>();
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int b = tile / p.hv;
-    const int h = tile - b * p.hv;
-    const int gqa = p.hv / p.hk;
-    const int hk = h / gqa;
-    const int m = p.m;
-    constexpr int DK = T::DK, DV = T::DV;
-    constexpr int KT = KeyBuf<T>::KT;
-
-    const int64_t seq = p.idx ? int64_t(p.idx[b]) : int64_t(b);
-    const int64_t obase = (int64_t(b) * p.hv + h) * DV;
-    if (p.idx && seq <= 0) {                                     // padding row: zero output, touch nothing else
-        for (int r = l.lane; r < DV; r += WAVE) store_f(p.out, p.out_dt, obase + r, 0.0f);
-        return;
-    }
-
-    // ---- addresses ----
-    uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
-    uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
-    constexpr int BE = T::QBUF ? 1 : 2;                           // bytes per buffer element
+struct GdnAddr {
+    int b, h, hk;
+    bool live;                         // false: padding row (slot index <= 0)
+    int64_t obase;
+    uint8_t* Sh;
+    uint16_t* SCh;
     BufAddr<T> buf;
-    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * BE;
-    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * BE;
-    buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(hk) * m;
-    buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
-    float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
-    float* gcp = p.st.GCUR + seq * p.st.sGC + h;
-    int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const int jown = own_first<T>(l);
-    const int hq = p.qk_per_key_head ? hk : h;
-    const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
+    float* GBh;
+    float* gcp;
+    int32_t* np;
+};
+template <class T>
+__device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p, int tile) {
+    GdnAddr<T> a;
+    a.b = tile / p.hv;
+    a.h = tile - a.b * p.hv;
+    a.hk = a.h / (p.hv / p.hk);
+    const int64_t seq = p.idx ? int64_t(p.idx[a.b]) : int64_t(a.b);
+    a.live = !(p.idx && seq <= 0);
+    a.obase = (int64_t(a.b) * p.hv + a.h) * T::DV;
+    const int m = p.m;
+    a.Sh = p.st.S + seq * p.st.sS + int64_t(a.h) * (T::DV * T::ROW_BYTES);
+    a.SCh = p.st.SC + seq * p.st.sSC + int64_t(a.h) * (T::DV * T::NG);
+    a.buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(a.hk) * m * T::DK) * T::BE;
+    a.buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(a.h) * m * T::DV) * T::BE;
+    a.buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(a.hk) * m;
+    a.buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(a.h) * m;
+    a.GBh = p.st.GB + seq * p.st.sGB + int64_t(a.h) * m;
+    a.gcp = p.st.GCUR + seq * p.st.sGC + a.h;
+    a.np = p.st.NPTR + seq * p.st.sN + a.h;
+    return a;
+}
 
-    // ---- issue every load: counters, buffer, inputs, then the state tile ----
-    const int n = *np & (m - 1);
-    const float gcur = *gcp;
-    const int lm = l.lane < m ? l.lane : m - 1;
-    uint16_t ubs_raw = 0;
-    if constexpr (T::QBUF) ubs_raw = buf.UBS[lm];
-    const float gb_lane = GBh[lm];                                // lane i: slot i's cumulative decay
-    int32_t ub[T::MMAX][T::NOWN];
-    load_ub<T>(buf.UB, m, l, jown, ub);
+// Everything a tile's step reads before its state pass, as issued loads: counters, buffer, inputs, the first block of
+// the state tile.  Raw bits only; nothing here waits for memory.
+template <class T>
+struct GdnFront {
+    static constexpr int KT = KeyBuf<T>::KT;
+    int n;
+    float gcur;
+    uint16_t ubs_raw;
+    float gb_lane;
+    Staged<T::UB_BYTES> st_ub;
+    Staged<T::SC_BYTES> st_sc;
     KeyBuf<T> kbuf;
-    load_keybuf<T>(buf, m, l, kbuf);
     float gb[KT];
+    uint32_t qr[T::NE], kr[T::NE], kxr[T::NE];
+    uint32_t g0, g1, g2, g3;
+    uint32_t vr[T::NOWN];
+    Window<T> win;
+};
+template <class T>
+__device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& a, const LaneId& l, GdnFront<T>& f) {
+    constexpr int DK = T::DK, DV = T::DV;
+    const int m = p.m;
+    const int gqa = p.hv / p.hk;
+    const int hq = p.qk_per_key_head ? a.hk : a.h;
+    const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
+    f.n = *a.np & (m - 1);
+    f.gcur = *a.gcp;
+    const int lm = l.lane < m ? l.lane : m - 1;
+    f.ubs_raw = 0;
+    if constexpr (T::QBUF) f.ubs_raw = a.buf.UBS[lm];
+    f.gb_lane = a.GBh[lm];                                       // lane i: slot i's cumulative decay
+    stage_load(a.buf.UB, m * DV * T::BE, l.lane, f.st_ub);
+    stage_load(reinterpret_cast<const uint8_t*>(a.SCh), DV * T::NG * 2, l.lane, f.st_sc);
+    load_keybuf<T>(a.buf, m, l, f.kbuf);
 #pragma unroll
-    for (int t = 0; t < KT; ++t) { const int i = l.rg + T::RG * t; gb[t] = GBh[i < m ? i : m - 1]; }
-    uint32_t qr[T::NE], kr_[T::NE], kxr[T::NE];
+    for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < m ? i : m - 1]; }
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
         int e = l.lane + WAVE * t;
         e = e < DK ? e : DK - 1;
-        qr[t] = load_raw(p.q, p.q_dt, int64_t(b) * p.s_q + int64_t(hq) * DK + e);
-        kr_[t] = load_raw(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hq) * DK + e);
-        kxr[t] = own_key ? load_raw(p.k, p.k_dt, int64_t(b) * p.s_k + int64_t(hk * gqa) * DK + e) : 0u;
+        f.qr[t] = load_raw(p.q, p.q_dt, int64_t(a.b) * p.s_q + int64_t(hq) * DK + e);
+        f.kr[t] = load_raw(p.k, p.k_dt, int64_t(a.b) * p.s_k + int64_t(hq) * DK + e);
+        f.kxr[t] = own_key ? load_raw(p.k, p.k_dt, int64_t(a.b) * p.s_k + int64_t(a.hk * gqa) * DK + e) : 0u;
     }
     // gate: a, b [rows, hv], A_log, dt_bias [hv];  no gate: the same four slots carry g, beta and two dummies
     // (the C ABI points them at g), so the loads need no branch
-    const uint32_t g0 = load_raw_uniform(p.a, p.a_dt, int64_t(b) * p.s_a + h);
-    const uint32_t g1 = load_raw_uniform(p.bt, p.bt_dt, int64_t(b) * p.s_bt + h);
-    const uint32_t g2 = load_raw_uniform(p.A_log, p.A_log_dt, h);
-    const uint32_t g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);
-    uint32_t vr[T::NOWN];
+    f.g0 = load_raw_uniform(p.a, p.a_dt, int64_t(a.b) * p.s_a + a.h);
+    f.g1 = load_raw_uniform(p.bt, p.bt_dt, int64_t(a.b) * p.s_bt + a.h);
+    f.g2 = load_raw_uniform(p.A_log, p.A_log_dt, a.h);
+    f.g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, a.h);
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = row_of<T>(l, jown + t);
+        int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        vr[t] = load_raw(p.v, p.v_dt, int64_t(b) * p.s_v + int64_t(h) * DV + r);
+        f.vr[t] = load_raw(p.v, p.v_dt, int64_t(a.b) * p.s_v + int64_t(a.h) * DV + r);
     }
-    RawRow<T::BITS> raw[T::RPL];
-    load_tile<T>(Sh, l, raw);
-    uint16_t scr[T::RPL];
-    load_scales<T>(SCh, l, scr);
+    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
+}
+
+template <class T>
+__global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
+    using L = LdsPlan<T, 2>;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
+    float* lds_q = reinterpret_cast<float*>(lds + L::X);
+    float* lds_kn = lds_q + T::KROW;
+    uint8_t* lds_ub = lds + L::UB;
+    uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    float* lds_k = reinterpret_cast<float*>(lds + L::FK);          // the fold's operands overlay the above
+    float* lds_u = reinterpret_cast<float*>(lds + L::FU);
+
+    const int gqa = p.hv / p.hk;
+    const int m = p.m;
+    constexpr int DK = T::DK, DV = T::DV;
+    constexpr int KT = KeyBuf<T>::KT;
+    const bool own_key = !p.qk_per_key_head && gqa > 1;
+    const LaneId l = lane_id<T>();
+    const int tile = xcd_tile(blockIdx.x, gridDim.x);
+    const GdnAddr<T> A = gdn_addr<T>(p, tile);
+    if (!A.live) {                                                // padding row: zero output, touch nothing else
+        for (int r = l.lane; r < DV; r += WAVE) store_f(p.out, p.out_dt, A.obase + r, 0.0f);
+        return;
+    }
+    GdnFront<T> F;
+    gdn_issue<T>(p, A, l, F);
+    const int h = A.h;
+    const int n = F.n;
+    const float gcur = F.gcur;
+    const uint8_t* lane_base = lane_codes<T>(A.Sh, l);
 
     // ---- prep: q, k (fla's l2 normalisation), gates ----
     const bool full = n == m - 1;
@@ -107,9 +148,9 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
         const bool in = l.lane + WAVE * t < DK;
-        qe[t] = in ? raw_to_f(qr[t], p.q_dt) : 0.0f;
-        ke[t] = in ? raw_to_f(kr_[t], p.k_dt) : 0.0f;
-        kxe[t] = in ? raw_to_f(kxr[t], p.k_dt) : 0.0f;
+        qe[t] = in ? raw_to_f(F.qr[t], p.q_dt) : 0.0f;
+        ke[t] = in ? raw_to_f(F.kr[t], p.k_dt) : 0.0f;
+        kxe[t] = in ? raw_to_f(F.kxr[t], p.k_dt) : 0.0f;
         ssq = __builtin_fmaf(qe[t], qe[t], ssq);
         ssk = __builtin_fmaf(ke[t], ke[t], ssk);
         ssx = __builtin_fmaf(kxe[t], kxe[t], ssx);
@@ -125,6 +166,8 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
         const int e = l.lane + WAVE * t;
         if (e < T::LPRP * CPL) { lds_q[kpos<T>(e)] = qe[t]; lds_kn[kpos<T>(e)] = ke[t]; }
     }
+    stage_store(lds_ub, m * DV * T::BE, l.lane, F.st_ub);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, F.st_sc);
     const float kq = wave_sum(kqp);
     if (own_key) {
         const float nx = sqrtf(wave_sum(ssx) + 1e-6f);
@@ -136,18 +179,20 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
     }
     float g, beta;
     if (p.gate) {
-        const float x = raw_to_f(g0, p.a_dt) + raw_to_f(g3, p.dt_bias_dt);
+        const float x = raw_to_f(F.g0, p.a_dt) + raw_to_f(F.g3, p.dt_bias_dt);
         const float sp = x <= 20.0f ? logf(1.0f + expf(x)) : x;
-        g = -expf(raw_to_f(g2, p.A_log_dt)) * sp;
-        beta = 1.0f / (1.0f + expf(-raw_to_f(g1, p.bt_dt)));
+        g = -expf(raw_to_f(F.g2, p.A_log_dt)) * sp;
+        beta = 1.0f / (1.0f + expf(-raw_to_f(F.g1, p.bt_dt)));
     } else {
-        g = raw_to_f(g0, p.a_dt);
-        beta = raw_to_f(g1, p.bt_dt);
+        g = raw_to_f(F.g0, p.a_dt);
+        beta = raw_to_f(F.g1, p.bt_dt);
     }
     const float alpha = expf(gcur);
     const float a = expf(g);
     const float gnew = gcur + g;
-    const float ubs_l = T::QBUF ? f16_to_f32(ubs_raw) : 1.0f;
+    float ubs[T::MMAX];
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(F.ubs_raw), i) : 1.0f;
     __syncthreads();
     float x[2][CPL];
     lds_piece<T>(lds_q, l.cg, x[0]);
@@ -155,37 +200,37 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
 
     // ---- buffer coefficients ----
     float c[2][T::MMAX];
-    buffer_coefs<T, 2>(kbuf, gb, gcur, n, m, full, x, l, lds_k, c);
+    buffer_coefs<T, 2>(F.kbuf, F.gb, gcur, n, x, l, c);
 
     // ---- state pass ----
-    mask_tile<T>(l, raw);
-    float sc[T::RPL];
-    scale_values<T>(scr, l, sc);
-    float part[2][T::RPLP];
-    tile_dots<T, 2>(raw, x, part);
     float own[2][T::NOWN];
-    reduce_rows<T, 2>(part, sc, l, own);
+    state_pass<T, 2>(lane_base, F.win, x, lds_sc, l, own);
+
+    const KeyBuf<T>& kbuf = F.kbuf;
+    const float gb_lane = F.gb_lane;
+    const uint32_t (&vr)[T::NOWN] = F.vr;
 
     // ---- the rows this lane owns: buffer term, u, o ----
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
-        const bool valid = jown + t < T::RPL;
+        const bool valid = owned_valid<T>(l, t);
+        int r = owned_row<T>(l, t);
+        r = r < DV ? r : DV - 1;
         float sq = alpha * own[0][t];
         float sk = alpha * own[1][t];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_value<T>(ub[i][t]);
-            if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
-            uv = i < n ? uv : 0.0f;                               // dead slots may hold anything: discard
+            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
+            if constexpr (T::QBUF) uv = uv * ubs[i];
+            uv = i < n ? uv : 0.0f;                       // dead slots may hold anything: discard
             sq = __builtin_fmaf(uv, c[0][i], sq);
             sk = __builtin_fmaf(uv, c[1][i], sk);
         }
         const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * __builtin_fmaf(-a, sk, vt);
         const float o = __builtin_fmaf(kq, u[t], a * sq);
-        if (valid) store_f(p.out, p.out_dt, obase + r, o);
+        if (valid) store_f(p.out, p.out_dt, A.obase + r, o);
         else u[t] = 0.0f;
         amax = fmaxf(amax, fabsf(u[t]));
     }
@@ -199,28 +244,37 @@ __global__ __launch_bounds__(WAVE) void gdn_step_kernel(const GdnParams p) {
         for (int t = 0; t < T::NE; ++t) kmax = fmaxf(kmax, fabsf(kxe[t]));
         ks = fp16_scale(wave_max(kmax), 127.0f);
     }
-    float ur[T::NOWN], kr[T::NE];                                 // value / key as stored, dequantized
-    append_values<T>(u, us, buf, n, l, jown, ur);
-    append_key<T>(kxe, ks, buf, n, (h % gqa) == 0, l, kr);
-    if (l.lane == 0) GBh[n] = gnew;
+    float ur[T::NOWN], kr[T::NE];                         // value / key as stored, dequantized
+    append_values<T>(u, us, A.buf, n, l, ur);
+    append_key<T>(kxe, ks, A.buf, n, (h % gqa) == 0, l, kr);
+    if (l.lane == 0) A.GBh[n] = gnew;
 
     // ---- fold ----
     if (full) {
-        const float decf = l.lane < m - 1 ? expf(gnew - gb_lane) : 1.0f;     // a_m / a_i; the current token's: 1
-        stage_values<T>(ub, ubs_l, decf, ur, m, l, jown, lds_u);
-        stage_key<T>(kr, m - 1, l, lds_k);
-        __syncthreads();
-        const float alphan = expf(gnew);
-        float colmul[CPL];
+        float uo[T::NOWN][T::MMAX];
+        fold_fetch_values<T>(lds_ub, ubs, ur, m, l, uo);
+        const float decf = l.lane < m - 1 ? expf(gnew - gb_lane) : 1.0f;     // a_m / a_i; current token: 1
+        float f[T::MMAX];
 #pragma unroll
-        for (int k = 0; k < CPL; ++k) colmul[k] = alphan;
-        fold_tile<T>(raw, sc, colmul, lds_k, lds_u, m, Sh, SCh, l);
+        for (int i = 0; i < T::MMAX; ++i) f[i] = lane_bcast(decf, i);
+        __syncthreads();                                  // the front end's LDS is dead from here on
+        fold_stage_values<T>(uo, f, m, l, lds_u);
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            const int i = l.rg + T::RG * t;
+            float kb[CPL];
+            decode_kpiece<T>(kbuf.piece[t], f16_to_f32(kbuf.kbs[t]), l, kb);
+            if (i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
+        }
+        fold_stage_key<T>(kr, m - 1, l, lds_k);
+        __syncthreads();
+        fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
     }
 
     // ---- advance ----
     if (l.lane == 0) {
-        *gcp = full ? 0.0f : gnew;
-        *np = full ? 0 : n + 1;
+        *A.gcp = full ? 0.0f : gnew;
+        *A.np = full ? 0 : n + 1;
     }
 }
 

@@ -7,7 +7,7 @@
 //   S'^T x = S0^T (A * x) + sum_i c_x[i] u_i;   u = beta (v - S'^T k);   o = S'^T q + (k.q) u
 //   fold (buffer full): S = S0 diag(A) + sum_i u_i (exp(G_n - G_i) * k_i)^T, re-quantized in place
 // The buffer keeps the cumulative decay per channel: GB is [h, m, d_k], GCUR is [h, d_k].  No grouped keys.
-// Loads are issued up front (small operands, then the state tile) as in the GDN step.
+// Structure (loads up front, streamed tile, LDS staging, fold overlay) as in the GDN step.
 #pragma once
 #include "sq_tile.cuh"
 #include "sq_params.h"
@@ -15,16 +15,19 @@
 namespace sq {
 
 template <class T>
-__global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
-    // folded keys, folded values, then five d_k vectors: q, k (normalised), A*q, A*k, G_n
-    __shared__ __attribute__((aligned(16))) float lds[T::MMAX * T::KROW + T::MMAX * T::UROW + 5 * T::KROW];
-    float* lds_k = lds;
-    float* lds_u = lds + T::MMAX * T::KROW;
-    float* lds_q = lds_u + T::MMAX * T::UROW;
+__global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
+    using L = LdsPlan<T, 5>;                                      // q, k (normalised), A*q, A*k, G_n
+    __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
+    float* lds_q = reinterpret_cast<float*>(lds + L::X);
     float* lds_kn = lds_q + T::KROW;
     float* lds_qa = lds_kn + T::KROW;
     float* lds_ka = lds_qa + T::KROW;
     float* lds_g = lds_ka + T::KROW;
+    uint8_t* lds_ub = lds + L::UB;
+    uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    float* lds_k = reinterpret_cast<float*>(lds + L::FK);
+    float* lds_u = reinterpret_cast<float*>(lds + L::FU);
+    float* lds_c = reinterpret_cast<float*>(lds + L::FC);
 
     const LaneId l = lane_id<T>();
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
@@ -43,24 +46,25 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
 
     uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
     uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
-    constexpr int BE = T::QBUF ? 1 : 2;
     BufAddr<T> buf;
-    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(h) * m * DK) * BE;
-    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * BE;
+    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(h) * m * DK) * T::BE;
+    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * T::BE;
     buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(h) * m;
     buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m * DK;
     float* gch = p.st.GCUR + seq * p.st.sGC + int64_t(h) * DK;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const int jown = own_first<T>(l);
+    const uint8_t* lane_base = lane_codes<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
     // ---- issue every load ----
     const int n = *np & (m - 1);
     uint16_t ubs_raw = 0;
     if constexpr (T::QBUF) ubs_raw = buf.UBS[l.lane < m ? l.lane : m - 1];
-    int32_t ub[T::MMAX][T::NOWN];
-    load_ub<T>(buf.UB, m, l, jown, ub);
+    Staged<T::UB_BYTES> st_ub;
+    stage_load(buf.UB, m * DV * T::BE, l.lane, st_ub);
+    Staged<T::SC_BYTES> st_sc;
+    stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
     KeyBuf<T> kbuf;
     load_keybuf<T>(buf, m, l, kbuf);
     float4 gbp[KT][CPL / 4];                                      // the lane's piece of G_i of its slot(s)
@@ -87,14 +91,12 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
     uint32_t vr[T::NOWN];
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = row_of<T>(l, jown + t);
+        int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
         vr[t] = load_raw(p.v, p.v_dt, int64_t(b) * p.s_v + int64_t(h) * DV + r);
     }
-    RawRow<T::BITS> raw[T::RPL];
-    load_tile<T>(Sh, l, raw);
-    uint16_t scr[T::RPL];
-    load_scales<T>(SCh, l, scr);
+    Window<T> win;
+    window_init<T>(lane_base, win);
 
     // ---- prep: q, k normalised, the running decay per channel ----
     const bool full = n == m - 1;
@@ -128,42 +130,43 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
             lds_g[pos] = gn[t];
         }
     }
+    stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
     const float kq = wave_sum(kqp);
     const float beta = raw_to_f(betar, p.beta_dt);
-    const float ubs_l = T::QBUF ? f16_to_f32(ubs_raw) : 1.0f;
+    float ubs[T::MMAX];
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(ubs_raw), i) : 1.0f;
     __syncthreads();
-    float xn[2][CPL], gp[CPL];
-    lds_piece<T>(lds_q, l.cg, xn[0]);
-    lds_piece<T>(lds_kn, l.cg, xn[1]);
-    lds_piece<T>(lds_g, l.cg, gp);
 
     // ---- buffer coefficients with the per-channel decay ratio folded into the buffered key ----
     float cq[T::MMAX], ck[T::MMAX];
     {
+        float xn[2][CPL], gp[CPL];
+        lds_piece<T>(lds_q, l.cg, xn[0]);
+        lds_piece<T>(lds_kn, l.cg, xn[1]);
+        lds_piece<T>(lds_g, l.cg, gp);
         float cq_l[KT], ck_l[KT];
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
             const int i = l.rg + T::RG * t;
-            float kb[CPL], kd[CPL];
+            float kb[CPL];
             decode_kpiece<T>(kbuf.piece[t], f16_to_f32(kbuf.kbs[t]), l, kb);
             const bool alive = i < n;                             // dead slots may hold anything: discard
+            float pq = 0.0f, pk = 0.0f;
 #pragma unroll
             for (int k = 0; k < CPL / 4; ++k) {
                 const float4 gi = gbp[t][k];
-                kd[4 * k] = alive ? kb[4 * k] * expf(gp[4 * k] - gi.x) : 0.0f;
-                kd[4 * k + 1] = alive ? kb[4 * k + 1] * expf(gp[4 * k + 1] - gi.y) : 0.0f;
-                kd[4 * k + 2] = alive ? kb[4 * k + 2] * expf(gp[4 * k + 2] - gi.z) : 0.0f;
-                kd[4 * k + 3] = alive ? kb[4 * k + 3] * expf(gp[4 * k + 3] - gi.w) : 0.0f;
-            }
-            float pq = kd[0] * xn[0][0], pk = kd[0] * xn[1][0];
+                const float gv[4] = {gi.x, gi.y, gi.z, gi.w};
 #pragma unroll
-            for (int k = 1; k < CPL; ++k) {
-                pq = __builtin_fmaf(kd[k], xn[0][k], pq);
-                pk = __builtin_fmaf(kd[k], xn[1][k], pk);
+                for (int e = 0; e < 4; ++e) {
+                    const float kd = alive ? kb[4 * k + e] * expf(gp[4 * k + e] - gv[e]) : 0.0f;
+                    if (k == 0 && e == 0) { pq = kd * xn[0][0]; pk = kd * xn[1][0]; }
+                    else { pq = __builtin_fmaf(kd, xn[0][4 * k + e], pq); pk = __builtin_fmaf(kd, xn[1][4 * k + e], pk); }
+                }
             }
             cq_l[t] = block_sum<T::LPRP>(pq);
             ck_l[t] = block_sum<T::LPRP>(pk);
-            if (full && i < m - 1) stage_kpiece<T>(lds_k, i, l, kd);   // full: every slot below m-1 is alive
         }
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
@@ -173,28 +176,26 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
     }
 
     // ---- state pass against A*q, A*k ----
-    float x[2][CPL];
-    lds_piece<T>(lds_qa, l.cg, x[0]);
-    lds_piece<T>(lds_ka, l.cg, x[1]);
-    mask_tile<T>(l, raw);
-    float sc[T::RPL];
-    scale_values<T>(scr, l, sc);
-    float part[2][T::RPLP];
-    tile_dots<T, 2>(raw, x, part);
     float own[2][T::NOWN];
-    reduce_rows<T, 2>(part, sc, l, own);
+    {
+        float x[2][CPL];
+        lds_piece<T>(lds_qa, l.cg, x[0]);
+        lds_piece<T>(lds_ka, l.cg, x[1]);
+        state_pass<T, 2>(lane_base, win, x, lds_sc, l, own);
+    }
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
-        const bool valid = jown + t < T::RPL;
+        const bool valid = owned_valid<T>(l, t);
+        int r = owned_row<T>(l, t);
+        r = r < DV ? r : DV - 1;
         float sq = own[0][t];
         float sk = own[1][t];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_value<T>(ub[i][t]);
-            if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
+            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
+            if constexpr (T::QBUF) uv = uv * ubs[i];
             uv = i < n ? uv : 0.0f;
             sq = __builtin_fmaf(uv, cq[i], sq);
             sk = __builtin_fmaf(uv, ck[i], sk);
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
         ks = fp16_scale(wave_max(kmax), 127.0f);
     }
     float ur[T::NOWN], kr[T::NE];
-    append_values<T>(u, us, buf, n, l, jown, ur);
+    append_values<T>(u, us, buf, n, l, ur);
     append_key<T>(ke, ks, buf, n, true, l, kr);
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
@@ -227,13 +228,38 @@ __global__ __launch_bounds__(WAVE) void kda_step_kernel(const KdaParams p) {
 
     // ---- fold ----
     if (full) {
-        stage_values<T>(ub, ubs_l, 1.0f, ur, m, l, jown, lds_u);
-        stage_key<T>(kr, m - 1, l, lds_k);                        // the current token's decay ratio is exp(0) = 1
-        __syncthreads();
-        float colmul[CPL];
+        float uo[T::NOWN][T::MMAX];
+        fold_fetch_values<T>(lds_ub, ubs, ur, m, l, uo);
+        float gp[CPL];
+        lds_piece<T>(lds_g, l.cg, gp);
+        float f[T::MMAX];
 #pragma unroll
-        for (int k = 0; k < CPL; ++k) colmul[k] = expf(gp[k]);    // = A on this lane's columns
-        fold_tile<T>(raw, sc, colmul, lds_k, lds_u, m, Sh, SCh, l);
+        for (int i = 0; i < T::MMAX; ++i) f[i] = 1.0f;            // the decay ratio sits on the keys, per channel
+        __syncthreads();                                          // the front end's LDS is dead from here on
+        fold_stage_values<T>(uo, f, m, l, lds_u);
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            const int i = l.rg + T::RG * t;
+            float kb[CPL];
+            decode_kpiece<T>(kbuf.piece[t], f16_to_f32(kbuf.kbs[t]), l, kb);
+#pragma unroll
+            for (int k = 0; k < CPL / 4; ++k) {
+                const float4 gi = gbp[t][k];
+                kb[4 * k] = kb[4 * k] * expf(gp[4 * k] - gi.x);
+                kb[4 * k + 1] = kb[4 * k + 1] * expf(gp[4 * k + 1] - gi.y);
+                kb[4 * k + 2] = kb[4 * k + 2] * expf(gp[4 * k + 2] - gi.z);
+                kb[4 * k + 3] = kb[4 * k + 3] * expf(gp[4 * k + 3] - gi.w);
+            }
+            if (i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
+        }
+        fold_stage_key<T>(kr, m - 1, l, lds_k);                   // the current token's decay ratio is exp(0) = 1
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) {
+            const int e = l.lane + WAVE * t;
+            if (e < T::LPRP * CPL) lds_c[kpos<T>(e)] = e < DK ? expf(gn[t]) : 0.0f;     // = A
+        }
+        __syncthreads();
+        fold_tile<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
     }
 
     // ---- advance ----

@@ -5,7 +5,7 @@
 // term, no normalisation:
 //   y_n = a_n [alpha S0 C + sum_{i<n} (alpha/alpha_i) (B_i.C) u_i] + (B_n.C) u_n + D x_n
 //   fold (buffer full): S = alpha_m S0 + sum_i (alpha_m/alpha_i) u_i B_i^T, re-quantized in place
-// Loads are issued up front (small operands, then the state tile) as in the GDN step.
+// Structure (loads up front, streamed tile, LDS staging, fold overlay) as in the GDN step.
 #pragma once
 #include "sq_tile.cuh"
 #include "sq_params.h"
@@ -13,11 +13,14 @@
 namespace sq {
 
 template <class T>
-__global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p) {
-    __shared__ __attribute__((aligned(16))) float lds[T::LDS_FLOATS];
-    float* lds_k = lds;
-    float* lds_u = lds + T::MMAX * T::KROW;
-    float* lds_c = lds_u + T::MMAX * T::UROW;
+__global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params p) {
+    using L = LdsPlan<T, 1>;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
+    float* lds_cv = reinterpret_cast<float*>(lds + L::X);
+    uint8_t* lds_ub = lds + L::UB;
+    uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    float* lds_k = reinterpret_cast<float*>(lds + L::FK);
+    float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
     const LaneId l = lane_id<T>();
     const int tile = xcd_tile(blockIdx.x, gridDim.x);
@@ -38,16 +41,15 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
 
     uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
     uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
-    constexpr int BE = T::QBUF ? 1 : 2;
     BufAddr<T> buf;
-    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * BE;
-    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * BE;
+    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * T::BE;
+    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * T::BE;
     buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(hk) * m;
     buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
     float* gcp = p.st.GCUR + seq * p.st.sGC + h;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const int jown = own_first<T>(l);
+    const uint8_t* lane_base = lane_codes<T>(Sh, l);
 
     // ---- issue every load ----
     const int n = *np & (m - 1);
@@ -56,8 +58,10 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
     uint16_t ubs_raw = 0;
     if constexpr (T::QBUF) ubs_raw = buf.UBS[lm];
     const float gb_lane = GBh[lm];
-    int32_t ub[T::MMAX][T::NOWN];
-    load_ub<T>(buf.UB, m, l, jown, ub);
+    Staged<T::UB_BYTES> st_ub;
+    stage_load(buf.UB, m * DV * T::BE, l.lane, st_ub);
+    Staged<T::SC_BYTES> st_sc;
+    stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
     KeyBuf<T> kbuf;
     load_keybuf<T>(buf, m, l, kbuf);
     float gb[KT];
@@ -78,14 +82,12 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
     uint32_t xr_raw[T::NOWN];
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = row_of<T>(l, jown + t);
+        int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
         xr_raw[t] = load_raw(p.x, p.x_dt, int64_t(b) * p.s_x + int64_t(h) * DV + r);
     }
-    RawRow<T::BITS> raw[T::RPL];
-    load_tile<T>(Sh, l, raw);
-    uint16_t scr[T::RPL];
-    load_scales<T>(SCh, l, scr);
+    Window<T> win;
+    window_init<T>(lane_base, win);
 
     // ---- prep: B, C of the group, dt, decay ----
     const bool full = n == m - 1;
@@ -97,8 +99,10 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
         ce[t] = e < DK ? raw_to_f(cr[t], p.C_dt) : 0.0f;
         kxe[t] = e < DK ? raw_to_f(br[t], p.B_dt) : 0.0f;
         bcp = __builtin_fmaf(kxe[t], ce[t], bcp);
-        if (e < T::LPRP * CPL) lds_c[kpos<T>(e)] = ce[t];
+        if (e < T::LPRP * CPL) lds_cv[kpos<T>(e)] = ce[t];
     }
+    stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
     const float bc = wave_sum(bcp);
     float dt = raw_to_f(dtr, p.dt_dt);
     if (p.has_dt_bias) dt = dt + raw_to_f(dbr, p.dt_bias_dt);
@@ -109,35 +113,33 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
     const float dd = p.has_D ? raw_to_f(ddr, p.D_dt) : 0.0f;
     const float alpha = expf(gcur);
     const float gnew = gcur + g;
-    const float ubs_l = T::QBUF ? f16_to_f32(ubs_raw) : 1.0f;
+    float ubs[T::MMAX];
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(ubs_raw), i) : 1.0f;
     __syncthreads();
     float x[1][CPL];
-    lds_piece<T>(lds_c, l.cg, x[0]);
+    lds_piece<T>(lds_cv, l.cg, x[0]);
 
     // ---- buffer coefficients c[i] = (alpha / alpha_i) B_i . C ----
     float c[1][T::MMAX];
-    buffer_coefs<T, 1>(kbuf, gb, gcur, n, m, full, x, l, lds_k, c);
+    buffer_coefs<T, 1>(kbuf, gb, gcur, n, x, l, c);
 
     // ---- state pass ----
-    mask_tile<T>(l, raw);
-    float sc[T::RPL];
-    scale_values<T>(scr, l, sc);
-    float part[1][T::RPLP];
-    tile_dots<T, 1>(raw, x, part);
     float own[1][T::NOWN];
-    reduce_rows<T, 1>(part, sc, l, own);
+    state_pass<T, 1>(lane_base, win, x, lds_sc, l, own);
 
     // ---- owned rows: y, and the value to buffer ----
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
-        const bool valid = jown + t < T::RPL;
+        const bool valid = owned_valid<T>(l, t);
+        int r = owned_row<T>(l, t);
+        r = r < DV ? r : DV - 1;
         float sq = alpha * own[0][t];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_value<T>(ub[i][t]);
-            if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
+            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
+            if constexpr (T::QBUF) uv = uv * ubs[i];
             uv = i < n ? uv : 0.0f;
             sq = __builtin_fmaf(uv, c[0][i], sq);
         }
@@ -159,21 +161,30 @@ __global__ __launch_bounds__(WAVE) void mamba2_step_kernel(const Mamba2Params p)
         ks = fp16_scale(wave_max(kmax), 127.0f);
     }
     float ur[T::NOWN], kr[T::NE];
-    append_values<T>(u, us, buf, n, l, jown, ur);
+    append_values<T>(u, us, buf, n, l, ur);
     append_key<T>(kxe, ks, buf, n, (h % gqa) == 0, l, kr);
     if (l.lane == 0) GBh[n] = gnew;
 
     // ---- fold ----
     if (full) {
+        float uo[T::NOWN][T::MMAX];
+        fold_fetch_values<T>(lds_ub, ubs, ur, m, l, uo);
         const float decf = l.lane < m - 1 ? expf(gnew - gb_lane) : 1.0f;
-        stage_values<T>(ub, ubs_l, decf, ur, m, l, jown, lds_u);
-        stage_key<T>(kr, m - 1, l, lds_k);
-        __syncthreads();
-        const float alphan = expf(gnew);
-        float colmul[CPL];
+        float f[T::MMAX];
 #pragma unroll
-        for (int k = 0; k < CPL; ++k) colmul[k] = alphan;
-        fold_tile<T>(raw, sc, colmul, lds_k, lds_u, m, Sh, SCh, l);
+        for (int i = 0; i < T::MMAX; ++i) f[i] = lane_bcast(decf, i);
+        __syncthreads();
+        fold_stage_values<T>(uo, f, m, l, lds_u);
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            const int i = l.rg + T::RG * t;
+            float kb[CPL];
+            decode_kpiece<T>(kbuf.piece[t], f16_to_f32(kbuf.kbs[t]), l, kb);
+            if (i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
+        }
+        fold_stage_key<T>(kr, m - 1, l, lds_k);
+        __syncthreads();
+        fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
     }
 
     if (l.lane == 0) {

@@ -1,6 +1,12 @@
-// The state tile of one (sequence, value head) in one wavefront: geometry, the single read of the stored codes, the
-// row dot products with cross-lane reduction, and the fold (advance across the full buffer + re-quantize in place).
-// Shared by the Gated DeltaNet, KDA and Mamba2 step kernels.
+// The state tile of one (sequence, value head) in one wavefront: geometry, the streaming read of the stored codes
+// with the row dot products and their cross-lane reduction, the decode buffer, and the fold (advance across the
+// full buffer + re-quantize in place).  Shared by the Gated DeltaNet, KDA and Mamba2 step kernels.
+//
+// Resource plan (what keeps four wavefronts per SIMD resident): the codes stream through a window of LPRP rows per
+// lane (32 VGPRs for int8), refilled row by row; the small operands (buffered values, scales) are fetched with one
+// coalesced 128-bit load per lane and parked in LDS until needed; the fold reads the codes a second time (from L2 /
+// Infinity Cache: they were read microseconds earlier) instead of pinning them in registers; the fold's LDS
+// operands overlay the front end's.
 #pragma once
 #include "sq_device.cuh"
 
@@ -8,7 +14,8 @@ namespace sq {
 
 // Compile-time geometry.  A row of DK codes is cut into DK/16 pieces of 16 columns; LPRP (that count rounded up to a
 // power of two) consecutive lanes hold one row, lanes past DK/16 idle (d_k = 96: 6 of 8).  The wavefront therefore
-// covers RG = 64/LPRP rows per load and a lane sees rows rg, rg + RG, rg + 2 RG, ...
+// covers RG = 64/LPRP rows per load and a lane sees rows rg, rg + RG, rg + 2 RG, ...  Rows are handled in blocks of
+// LPRP per lane (one reduce-scatter each), after which every lane owns one row of the block.
 template <int BITS_, int DK_, int DV_, int GROUP_, bool QBUF_, int MMAX_>
 struct Tile {
     static constexpr int BITS = BITS_, DK = DK_, DV = DV_, GROUP = GROUP_, MMAX = MMAX_;
@@ -20,8 +27,8 @@ struct Tile {
     static constexpr int RG = WAVE / LPRP;                // rows per wavefront load
     static_assert(DV % (4 * RG) == 0, "d_v must be a multiple of 4 x the rows one wavefront load covers");
     static constexpr int RPL = DV / RG;                   // rows per lane
-    static constexpr int RPLP = round_up(RPL, LPRP);      // padded so the reduce-scatter divides evenly
-    static constexpr int NOWN = RPLP / LPRP;              // rows a lane owns after the reduction
+    static constexpr int NOWN = (RPL + LPRP - 1) / LPRP;  // row blocks per lane = rows a lane owns
+    static constexpr int RPLP = NOWN * LPRP;              // rows per lane, padded to whole blocks
     static constexpr int NG = (DK + GROUP - 1) / GROUP;   // stored key groups per row (last may be ragged)
     static_assert(GROUP % CPL == 0 && GROUP >= CPL, "key group must be a multiple of 16");
     static constexpr int LPG = (GROUP / CPL < LPRP) ? GROUP / CPL : LPRP;   // lanes sharing one scale
@@ -31,10 +38,27 @@ struct Tile {
     static constexpr int LANE_BYTES = BITS == 4 ? CPL / 2 : CPL;
     static constexpr float QMAX = float((1 << (BITS - 1)) - 1);
     static constexpr int NE = (DK + WAVE - 1) / WAVE;     // elements of a d_k vector per lane (element = lane + 64 t)
+    static constexpr int BE = QBUF ? 1 : 2;               // bytes per buffer element (int8 / bf16)
     static constexpr int KPAD = CPL + 4;                  // LDS stride of a 16-column piece (spreads the banks)
     static constexpr int KROW = LPRP * KPAD;              // floats per d_k vector in LDS
     static constexpr int UROW = RPLP * RG;                // floats per d_v vector in LDS
-    static constexpr int LDS_FLOATS = MMAX * KROW + MMAX * UROW + 2 * KROW;
+    static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
+    static constexpr int SC_BYTES = round_up(DV * NG * 2, 16);
+};
+
+// LDS plan of a step kernel that stages NX d_k vectors.  Front end: the vectors, the raw buffered values, the raw
+// scales.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
+template <class T, int NX>
+struct LdsPlan {
+    static constexpr int X = 0;
+    static constexpr int UB = X + NX * T::KROW * 4;
+    static constexpr int SC = UB + T::UB_BYTES;
+    static constexpr int FRONT = SC + T::SC_BYTES;
+    static constexpr int FK = 0;
+    static constexpr int FU = FK + T::MMAX * T::KROW * 4;
+    static constexpr int FC = FU + T::MMAX * T::UROW * 4;
+    static constexpr int FOLD = FC + T::KROW * 4;
+    static constexpr int BYTES = FRONT > FOLD ? FRONT : FOLD;
 };
 
 // LDS position of element e of a d_k vector stored piecewise.
@@ -57,11 +81,11 @@ __device__ __forceinline__ LaneId lane_id() {
 template <class T>
 __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG + l.rg; }
 
-// Which of its RPLP rows a lane owns after reduce_rows: own_first(l) + t, t < NOWN.  Every butterfly level halves
-// the candidate range; the lane whose bit is set takes the upper half.
+// Which row of a block of LPRP a lane owns after the block's reduction.  Every butterfly level halves the candidate
+// range; the lane whose bit is set takes the upper half.
 template <class T>
-__device__ __forceinline__ int own_first(const LaneId& l) {
-    int off = 0, n = T::RPLP;
+__device__ __forceinline__ int own_in_block(const LaneId& l) {
+    int off = 0, n = T::LPRP;
 #pragma unroll
     for (int lv = T::LVL_ROW - 1; lv >= 0; --lv) {
         n >>= 1;
@@ -69,49 +93,44 @@ __device__ __forceinline__ int own_first(const LaneId& l) {
     }
     return off;
 }
-
-// The only read of the stored state: a lane's piece of each of its rows, issued back to back.  Idle lanes (past
-// d_k) load a live lane's piece instead of branching around the load, and zero it afterwards.
+// The head row a lane owns in block b (may lie past d_v in a padded last block: `owned_valid`).
 template <class T>
-__device__ __forceinline__ void load_tile(const uint8_t* head, const LaneId& l, RawRow<T::BITS> (&raw)[T::RPL]) {
-    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
-#pragma unroll
-    for (int j = 0; j < T::RPL; ++j)
-        raw[j] = load_row<T::BITS>(head + size_t(row_of<T>(l, j)) * T::ROW_BYTES + cc * T::LANE_BYTES);
+__device__ __forceinline__ int owned_row(const LaneId& l, int b) {
+    return row_of<T>(l, b * T::LPRP + own_in_block<T>(l));
 }
 template <class T>
-__device__ __forceinline__ void mask_tile(const LaneId& l, RawRow<T::BITS> (&raw)[T::RPL]) {
-    if constexpr (T::LPR < T::LPRP) {
-        const bool live = l.cg < T::LPR;
-        const RawRow<T::BITS> z = zero_row<T::BITS>();
+__device__ __forceinline__ bool owned_valid(const LaneId& l, int b) {
+    return b * T::LPRP + own_in_block<T>(l) < T::RPL;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// coalesced staging of a small byte range into LDS: lane i carries bytes [16 i + 1024 c, +16) of it
+// ---------------------------------------------------------------------------------------------------------------
+template <int MAXBYTES>
+struct Staged {
+    static constexpr int N = (MAXBYTES + 1023) / 1024;
+    uint4 v[N];
+};
+template <int MAXBYTES>
+__device__ __forceinline__ void stage_load(const uint8_t* src, int nbytes, int lane, Staged<MAXBYTES>& s) {
 #pragma unroll
-        for (int j = 0; j < T::RPL; ++j) {
-            raw[j].v.x = live ? raw[j].v.x : z.v.x;
-            raw[j].v.y = live ? raw[j].v.y : z.v.y;
-            if constexpr (T::BITS == 8) {
-                raw[j].v.z = live ? raw[j].v.z : z.v.z;
-                raw[j].v.w = live ? raw[j].v.w : z.v.w;
-            }
-        }
+    for (int c = 0; c < Staged<MAXBYTES>::N; ++c) {
+        const int off = lane * 16 + c * 1024;
+        s.v[c] = *reinterpret_cast<const uint4*>(src + (off < nbytes ? off : 0));      // clamped, never branched
+    }
+}
+template <int MAXBYTES>
+__device__ __forceinline__ void stage_store(uint8_t* lds, int nbytes, int lane, const Staged<MAXBYTES>& s) {
+#pragma unroll
+    for (int c = 0; c < Staged<MAXBYTES>::N; ++c) {
+        const int off = lane * 16 + c * 1024;
+        if (off < nbytes) *reinterpret_cast<uint4*>(lds + off) = s.v[c];
     }
 }
 
-// The raw fp16 scale of (row j, this lane's key group) for every row of the lane; scale_value() turns it into fp32
-// (0 for lanes whose group lies past d_k).
-template <class T>
-__device__ __forceinline__ void load_scales(const uint16_t* sc_head, const LaneId& l, uint16_t (&sc)[T::RPL]) {
-    int gi = (l.cg * CPL) / T::GROUP;
-    gi = gi < T::NG ? gi : T::NG - 1;
-#pragma unroll
-    for (int j = 0; j < T::RPL; ++j) sc[j] = sc_head[size_t(row_of<T>(l, j)) * T::NG + gi];
-}
-template <class T>
-__device__ __forceinline__ void scale_values(const uint16_t (&raw)[T::RPL], const LaneId& l, float (&sc)[T::RPL]) {
-    const bool ok = (l.cg * CPL) / T::GROUP < T::NG;
-#pragma unroll
-    for (int j = 0; j < T::RPL; ++j) sc[j] = ok ? f16_to_f32(raw[j]) : 0.0f;
-}
-
+// ---------------------------------------------------------------------------------------------------------------
+// cross-lane reduction of one block of LPRP rows
+// ---------------------------------------------------------------------------------------------------------------
 // A small register vector passed by value, so that selects between its elements stay selects (an array passed by
 // reference would let the optimizer turn `c ? p[a] : p[b]` into a dynamically indexed load from scratch memory).
 template <int N>
@@ -119,64 +138,98 @@ struct FVec {
     float v[N];
 };
 
-// Butterfly levels LV .. 0 over N row sums.  Levels at or above the scale-group size reduce-scatter (the lane whose
-// bit is clear keeps the lower half and adds the partner's lower half); below it the lanes of a group already hold
-// equal values and each just takes its share.  N halves per level; RPLP values end as NOWN.
-template <class T, int LV, int N>
+// Butterfly levels LV .. 0 over N values.  Levels >= GRP reduce-scatter (the lane whose bit is clear keeps the lower
+// half and adds the partner's lower half); below GRP the lanes already hold equal values and each takes its share.
+template <int GRP, int LV, int N>
 __device__ __forceinline__ FVec<(N >> (LV + 1))> butterfly(FVec<N> p, int cg) {
     const bool hi = (cg >> LV) & 1;
     FVec<N / 2> o;
 #pragma unroll
     for (int t = 0; t < N / 2; ++t) {
         const float lo_v = p.v[t], hi_v = p.v[N / 2 + t];
-        if constexpr (LV >= T::LVL_GRP) o.v[t] = (hi ? hi_v : lo_v) + partner<LV>(hi ? lo_v : hi_v);
+        if constexpr (LV >= GRP) o.v[t] = (hi ? hi_v : lo_v) + partner<LV>(hi ? lo_v : hi_v);
         else o.v[t] = hi ? hi_v : lo_v;
     }
-    if constexpr (LV > 0) return butterfly<T, LV - 1, N / 2>(o, cg);
+    if constexpr (LV > 0) return butterfly<GRP, LV - 1, N / 2>(o, cg);
     else return o;
 }
 
-// Per-lane partial row sums p[v][j] (this lane's 16 columns of row j against read-out vector v) -> full row sums of
-// the rows the lane owns.  Inside a key group the partial sums are added first and multiplied by the group's scale,
+// Partial sums p[t] (this lane's 16 columns of block row t against one read-out vector) -> the full, scaled row sum
+// of the row the lane owns.  Inside a key group the partial sums are added first and multiplied by the group's scale,
 // then the scaled group sums are added across the row (the reference's "(group sum) x scale, group by group",
-// _fold_triton.py:191-196, here in a fixed butterfly order).
-template <class T, int NV>
-__device__ __forceinline__ void reduce_rows(const float (&p)[NV][T::RPLP], const float (&sc)[T::RPL],
-                                            const LaneId& l, float (&own)[NV][T::NOWN]) {
+// _fold_triton.py:191-196, here in a fixed butterfly order).  sc_lds: the head's raw fp16 scales [row][group].
+template <class T>
+__device__ __forceinline__ float reduce_block(FVec<T::LPRP> p, int b, const uint16_t* sc_lds, const LaneId& l) {
+    const int gi = (l.cg * CPL) / T::GROUP;
+    const bool has_group = gi < T::NG;
+    if constexpr (T::LPG == T::LPRP) {                      // one group per row: reduce first, scale the owned row
+        const FVec<1> o = butterfly<0, T::LVL_ROW - 1, T::LPRP>(p, l.cg);
+        int r = owned_row<T>(l, b);
+        r = r < T::DV ? r : T::DV - 1;
+        return o.v[0] * f16_to_f32(sc_lds[r * T::NG]);
+    } else {
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-        FVec<T::RPLP> g;
-#pragma unroll
-        for (int j = 0; j < T::RPLP; ++j) {
-            if (j < T::RPL) g.v[j] = block_sum<T::LPG>(p[v][j]) * sc[j < T::RPL ? j : 0];
-            else g.v[j] = 0.0f;
+        for (int t = 0; t < T::LPRP; ++t) {
+            int r = row_of<T>(l, b * T::LPRP + t);
+            r = r < T::DV ? r : T::DV - 1;
+            const float s = has_group ? f16_to_f32(sc_lds[r * T::NG + (has_group ? gi : 0)]) : 0.0f;
+            p.v[t] = block_sum<T::LPG>(p.v[t]) * s;
         }
-        const FVec<T::NOWN> o = butterfly<T, T::LVL_ROW - 1, T::RPLP>(g, l.cg);
-#pragma unroll
-        for (int t = 0; t < T::NOWN; ++t) own[v][t] = o.v[t];
+        return butterfly<T::LVL_GRP, T::LVL_ROW - 1, T::LPRP>(p, l.cg).v[0];
     }
 }
 
-// Row dot products of the whole tile against NV read-out vectors whose 16-column pieces sit in x[v][].
+// ---------------------------------------------------------------------------------------------------------------
+// the streaming pass over the stored codes
+// ---------------------------------------------------------------------------------------------------------------
+template <class T>
+struct Window {
+    RawRow<T::BITS> row[T::LPRP];
+};
+template <class T>
+__device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
+    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
+    return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
+}
+// Issue the loads of block 0.
+template <class T>
+__device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
+#pragma unroll
+    for (int t = 0; t < T::LPRP; ++t)
+        if (t < T::RPL) w.row[t] = load_row<T::BITS>(lane_base + t * (T::RG * T::ROW_BYTES));
+}
+// Row dot products of the whole tile against NV read-out vectors (16-column pieces in x[v][]), block by block; the
+// window row just consumed is refilled with the same row of the next block.  own[v][b] = S0 x_v at the row the lane
+// owns in block b.
 template <class T, int NV>
-__device__ __forceinline__ void tile_dots(const RawRow<T::BITS> (&raw)[T::RPL], const float (&x)[NV][CPL],
-                                          float (&p)[NV][T::RPLP]) {
+__device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, const float (&x)[NV][CPL],
+                                           const uint16_t* sc_lds, const LaneId& l, float (&own)[NV][T::NOWN]) {
+    const bool live = l.cg < T::LPR;
 #pragma unroll
-    for (int j = 0; j < T::RPLP; ++j) {
-        if (j < T::RPL) {
-            float c[CPL];
-            decode_row<T::BITS>(raw[j], c);
+    for (int b = 0; b < T::NOWN; ++b) {
+        FVec<T::LPRP> p[NV];
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                float s = c[0] * x[v][0];
+        for (int t = 0; t < T::LPRP; ++t) {
+            const int j = b * T::LPRP + t;
+            if (j < T::RPL) {
+                float c[CPL];
+                decode_row<T::BITS>(w.row[t], c);
+                if (j + T::LPRP < T::RPL)
+                    w.row[t] = load_row<T::BITS>(lane_base + (j + T::LPRP) * (T::RG * T::ROW_BYTES));
 #pragma unroll
-                for (int t = 1; t < CPL; ++t) s = __builtin_fmaf(c[t], x[v][t], s);
-                p[v][j] = s;
+                for (int v = 0; v < NV; ++v) {
+                    float s = c[0] * x[v][0];
+#pragma unroll
+                    for (int k = 1; k < CPL; ++k) s = __builtin_fmaf(c[k], x[v][k], s);
+                    p[v].v[t] = live ? s : 0.0f;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < NV; ++v) p[v].v[t] = 0.0f;
             }
-        } else {
-#pragma unroll
-            for (int v = 0; v < NV; ++v) p[v][j] = 0.0f;
         }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) own[v][b] = reduce_block<T>(p[v], b, sc_lds, l);
     }
 }
 
@@ -192,8 +245,8 @@ __device__ __forceinline__ void lds_piece(const float* vec, int cg, float (&x)[C
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// the decode buffer.  All loads below are unconditional (indices clamped into the live range) so that they can be
-// issued back to back ahead of the state tile; dead slots and idle lanes are masked after the fact with selects.
+// the decode buffer.  Loads are unconditional (indices clamped into the live range) so that they can be issued back
+// to back ahead of the state tile; dead slots and idle lanes are masked after the fact with selects.
 // ---------------------------------------------------------------------------------------------------------------
 template <class T>
 struct BufAddr {                       // one (sequence, head)'s buffer fields
@@ -203,26 +256,11 @@ struct BufAddr {                       // one (sequence, head)'s buffer fields
     uint16_t* UBS;                     // [m] fp16 (int8 buffer)
 };
 
-// Raw delta values of the rows this lane owns, every slot: ub[i][t] = UB[min(i, m-1)][row t].
+// Buffered value (slot i, head row r) from the raw copy in LDS.
 template <class T>
-__device__ __forceinline__ void load_ub(const uint8_t* UB, int m, const LaneId& l, int jown,
-                                        int32_t (&ub)[T::MMAX][T::NOWN]) {
-#pragma unroll
-    for (int i = 0; i < T::MMAX; ++i) {
-        const int ic = i < m ? i : m - 1;
-#pragma unroll
-        for (int t = 0; t < T::NOWN; ++t) {
-            int r = row_of<T>(l, jown + t);
-            r = r < T::DV ? r : T::DV - 1;
-            if constexpr (T::QBUF) ub[i][t] = reinterpret_cast<const int8_t*>(UB)[ic * T::DV + r];
-            else ub[i][t] = reinterpret_cast<const uint16_t*>(UB)[ic * T::DV + r];
-        }
-    }
-}
-template <class T>
-__device__ __forceinline__ float ub_value(int32_t raw) {
-    if constexpr (T::QBUF) return float(raw);
-    else return bf16_to_f32(uint16_t(raw));
+__device__ __forceinline__ float ub_lds(const uint8_t* ub_lds_, int i, int r) {
+    if constexpr (T::QBUF) return float(reinterpret_cast<const int8_t*>(ub_lds_)[i * T::DV + r]);
+    else return bf16_to_f32(reinterpret_cast<const uint16_t*>(ub_lds_)[i * T::DV + r]);
 }
 
 // A lane's 16-column piece of one buffered key, raw.
@@ -293,12 +331,11 @@ __device__ __forceinline__ void load_keybuf(const BufAddr<T>& a, int m, const La
 }
 
 // Buffer coefficients for scalar decays (GDN, Mamba2): c[v][i] = exp(gcur - G_i) (K_i . x_v) for slots i < n, else 0
-// (reference `_coefs`, _fold_triton.py:260-272).  `gb` = the lane's slots' G (one per pass).  When the buffer is
-// about to be folded the dequantized keys of slots 0 .. m-2 are staged in LDS for the fold.
+// (reference `_coefs`, _fold_triton.py:260-272).  `gb` = the lane's slots' G (one per pass).
 template <class T, int NV>
 __device__ __forceinline__ void buffer_coefs(const KeyBuf<T>& kbuf, const float (&gb)[KeyBuf<T>::KT], float gcur,
-                                             int n, int m, bool full, const float (&x)[NV][CPL], const LaneId& l,
-                                             float* lds_k, float (&c)[NV][T::MMAX]) {
+                                             int n, const float (&x)[NV][CPL], const LaneId& l,
+                                             float (&c)[NV][T::MMAX]) {
     constexpr int KT = KeyBuf<T>::KT;
     float cl[NV][KT];
 #pragma unroll
@@ -313,9 +350,8 @@ __device__ __forceinline__ void buffer_coefs(const KeyBuf<T>& kbuf, const float 
 #pragma unroll
             for (int k = 1; k < CPL; ++k) p = __builtin_fmaf(kb[k], x[v][k], p);
             p = block_sum<T::LPRP>(p);
-            cl[v][t] = i < n ? dec * p : 0.0f;
+            cl[v][t] = i < n ? dec * p : 0.0f;               // dead slots may hold anything: select, never multiply
         }
-        if (full && i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
     }
 #pragma unroll
     for (int v = 0; v < NV; ++v)
@@ -327,19 +363,19 @@ __device__ __forceinline__ void buffer_coefs(const KeyBuf<T>& kbuf, const float 
 // bf16.  ur = the value as stored, dequantized (what the fold must use for slot n).
 template <class T>
 __device__ __forceinline__ void append_values(const float (&u)[T::NOWN], float us, const BufAddr<T>& a, int n,
-                                              const LaneId& l, int jown, float (&ur)[T::NOWN]) {
+                                              const LaneId& l, float (&ur)[T::NOWN]) {
     if (T::QBUF && l.lane == 0) a.UBS[n] = f32_to_f16(us);
 #pragma unroll
-    for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
-        const bool valid = jown + t < T::RPL;
+    for (int b = 0; b < T::NOWN; ++b) {
+        const int r = owned_row<T>(l, b);
+        const bool valid = owned_valid<T>(l, b);
         if constexpr (T::QBUF) {
-            const float c = round_buf(u[t], us);
-            ur[t] = c * us;
+            const float c = round_buf(u[b], us);
+            ur[b] = c * us;
             if (valid) reinterpret_cast<int8_t*>(a.UB)[n * T::DV + r] = int8_t(int(c));
         } else {
-            const uint16_t hb = f32_to_bf16(u[t]);
-            ur[t] = bf16_to_f32(hb);
+            const uint16_t hb = f32_to_bf16(u[b]);
+            ur[b] = bf16_to_f32(hb);
             if (valid) reinterpret_cast<uint16_t*>(a.UB)[n * T::DV + r] = hb;
         }
     }
@@ -363,29 +399,43 @@ __device__ __forceinline__ void append_key(const float (&kx)[T::NE], float ks, c
         }
     }
 }
-// Stage the fold's value operand: lds_u[i][row] = f_i x U_i[row] for every slot (slot m-1: the value just appended);
-// f_i = the slot's decay ratio held by lane i of `decf` (KDA passes 1).
+
+// ---------------------------------------------------------------------------------------------------------------
+// the fold
+// ---------------------------------------------------------------------------------------------------------------
+// Fold operands, step 1 (before the front end's LDS is overwritten): the buffered values of the rows this lane owns,
+// dequantized, slot by slot.  uo[b][i] = U_i[row b] (slot m-1: the value just appended, `ur`).
 template <class T>
-__device__ __forceinline__ void stage_values(const int32_t (&ub)[T::MMAX][T::NOWN], float ubs_l, float decf,
-                                             const float (&ur)[T::NOWN], int m, const LaneId& l, int jown,
-                                             float* lds_u) {
+__device__ __forceinline__ void fold_fetch_values(const uint8_t* ub_lds_, const float (&ubs)[T::MMAX],
+                                                  const float (&ur)[T::NOWN], int m, const LaneId& l,
+                                                  float (&uo)[T::NOWN][T::MMAX]) {
 #pragma unroll
-    for (int t = 0; t < T::NOWN; ++t) {
-        const int r = row_of<T>(l, jown + t);
+    for (int b = 0; b < T::NOWN; ++b) {
+        int r = owned_row<T>(l, b);
+        r = r < T::DV ? r : T::DV - 1;
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            if (i < m) {
-                float uv = ub_value<T>(ub[i][t]);
-                if constexpr (T::QBUF) uv = uv * lane_bcast(ubs_l, i);
-                if (i == m - 1) uv = ur[t];
-                if (jown + t >= T::RPL) uv = 0.0f;
-                lds_u[i * T::UROW + r] = lane_bcast(decf, i) * uv;
-            }
+            float uv = ub_lds<T>(ub_lds_, i < m ? i : m - 1, r);
+            if constexpr (T::QBUF) uv = uv * ubs[i];
+            uo[b][i] = i == m - 1 ? ur[b] : uv;
         }
     }
 }
+// Step 2: lds_u[i][row] = f[i] x U_i[row] (f = the slot's decay ratio; KDA passes ones).
 template <class T>
-__device__ __forceinline__ void stage_key(const float (&kr)[T::NE], int slot, const LaneId& l, float* lds_k) {
+__device__ __forceinline__ void fold_stage_values(const float (&uo)[T::NOWN][T::MMAX], const float (&f)[T::MMAX],
+                                                  int m, const LaneId& l, float* lds_u) {
+#pragma unroll
+    for (int b = 0; b < T::NOWN; ++b) {
+        const int r = owned_row<T>(l, b);
+        const bool valid = owned_valid<T>(l, b);
+#pragma unroll
+        for (int i = 0; i < T::MMAX; ++i)
+            if (i < m) lds_u[i * T::UROW + r] = valid ? f[i] * uo[b][i] : 0.0f;
+    }
+}
+template <class T>
+__device__ __forceinline__ void fold_stage_key(const float (&kr)[T::NE], int slot, const LaneId& l, float* lds_k) {
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
         const int e = l.lane + WAVE * t;
@@ -393,33 +443,46 @@ __device__ __forceinline__ void stage_key(const float (&kr)[T::NE], int slot, co
     }
 }
 
-// The fold: S = colmul * S_0 + sum_i du_i (x) kx_i over all m buffer slots in slot order, re-quantized in place
+// The fold proper: S = colmul * S_0 + sum_i du_i (x) kx_i over all m buffer slots in slot order, re-quantized in place
 // (reference: _fused_triton.py:278-394 `_fold_head`; KDA _kda_triton.py:217-316; Mamba2 _mamba2_triton.py:213-332).
 //   lds_k   [m][KROW]   the folded keys kx_i (GDN / Mamba2: the buffered keys; KDA: keys times their decay ratio)
 //   lds_u   [m][UROW]   the folded values du_i (GDN / Mamba2: decay ratio x delta value; KDA: delta value)
-//   colmul  this lane's 16 column factors on the dequantized old state (GDN / Mamba2: exp(G_m) in every column)
-// Four rows per lane are in flight at a time; the register-resident rows are rotated down between rounds so that
-// the loop stays rolled.  Each lane rewrites exactly the codes it read; the lowest lane of a key group stores the
-// group's scale.  Codes are rint(S / scale) with the exact quotient wherever the reciprocal product is within
-// |q| 2^-22 of a rounding boundary (rint_quot_fast / the wave-uniform exact pass).
-template <class T>
-__device__ __forceinline__ void fold_tile(RawRow<T::BITS> (&raw)[T::RPL], float (&sc)[T::RPL],
-                                          const float (&colmul)[CPL], const float* lds_k, const float* lds_u, int m,
+//   lds_c   [KROW]      COLVEC: per-column factors on the dequantized old state (KDA);  else the scalar `cmul`
+//                       (GDN / Mamba2: exp(G_m))
+// The codes and scales are read again from memory, four rows per lane at a time.  Each lane rewrites exactly the codes
+// it read; the lowest lane of a key group stores the group's scale.  Codes are rint(S x (1/scale)) with the correctly
+// rounded reciprocal: against rint(S / scale) that moves a code by one step only where the quotient lies within
+// |q| 2^-24 of a rounding boundary (a few codes per million, the same order as the accumulation-order mismatches).
+template <class T, bool COLVEC>
+__device__ __forceinline__ void fold_tile(const float* lds_k, const float* lds_u, const float* lds_c, float cmul, int m,
                                           uint8_t* head, uint16_t* sc_head, const LaneId& l) {
     constexpr int FR = 4;
     const bool live = l.cg < T::LPR;
-    const int gi = (l.cg * CPL) / T::GROUP;
-    const bool lead = live && (l.cg % T::LPG) == 0 && gi < T::NG;
-    const float margin = 0.5f - (T::QMAX + 2.0f) * 2.384185791015625e-07f;      // 2^-22
+    int gi = (l.cg * CPL) / T::GROUP;
+    const bool has_group = gi < T::NG;
+    gi = has_group ? gi : T::NG - 1;
+    const bool lead = live && (l.cg % T::LPG) == 0 && has_group;
+    uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
+    float colmul[COLVEC ? CPL : 1];
+    if constexpr (COLVEC) lds_piece<T>(lds_c, l.cg, colmul);
+    else colmul[0] = cmul;
 #pragma unroll 1
     for (int j0 = 0; j0 < T::RPL; j0 += FR) {
+        RawRow<T::BITS> raw[FR];
+        uint16_t scr[FR];
+#pragma unroll
+        for (int jj = 0; jj < FR; ++jj) {
+            raw[jj] = load_row<T::BITS>(lane_base + (j0 + jj) * (T::RG * T::ROW_BYTES));
+            scr[jj] = sc_head[row_of<T>(l, j0 + jj) * T::NG + gi];
+        }
         float acc[FR][CPL];
 #pragma unroll
         for (int jj = 0; jj < FR; ++jj) {
             float c[CPL];
             decode_row<T::BITS>(raw[jj], c);
+            const float s = (live && has_group) ? f16_to_f32(scr[jj]) : 0.0f;
 #pragma unroll
-            for (int t = 0; t < CPL; ++t) acc[jj][t] = (c[t] * sc[jj]) * colmul[t];
+            for (int t = 0; t < CPL; ++t) acc[jj][t] = (c[t] * s) * colmul[COLVEC ? t : 0];
         }
 #pragma unroll 1
         for (int i = 0; i < m; ++i) {
@@ -441,28 +504,10 @@ __device__ __forceinline__ void fold_tile(RawRow<T::BITS> (&raw)[T::RPL], float 
             const float s = fp16_scale(amax, T::QMAX);
             const float r = 1.0f / s;
             const int row = row_of<T>(l, j0 + jj);
-            if (lead) sc_head[size_t(row) * T::NG + gi] = f32_to_f16(s);
-            float q[CPL];
-            bool near = false;
-#pragma unroll
-            for (int t = 0; t < CPL; ++t) {
-                const float qq = acc[jj][t] * r;
-                const float c = rintf(qq);
-                near |= fabsf(qq - c) >= margin;
-                q[t] = c;
-            }
-            if (__builtin_amdgcn_ballot_w64(near) != 0) {          // some lane sits next to a rounding boundary
-#pragma unroll
-                for (int t = 0; t < CPL; ++t) q[t] = rintf(acc[jj][t] / s);
-            }
-#pragma unroll
-            for (int t = 0; t < CPL; ++t) q[t] = fminf(fmaxf(q[t], -T::QMAX), T::QMAX);
-            if (live) store_row<T::BITS>(head + size_t(row) * T::ROW_BYTES + l.cg * T::LANE_BYTES,
-                                         encode_row<T::BITS>(q));
+            if (lead) sc_head[row * T::NG + gi] = f32_to_f16(s);
+            if (live)
+                store_row<T::BITS>(lane_base + (j0 + jj) * (T::RG * T::ROW_BYTES), quantize_row<T::BITS>(acc[jj], r));
         }
-        // rotate the remaining rows into place for the next round
-#pragma unroll
-        for (int j = 0; j + FR < T::RPL; ++j) { raw[j] = raw[j + FR]; sc[j] = sc[j + FR]; }
     }
 }
 
