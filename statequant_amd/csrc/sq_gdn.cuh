@@ -3,8 +3,9 @@
 // Replaces the reference's fused Triton step (/root/reference/src/statequant/kernels/_fused_triton.py:48-190) with
 // the same arithmetic per head:
 //   prep     q, k l2-normalised (eps inside the sqrt), the gates, c_q[i] = (a_n/a_i) k_i.q, c_k[i] likewise
-//   state    the stored codes streamed once through a register window; S0 q, S0 k by 16-column pieces + butterfly
-//            reduction; buffer term as a slot-ordered fma chain; u = beta (v - a sk), o = a sq + (k.q) u
+//   state    the stored codes streamed once through a register window; S0 q, S0 k as integer dot products against
+//            fixed-point digit planes of q, k; buffer term as a slot-ordered fma chain; u = beta (v - a sk),
+//            o = a sq + (k.q) u
 //   append   G_n, the delta value (int8 with one absmax scale over the row, or bf16), the key (first head of a
 //            GQA group only)
 //   fold     buffer full: S = a_m S0 + sum_i (a_m/a_i) u_i k_i^T, re-quantized in place
@@ -108,7 +109,7 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
         r = r < DV ? r : DV - 1;
         f.vr[t] = load_raw(p.v, p.v_dt, int64_t(a.b) * p.s_v + int64_t(a.h) * DV + r);
     }
-    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
+    window_init<T>(lane_codes_m<T>(a.Sh, l), f.win);
 }
 
 template <class T>
@@ -119,6 +120,10 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     float* lds_kn = lds_q + T::KROW;
     uint8_t* lds_ub = lds + L::UB;
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    uint8_t* lds_b = lds + L::B;
+    float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
+    float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);          // the fold's operands overlay the above
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     const int h = A.h;
     const int n = F.n;
     const float gcur = F.gcur;
-    const uint8_t* lane_base = lane_codes<T>(A.Sh, l);
+    const uint8_t* lane_base = lane_codes_m<T>(A.Sh, l);
 
     // ---- prep: q, k (fla's l2 normalisation), gates ----
     const bool full = n == m - 1;
@@ -165,6 +170,12 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         kqp = __builtin_fmaf(ke[t], qe[t], kqp);
         const int e = l.lane + WAVE * t;
         if (e < T::LPRP * CPL) { lds_q[kpos<T>(e)] = qe[t]; lds_kn[kpos<T>(e)] = ke[t]; }
+    }
+    {
+        float xe[2][T::NE];
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) { xe[0][t] = qe[t]; xe[1][t] = ke[t]; }
+        stage_planes<T, 2>(xe, l, lds_b, lds_xs);
     }
     stage_store(lds_ub, m * DV * T::BE, l.lane, F.st_ub);
     stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, F.st_sc);
@@ -204,7 +215,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
 
     // ---- state pass ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, F.win, x, lds_sc, l, own);
+    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_c, lds_own, l, own);
 
     const KeyBuf<T>& kbuf = F.kbuf;
     const float gb_lane = F.gb_lane;

@@ -16,15 +16,17 @@ namespace sq {
 
 template <class T>
 __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
-    using L = LdsPlan<T, 5>;                                      // q, k (normalised), A*q, A*k, G_n
+    using L = LdsPlan<T, 3, 2>;                                   // q, k (normalised), G_n
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_q = reinterpret_cast<float*>(lds + L::X);
     float* lds_kn = lds_q + T::KROW;
-    float* lds_qa = lds_kn + T::KROW;
-    float* lds_ka = lds_qa + T::KROW;
-    float* lds_g = lds_ka + T::KROW;
+    float* lds_g = lds_kn + T::KROW;
     uint8_t* lds_ub = lds + L::UB;
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    uint8_t* lds_b = lds + L::B;
+    float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    int32_t* lds_ci = reinterpret_cast<int32_t*>(lds + L::C);
+    float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
     float* lds_c = reinterpret_cast<float*>(lds + L::FC);
@@ -54,7 +56,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m * DK;
     float* gch = p.st.GCUR + seq * p.st.sGC + int64_t(h) * DK;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const uint8_t* lane_base = lane_codes<T>(Sh, l);
+    const uint8_t* lane_base = lane_codes_m<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
     // ---- issue every load ----
@@ -114,22 +116,24 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     const float nq = sqrtf(wave_sum(ssq) + 1e-6f);
     const float nk = sqrtf(wave_sum(ssk) + 1e-6f);
     float kqp = 0.0f;
+    float xa[2][T::NE];                                           // A * q, A * k: what the stored state is read against
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
         qe[t] = qe[t] / nq * p.scale;
         ke[t] = ke[t] / nk;
         kqp = __builtin_fmaf(ke[t], qe[t], kqp);
         const int e = l.lane + WAVE * t;
+        const float A = e < DK ? expf(gn[t]) : 0.0f;
+        xa[0][t] = A * qe[t];
+        xa[1][t] = A * ke[t];
         if (e < T::LPRP * CPL) {
-            const float A = e < DK ? expf(gn[t]) : 0.0f;
             const int pos = kpos<T>(e);
             lds_q[pos] = qe[t];
             lds_kn[pos] = ke[t];
-            lds_qa[pos] = A * qe[t];
-            lds_ka[pos] = A * ke[t];
             lds_g[pos] = gn[t];
         }
     }
+    stage_planes<T, 2>(xa, l, lds_b, lds_xs);
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
     stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
     const float kq = wave_sum(kqp);
@@ -177,12 +181,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
 
     // ---- state pass against A*q, A*k ----
     float own[2][T::NOWN];
-    {
-        float x[2][CPL];
-        lds_piece<T>(lds_qa, l.cg, x[0]);
-        lds_piece<T>(lds_ka, l.cg, x[1]);
-        state_pass<T, 2>(lane_base, win, x, lds_sc, l, own);
-    }
+    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_ci, lds_own, l, own);
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll

@@ -14,11 +14,15 @@ namespace sq {
 
 template <class T>
 __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params p) {
-    using L = LdsPlan<T, 1>;
+    using L = LdsPlan<T, 1, 1>;
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_cv = reinterpret_cast<float*>(lds + L::X);
     uint8_t* lds_ub = lds + L::UB;
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
+    uint8_t* lds_b = lds + L::B;
+    float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
+    float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
@@ -49,7 +53,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
     float* gcp = p.st.GCUR + seq * p.st.sGC + h;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const uint8_t* lane_base = lane_codes<T>(Sh, l);
+    const uint8_t* lane_base = lane_codes_m<T>(Sh, l);
 
     // ---- issue every load ----
     const int n = *np & (m - 1);
@@ -101,6 +105,12 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         bcp = __builtin_fmaf(kxe[t], ce[t], bcp);
         if (e < T::LPRP * CPL) lds_cv[kpos<T>(e)] = ce[t];
     }
+    {
+        float xe[1][T::NE];
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) xe[0][t] = ce[t];
+        stage_planes<T, 1>(xe, l, lds_b, lds_xs);
+    }
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
     stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
     const float bc = wave_sum(bcp);
@@ -126,7 +136,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
 
     // ---- state pass ----
     float own[1][T::NOWN];
-    state_pass<T, 1>(lane_base, win, x, lds_sc, l, own);
+    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_c, lds_own, l, own);
 
     // ---- owned rows: y, and the value to buffer ----
     float u[T::NOWN], amax = 0.0f;

@@ -1,12 +1,22 @@
 // The state tile of one (sequence, value head) in one wavefront: geometry, the streaming read of the stored codes
-// with the row dot products and their cross-lane reduction, the decode buffer, and the fold (advance across the
-// full buffer + re-quantize in place).  Shared by the Gated DeltaNet, KDA and Mamba2 step kernels.
+// with the row dot products, the decode buffer, and the fold (advance across the full buffer + re-quantize in
+// place).  Shared by the Gated DeltaNet, KDA and Mamba2 step kernels.
 //
-// Resource plan (what keeps four wavefronts per SIMD resident): the codes stream through a window of LPRP rows per
-// lane (32 VGPRs for int8), refilled row by row; the small operands (buffered values, scales) are fetched with one
-// coalesced 128-bit load per lane and parked in LDS until needed; the fold reads the codes a second time (from L2 /
-// Infinity Cache: they were read microseconds earlier) instead of pinning them in registers; the fold's LDS
-// operands overlay the front end's.
+// Row dot products.  S0 x (x = q, k, ...) over int8 / int4 codes is an integer dot product per row and scale group
+// once x is in fixed point.  x is cut, per scale group, into three signed 8-bit digits of a 23-bit fixed-point
+// number (exponent = that of the group's largest |x|), and the codes meet the digit planes in the matrix core's
+// int8 dot-product instruction (v_mfma_i32_32x32x32_i8: 32 rows x 32 columns of codes against up to 32 planes per
+// issue, int32 accumulation, exact).  A vector-ALU formulation (convert every code to fp32, one fma per code and
+// vector) costs ~50 instructions per 16-code row piece and made the step ALU-bound at under half the HBM rate; the
+// matrix core takes the codes as loaded (int8) or after a nibble split (int4) and leaves the vector ALU to the
+// per-row work.  The digits' rounding (|x| 2^-23 of the group maximum per element) is of the order of fp32
+// accumulation error.
+//
+// Resource plan (what keeps four wavefronts per SIMD resident): the codes stream through a window of two 32-row
+// blocks per wavefront (32 VGPRs for int8), refilled block by block; the small operands (buffered values, scales)
+// are fetched with one coalesced 128-bit load per lane and parked in LDS until needed; the fold reads the codes a
+// second time (from L2 / Infinity Cache: they were read microseconds earlier) instead of pinning them in registers;
+// the fold's LDS operands overlay the front end's.
 #pragma once
 #include "sq_device.cuh"
 
@@ -14,8 +24,8 @@ namespace sq {
 
 // Compile-time geometry.  A row of DK codes is cut into DK/16 pieces of 16 columns; LPRP (that count rounded up to a
 // power of two) consecutive lanes hold one row, lanes past DK/16 idle (d_k = 96: 6 of 8).  The wavefront therefore
-// covers RG = 64/LPRP rows per load and a lane sees rows rg, rg + RG, rg + 2 RG, ...  Rows are handled in blocks of
-// LPRP per lane (one reduce-scatter each), after which every lane owns one row of the block.
+// covers RG = 64/LPRP rows per load and a lane sees rows rg, rg + RG, rg + 2 RG, ...  (the fold and the buffer passes
+// use this shape; the state pass uses the matrix core's, below).
 template <int BITS_, int DK_, int DV_, int GROUP_, bool QBUF_, int MMAX_>
 struct Tile {
     static constexpr int BITS = BITS_, DK = DK_, DV = DV_, GROUP = GROUP_, MMAX = MMAX_;
@@ -26,14 +36,11 @@ struct Tile {
     static constexpr int LPRP = pow2_ceil(LPR);           // lanes per row incl. idle ones
     static constexpr int RG = WAVE / LPRP;                // rows per wavefront load
     static_assert(DV % (4 * RG) == 0, "d_v must be a multiple of 4 x the rows one wavefront load covers");
-    static constexpr int RPL = DV / RG;                   // rows per lane
-    static constexpr int NOWN = (RPL + LPRP - 1) / LPRP;  // row blocks per lane = rows a lane owns
-    static constexpr int RPLP = NOWN * LPRP;              // rows per lane, padded to whole blocks
+    static constexpr int RPL = DV / RG;                   // rows per lane (fold, buffer passes)
+    static constexpr int NOWN = (DV + WAVE - 1) / WAVE;   // rows a lane owns after the state pass: lane + 64 t
     static constexpr int NG = (DK + GROUP - 1) / GROUP;   // stored key groups per row (last may be ragged)
     static_assert(GROUP % CPL == 0 && GROUP >= CPL, "key group must be a multiple of 16");
     static constexpr int LPG = (GROUP / CPL < LPRP) ? GROUP / CPL : LPRP;   // lanes sharing one scale
-    static constexpr int LVL_ROW = ilog2(LPRP);           // butterfly levels across a row
-    static constexpr int LVL_GRP = ilog2(LPG);            // ... of which inside one scale group
     static constexpr int ROW_BYTES = BITS == 4 ? DK / 2 : DK;
     static constexpr int LANE_BYTES = BITS == 4 ? CPL / 2 : CPL;
     static constexpr float QMAX = float((1 << (BITS - 1)) - 1);
@@ -41,19 +48,31 @@ struct Tile {
     static constexpr int BE = QBUF ? 1 : 2;               // bytes per buffer element (int8 / bf16)
     static constexpr int KPAD = CPL + 4;                  // LDS stride of a 16-column piece (spreads the banks)
     static constexpr int KROW = LPRP * KPAD;              // floats per d_k vector in LDS
-    static constexpr int UROW = RPLP * RG;                // floats per d_v vector in LDS
+    static constexpr int UROW = NOWN * WAVE;              // floats per d_v vector in LDS
+    // matrix-core pass: blocks of MR rows x MK columns (one lane: one row, 16 columns; lanes 32.. the next 16)
+    static constexpr int MR = 32, MK = 32;
+    static_assert(DV % MR == 0 && DK % MK == 0 && GROUP % MK == 0, "tile / group must be multiples of 32");
+    static constexpr int NRB = DV / MR;                   // row blocks
+    static constexpr int NKS = DK / MK;                   // column steps
+    static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
+    static constexpr int B_BYTES = (DK / CPL) * 8 * CPL;  // digit planes: [16-column piece][8 planes][16]
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
     static constexpr int SC_BYTES = round_up(DV * NG * 2, 16);
 };
 
-// LDS plan of a step kernel that stages NX d_k vectors.  Front end: the vectors, the raw buffered values, the raw
-// scales.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
-template <class T, int NX>
+// LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
+// vectors, the raw buffered values, the raw scales, the digit planes with their exponents, one row block's integer
+// sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
+template <class T, int NX, int NV = 2>
 struct LdsPlan {
     static constexpr int X = 0;
     static constexpr int UB = X + NX * T::KROW * 4;
     static constexpr int SC = UB + T::UB_BYTES;
-    static constexpr int FRONT = SC + T::SC_BYTES;
+    static constexpr int B = SC + T::SC_BYTES;
+    static constexpr int XS = B + T::B_BYTES;
+    static constexpr int C = XS + round_up(NV * T::NG * 4, 16);
+    static constexpr int OWN = C + T::NG * T::PLANES * NV * T::MR * 4;
+    static constexpr int FRONT = OWN + NV * T::UROW * 4;
     static constexpr int FK = 0;
     static constexpr int FU = FK + T::MMAX * T::KROW * 4;
     static constexpr int FC = FU + T::MMAX * T::UROW * 4;
@@ -81,27 +100,11 @@ __device__ __forceinline__ LaneId lane_id() {
 template <class T>
 __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG + l.rg; }
 
-// Which row of a block of LPRP a lane owns after the block's reduction.  Every butterfly level halves the candidate
-// range; the lane whose bit is set takes the upper half.
+// The head rows a lane owns after the state pass (epilogue, append, fold staging): lane + 64 t.
 template <class T>
-__device__ __forceinline__ int own_in_block(const LaneId& l) {
-    int off = 0, n = T::LPRP;
-#pragma unroll
-    for (int lv = T::LVL_ROW - 1; lv >= 0; --lv) {
-        n >>= 1;
-        if ((l.cg >> lv) & 1) off += n;
-    }
-    return off;
-}
-// The head row a lane owns in block b (may lie past d_v in a padded last block: `owned_valid`).
+__device__ __forceinline__ int owned_row(const LaneId& l, int t) { return l.lane + WAVE * t; }
 template <class T>
-__device__ __forceinline__ int owned_row(const LaneId& l, int b) {
-    return row_of<T>(l, b * T::LPRP + own_in_block<T>(l));
-}
-template <class T>
-__device__ __forceinline__ bool owned_valid(const LaneId& l, int b) {
-    return b * T::LPRP + own_in_block<T>(l) < T::RPL;
-}
+__device__ __forceinline__ bool owned_valid(const LaneId& l, int t) { return l.lane + WAVE * t < T::DV; }
 
 // ---------------------------------------------------------------------------------------------------------------
 // coalesced staging of a small byte range into LDS: lane i carries bytes [16 i + 1024 c, +16) of it
@@ -129,108 +132,164 @@ __device__ __forceinline__ void stage_store(uint8_t* lds, int nbytes, int lane, 
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// cross-lane reduction of one block of LPRP rows
-// ---------------------------------------------------------------------------------------------------------------
-// A small register vector passed by value, so that selects between its elements stay selects (an array passed by
-// reference would let the optimizer turn `c ? p[a] : p[b]` into a dynamically indexed load from scratch memory).
-template <int N>
-struct FVec {
-    float v[N];
-};
-
-// Butterfly levels LV .. 0 over N values.  Levels >= GRP reduce-scatter (the lane whose bit is clear keeps the lower
-// half and adds the partner's lower half); below GRP the lanes already hold equal values and each takes its share.
-template <int GRP, int LV, int N>
-__device__ __forceinline__ FVec<(N >> (LV + 1))> butterfly(FVec<N> p, int cg) {
-    const bool hi = (cg >> LV) & 1;
-    FVec<N / 2> o;
-#pragma unroll
-    for (int t = 0; t < N / 2; ++t) {
-        const float lo_v = p.v[t], hi_v = p.v[N / 2 + t];
-        if constexpr (LV >= GRP) o.v[t] = (hi ? hi_v : lo_v) + partner<LV>(hi ? lo_v : hi_v);
-        else o.v[t] = hi ? hi_v : lo_v;
-    }
-    if constexpr (LV > 0) return butterfly<GRP, LV - 1, N / 2>(o, cg);
-    else return o;
-}
-
-// Partial sums p[t] (this lane's 16 columns of block row t against one read-out vector) -> the full, scaled row sum
-// of the row the lane owns.  Inside a key group the partial sums are added first and multiplied by the group's scale,
-// then the scaled group sums are added across the row (the reference's "(group sum) x scale, group by group",
-// _fold_triton.py:191-196, here in a fixed butterfly order).  sc_lds: the head's raw fp16 scales [row][group].
-template <class T>
-__device__ __forceinline__ float reduce_block(FVec<T::LPRP> p, int b, const uint16_t* sc_lds, const LaneId& l) {
-    const int gi = (l.cg * CPL) / T::GROUP;
-    const bool has_group = gi < T::NG;
-    if constexpr (T::LPG == T::LPRP) {                      // one group per row: reduce first, scale the owned row
-        const FVec<1> o = butterfly<0, T::LVL_ROW - 1, T::LPRP>(p, l.cg);
-        int r = owned_row<T>(l, b);
-        r = r < T::DV ? r : T::DV - 1;
-        return o.v[0] * f16_to_f32(sc_lds[r * T::NG]);
-    } else {
-#pragma unroll
-        for (int t = 0; t < T::LPRP; ++t) {
-            int r = row_of<T>(l, b * T::LPRP + t);
-            r = r < T::DV ? r : T::DV - 1;
-            const float s = has_group ? f16_to_f32(sc_lds[r * T::NG + (has_group ? gi : 0)]) : 0.0f;
-            p.v[t] = block_sum<T::LPG>(p.v[t]) * s;
-        }
-        return butterfly<T::LVL_GRP, T::LVL_ROW - 1, T::LPRP>(p, l.cg).v[0];
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------------
 // the streaming pass over the stored codes
 // ---------------------------------------------------------------------------------------------------------------
-template <class T>
-struct Window {
-    RawRow<T::BITS> row[T::LPRP];
-};
-template <class T>
-__device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
-    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
-    return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// Byte position, inside a lane's 16-byte matrix operand, of the lane's column c (0..15).  int8: as stored.  int4: the
+// operand is {low nibbles of word 0, high nibbles of word 0, low of word 1, high of word 1}, byte k of a word holding
+// columns 2k and 2k + 1.
+template <int BITS>
+__device__ __forceinline__ int operand_pos(int c) {
+    if constexpr (BITS == 8) return c;
+    else return 4 * (2 * (c / 8) + (c % 2)) + (c % 8) / 2;
 }
-// Issue the loads of block 0.
-template <class T>
-__device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
-#pragma unroll
-    for (int t = 0; t < T::LPRP; ++t)
-        if (t < T::RPL) w.row[t] = load_row<T::BITS>(lane_base + t * (T::RG * T::ROW_BYTES));
+// A lane's codes of one row piece as a matrix operand of 16 signed bytes.  int4: a stored nibble is code + 8; with
+// bit 3 flipped it is the code in 4-bit two's complement, and in the HIGH half of a byte that reads as 16 x code
+// (the pass divides the sums by 16 again, exactly).
+template <int BITS>
+__device__ __forceinline__ v4i operand(const RawRow<BITS>& r) {
+    if constexpr (BITS == 8) {
+        return v4i{int(r.v.x), int(r.v.y), int(r.v.z), int(r.v.w)};
+    } else {
+        const uint32_t w0 = r.v.x ^ 0x88888888u, w1 = r.v.y ^ 0x88888888u;
+        return v4i{int((w0 << 4) & 0xF0F0F0F0u), int(w0 & 0xF0F0F0F0u), int((w1 << 4) & 0xF0F0F0F0u),
+                   int(w1 & 0xF0F0F0F0u)};
+    }
 }
-// Row dot products of the whole tile against NV read-out vectors (16-column pieces in x[v][]), block by block; the
-// window row just consumed is refilled with the same row of the next block.  own[v][b] = S0 x_v at the row the lane
-// owns in block b.
+
+// Read-out vectors -> digit planes.  xe[v][t] = element lane + 64 t of vector v (0 past d_k).  Per vector and scale
+// group: e = exponent of the group's largest |x| (|x| < 2^e), fixed point q = rint(x 2^(22-e)), |q| <= 2^22,
+// q = d0 + 2^8 d1 + 2^16 d2 with signed 8-bit digits.  x 2^(22-e) + 1.5 2^23 (one fma) leaves 2^22 + q in the low
+// mantissa bits; adding the digit bias 0x808080 - 2^22 and flipping the three sign bits yields the digits as bytes.
+// lds_b[piece][plane 3 v + d][operand_pos]: what `state_pass` loads as its second operand;  lds_xs[v][group] =
+// 2^(e-22) (int4: / 16), the factor that turns the integer sums back.
 template <class T, int NV>
-__device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, const float (&x)[NV][CPL],
-                                           const uint16_t* sc_lds, const LaneId& l, float (&own)[NV][T::NOWN]) {
-    const bool live = l.cg < T::LPR;
+__device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const LaneId& l, uint8_t* lds_b,
+                                             float* lds_xs) {
+    constexpr int NBLK = WAVE / 16;
 #pragma unroll
-    for (int b = 0; b < T::NOWN; ++b) {
-        FVec<T::LPRP> p[NV];
+    for (int v = 0; v < NV; ++v) {
+        float mb[T::NE][NBLK];                               // max |x| over each run of 16 columns (wave-uniform)
 #pragma unroll
-        for (int t = 0; t < T::LPRP; ++t) {
-            const int j = b * T::LPRP + t;
-            if (j < T::RPL) {
-                float c[CPL];
-                decode_row<T::BITS>(w.row[t], c);
-                if (j + T::LPRP < T::RPL)
-                    w.row[t] = load_row<T::BITS>(lane_base + (j + T::LPRP) * (T::RG * T::ROW_BYTES));
+        for (int t = 0; t < T::NE; ++t) {
+            const float m16 = block_max<16>(fabsf(xe[v][t]));
 #pragma unroll
-                for (int v = 0; v < NV; ++v) {
-                    float s = c[0] * x[v][0];
-#pragma unroll
-                    for (int k = 1; k < CPL; ++k) s = __builtin_fmaf(c[k], x[v][k], s);
-                    p[v].v[t] = live ? s : 0.0f;
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < NV; ++v) p[v].v[t] = 0.0f;
-            }
+            for (int k = 0; k < NBLK; ++k) mb[t][k] = lane_bcast(m16, 16 * k);
         }
 #pragma unroll
-        for (int v = 0; v < NV; ++v) own[v][b] = reduce_block<T>(p[v], b, sc_lds, l);
+        for (int t = 0; t < T::NE; ++t) {
+            float gm[2];                                     // group maximum for the lanes below / from 32
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const int g = (WAVE * t + 32 * hf) / T::GROUP;
+                float mx = 0.0f;
+#pragma unroll
+                for (int t2 = 0; t2 < T::NE; ++t2)
+#pragma unroll
+                    for (int k = 0; k < NBLK; ++k)
+                        if ((WAVE * t2 + 16 * k) / T::GROUP == g && WAVE * t2 + 16 * k < T::DK)
+                            mx = fmaxf(mx, mb[t2][k]);
+                gm[hf] = mx;
+            }
+            const float gmax = l.lane < 32 ? gm[0] : gm[1];
+            int ex = __builtin_amdgcn_frexp_expf(gmax);
+            ex = ex < -100 ? -100 : ex;
+            const float f = __builtin_fmaf(xe[v][t], __builtin_ldexpf(1.0f, 22 - ex), 12582912.0f);
+            const uint32_t d = (as_u32(f) + 0x408080u) ^ 0x808080u;
+            const int e = l.lane + WAVE * t;
+            if (e < T::DK) {
+                uint8_t* at = lds_b + ((e / CPL) * 8 + T::PLANES * v) * CPL + operand_pos<T::BITS>(e % CPL);
+                at[0] = uint8_t(d);
+                at[CPL] = uint8_t(d >> 8);
+                at[2 * CPL] = uint8_t(d >> 16);
+                if (e % T::GROUP == 0) lds_xs[v * T::NG + e / T::GROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
+            }
+        }
     }
+}
+
+// Two row blocks of codes in flight per wavefront.  Lane (i = lane % 32, kb = lane / 32) holds, for column step ks,
+// the 16 codes at row 32 rb + i, columns 32 ks + 16 kb ...
+template <class T>
+struct Window {
+    RawRow<T::BITS> a[2][T::NKS];
+};
+template <class T>
+__device__ __forceinline__ const uint8_t* lane_codes_m(const uint8_t* head, const LaneId& l) {
+    return head + (l.lane % T::MR) * T::ROW_BYTES + (l.lane / T::MR) * T::LANE_BYTES;
+}
+template <class T>
+__device__ __forceinline__ void window_load(const uint8_t* lane_base, int rb, Window<T>& w) {
+#pragma unroll
+    for (int ks = 0; ks < T::NKS; ++ks)
+        w.a[rb & 1][ks] = load_row<T::BITS>(lane_base + rb * (T::MR * T::ROW_BYTES) + ks * (2 * T::LANE_BYTES));
+}
+template <class T>
+__device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
+    window_load<T>(lane_base, 0, w);
+    if constexpr (T::NRB > 1) window_load<T>(lane_base, 1, w);
+}
+
+// Row sums of the whole tile against NV read-out vectors: own[v][t] = (S0 x_v)[lane + 64 t], scales applied.
+// Per block of 32 rows: one matrix instruction per column step accumulates, per scale group, the 32 x (3 NV) integer
+// sums (row x digit plane); the lanes holding a plane's column park them in LDS; then lane (i, v) turns row i's sums
+// for vector v into fp32 -- (d0 + 2^8 d1 + 2^16 d2) 2^(e-22) is the group's dot product, times the group's scale,
+// groups added in order (the reference's "(group sum) x scale, group by group", _fold_triton.py:191-196).  The block
+// just consumed is refilled with the block after next.  Result layout of the instruction: lane (j = lane % 32,
+// kb = lane / 32) holds column j (= plane), rows 8 a + 4 kb + b in element 4 a + b.
+template <class T, int NV>
+__device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, const uint8_t* lds_b,
+                                           const float* lds_xs, const uint16_t* lds_sc, int32_t* lds_c, float* lds_own,
+                                           const LaneId& l, float (&own)[NV][T::NOWN]) {
+    constexpr int NPL = T::PLANES * NV;
+    static_assert(NPL <= 8 && NV <= 2, "digit planes fill at most 8 operand columns");
+    const int j = l.lane % T::MR, kb = l.lane / T::MR;
+    v4i bop[T::NKS];
+#pragma unroll
+    for (int ks = 0; ks < T::NKS; ++ks)
+        bop[ks] = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (j & 7)) * CPL);
+    float xs[T::NG];
+#pragma unroll
+    for (int g = 0; g < T::NG; ++g) xs[g] = lds_xs[(kb < NV ? kb : 0) * T::NG + g];
+
+#pragma unroll
+    for (int rb = 0; rb < T::NRB; ++rb) {
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) {
+            v16i acc = {0};
+#pragma unroll
+            for (int ks = 0; ks < T::NKS; ++ks)
+                if ((ks * T::MK) / T::GROUP == g)
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(w.a[rb & 1][ks]), bop[ks], acc, 0, 0, 0);
+            if (j < NPL) {
+                int4* dst = reinterpret_cast<int4*>(lds_c + (g * NPL + j) * T::MR + 4 * kb);
+#pragma unroll
+                for (int a = 0; a < 4; ++a) dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+            }
+        }
+        if (rb + 2 < T::NRB) window_load<T>(lane_base, rb + 2, w);
+        __syncthreads();
+        if (kb < NV) {
+            const int row = rb * T::MR + j;
+            float s = 0.0f;
+#pragma unroll
+            for (int g = 0; g < T::NG; ++g) {
+                const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
+                const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f, __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
+                const float term = (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
+                s = g == 0 ? term : s + term;
+            }
+            lds_own[kb * T::UROW + row] = s;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int t = 0; t < T::NOWN; ++t)
+            own[v][t] = owned_valid<T>(l, t) ? lds_own[v * T::UROW + owned_row<T>(l, t)] : 0.0f;
 }
 
 // A lane's 16-column piece of a d_k vector kept piecewise in LDS.
@@ -403,6 +462,12 @@ __device__ __forceinline__ void append_key(const float (&kx)[T::NE], float ks, c
 // ---------------------------------------------------------------------------------------------------------------
 // the fold
 // ---------------------------------------------------------------------------------------------------------------
+// A lane's first row piece in the row-shaped layout (LPRP lanes per row).
+template <class T>
+__device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
+    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
+    return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
+}
 // Fold operands, step 1 (before the front end's LDS is overwritten): the buffered values of the rows this lane owns,
 // dequantized, slot by slot.  uo[b][i] = U_i[row b] (slot m-1: the value just appended, `ur`).
 template <class T>
