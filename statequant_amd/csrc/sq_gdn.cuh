@@ -109,7 +109,7 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
         r = r < DV ? r : DV - 1;
         f.vr[t] = load_raw(p.v, p.v_dt, int64_t(a.b) * p.s_v + int64_t(a.h) * DV + r);
     }
-    window_init<T>(lane_codes_m<T>(a.Sh, l), f.win);
+    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
 }
 
 template <class T>
@@ -122,6 +122,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    uint8_t* lds_a = lds + L::A;
     int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);          // the fold's operands overlay the above
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     const int h = A.h;
     const int n = F.n;
     const float gcur = F.gcur;
-    const uint8_t* lane_base = lane_codes_m<T>(A.Sh, l);
+    const uint8_t* lane_base = lane_codes<T>(A.Sh, l);
 
     // ---- prep: q, k (fla's l2 normalisation), gates ----
     const bool full = n == m - 1;
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
 
     // ---- state pass ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_c, lds_own, l, own);
+    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, own);
 
     const KeyBuf<T>& kbuf = F.kbuf;
     const float gb_lane = F.gb_lane;

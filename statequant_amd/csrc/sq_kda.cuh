@@ -25,6 +25,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    uint8_t* lds_a = lds + L::A;
     int32_t* lds_ci = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m * DK;
     float* gch = p.st.GCUR + seq * p.st.sGC + int64_t(h) * DK;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const uint8_t* lane_base = lane_codes_m<T>(Sh, l);
+    const uint8_t* lane_base = lane_codes<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
     // ---- issue every load ----
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
 
     // ---- state pass against A*q, A*k ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_ci, lds_own, l, own);
+    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_ci, lds_own, l, own);
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll

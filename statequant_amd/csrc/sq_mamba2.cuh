@@ -21,6 +21,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC);
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    uint8_t* lds_a = lds + L::A;
     int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
@@ -53,7 +54,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
     float* gcp = p.st.GCUR + seq * p.st.sGC + h;
     int32_t* np = p.st.NPTR + seq * p.st.sN + h;
-    const uint8_t* lane_base = lane_codes_m<T>(Sh, l);
+    const uint8_t* lane_base = lane_codes<T>(Sh, l);
 
     // ---- issue every load ----
     const int n = *np & (m - 1);
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
 
     // ---- state pass ----
     float own[1][T::NOWN];
-    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_c, lds_own, l, own);
+    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, own);
 
     // ---- owned rows: y, and the value to buffer ----
     float u[T::NOWN], amax = 0.0f;

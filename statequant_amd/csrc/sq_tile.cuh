@@ -56,13 +56,15 @@ struct Tile {
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
     static constexpr int B_BYTES = (DK / CPL) * 8 * CPL;  // digit planes: [16-column piece][8 planes][16]
+    static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
+    static constexpr int A_BYTES = MR * A_PITCH;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
     static constexpr int SC_BYTES = round_up(DV * NG * 2, 16);
 };
 
 // LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
-// vectors, the raw buffered values, the raw scales, the digit planes with their exponents, one row block's integer
-// sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
+// vectors, the raw buffered values, the raw scales, the digit planes with their exponents, one row block of codes,
+// its integer sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
 template <class T, int NX, int NV = 2>
 struct LdsPlan {
     static constexpr int X = 0;
@@ -70,7 +72,8 @@ struct LdsPlan {
     static constexpr int SC = UB + T::UB_BYTES;
     static constexpr int B = SC + T::SC_BYTES;
     static constexpr int XS = B + T::B_BYTES;
-    static constexpr int C = XS + round_up(NV * T::NG * 4, 16);
+    static constexpr int A = XS + round_up(NV * T::NG * 4, 16);
+    static constexpr int C = A + T::A_BYTES;
     static constexpr int OWN = C + T::NG * T::PLANES * NV * T::MR * 4;
     static constexpr int FRONT = OWN + NV * T::UROW * 4;
     static constexpr int FK = 0;
@@ -210,21 +213,26 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
     }
 }
 
-// Two row blocks of codes in flight per wavefront.  Lane (i = lane % 32, kb = lane / 32) holds, for column step ks,
-// the 16 codes at row 32 rb + i, columns 32 ks + 16 kb ...
+// A lane's first row piece in the row-shaped layout (LPRP lanes per row).
+template <class T>
+__device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
+    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
+    return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
+}
+
+// Two row blocks of codes in flight per wavefront, loaded row-shaped (LPRP lanes per row, so every load instruction
+// covers whole, consecutive rows and costs the address unit one cycle per 64 bytes; fetched in operand shape -- 32
+// different rows per instruction -- the same bytes cost it 8 x as many cycles and the step became address-bound).
 template <class T>
 struct Window {
-    RawRow<T::BITS> a[2][T::NKS];
+    static constexpr int NL = T::MR / T::RG;              // loads per row block
+    RawRow<T::BITS> a[2][NL];
 };
-template <class T>
-__device__ __forceinline__ const uint8_t* lane_codes_m(const uint8_t* head, const LaneId& l) {
-    return head + (l.lane % T::MR) * T::ROW_BYTES + (l.lane / T::MR) * T::LANE_BYTES;
-}
 template <class T>
 __device__ __forceinline__ void window_load(const uint8_t* lane_base, int rb, Window<T>& w) {
 #pragma unroll
-    for (int ks = 0; ks < T::NKS; ++ks)
-        w.a[rb & 1][ks] = load_row<T::BITS>(lane_base + rb * (T::MR * T::ROW_BYTES) + ks * (2 * T::LANE_BYTES));
+    for (int j = 0; j < Window<T>::NL; ++j)
+        w.a[rb & 1][j] = load_row<T::BITS>(lane_base + (rb * T::MR + j * T::RG) * T::ROW_BYTES);
 }
 template <class T>
 __device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
@@ -237,12 +245,15 @@ __device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>&
 // sums (row x digit plane); the lanes holding a plane's column park them in LDS; then lane (i, v) turns row i's sums
 // for vector v into fp32 -- (d0 + 2^8 d1 + 2^16 d2) 2^(e-22) is the group's dot product, times the group's scale,
 // groups added in order (the reference's "(group sum) x scale, group by group", _fold_triton.py:191-196).  The block
-// just consumed is refilled with the block after next.  Result layout of the instruction: lane (j = lane % 32,
-// kb = lane / 32) holds column j (= plane), rows 8 a + 4 kb + b in element 4 a + b.
+// just consumed is refilled with the block after next.  A block changes from row shape to operand shape through LDS
+// (lds_a, row pitch = row + one lane piece: both the row-shaped writes and the operand-shaped reads are conflict
+// free): operand lane (i = lane % 32, kb = lane / 32) takes, for column step ks, the 16 codes at row i, columns
+// 32 ks + 16 kb.  Result layout of the instruction: lane (j, kb) holds column j (= plane), rows 8 a + 4 kb + b in
+// element 4 a + b.
 template <class T, int NV>
 __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, const uint8_t* lds_b,
-                                           const float* lds_xs, const uint16_t* lds_sc, int32_t* lds_c, float* lds_own,
-                                           const LaneId& l, float (&own)[NV][T::NOWN]) {
+                                           const float* lds_xs, const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c,
+                                           float* lds_own, const LaneId& l, float (&own)[NV][T::NOWN]) {
     constexpr int NPL = T::PLANES * NV;
     static_assert(NPL <= 8 && NV <= 2, "digit planes fill at most 8 operand columns");
     const int j = l.lane % T::MR, kb = l.lane / T::MR;
@@ -256,20 +267,28 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 
 #pragma unroll
     for (int rb = 0; rb < T::NRB; ++rb) {
+        if (l.cg < T::LPR) {
+#pragma unroll
+            for (int t = 0; t < Window<T>::NL; ++t)
+                store_row<T::BITS>(lds_a + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES, w.a[rb & 1][t]);
+        }
+        if (rb + 2 < T::NRB) window_load<T>(lane_base, rb + 2, w);
+        __syncthreads();
 #pragma unroll
         for (int g = 0; g < T::NG; ++g) {
             v16i acc = {0};
 #pragma unroll
             for (int ks = 0; ks < T::NKS; ++ks)
-                if ((ks * T::MK) / T::GROUP == g)
-                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(w.a[rb & 1][ks]), bop[ks], acc, 0, 0, 0);
+                if ((ks * T::MK) / T::GROUP == g) {
+                    const RawRow<T::BITS> r = load_row<T::BITS>(lds_a + j * T::A_PITCH + (2 * ks + kb) * T::LANE_BYTES);
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), bop[ks], acc, 0, 0, 0);
+                }
             if (j < NPL) {
                 int4* dst = reinterpret_cast<int4*>(lds_c + (g * NPL + j) * T::MR + 4 * kb);
 #pragma unroll
                 for (int a = 0; a < 4; ++a) dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
             }
         }
-        if (rb + 2 < T::NRB) window_load<T>(lane_base, rb + 2, w);
         __syncthreads();
         if (kb < NV) {
             const int row = rb * T::MR + j;
@@ -462,12 +481,7 @@ __device__ __forceinline__ void append_key(const float (&kx)[T::NE], float ks, c
 // ---------------------------------------------------------------------------------------------------------------
 // the fold
 // ---------------------------------------------------------------------------------------------------------------
-// A lane's first row piece in the row-shaped layout (LPRP lanes per row).
-template <class T>
-__device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
-    const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
-    return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
-}
+
 // Fold operands, step 1 (before the front end's LDS is overwritten): the buffered values of the rows this lane owns,
 // dequantized, slot by slot.  uo[b][i] = U_i[row b] (slot m-1: the value just appended, `ur`).
 template <class T>
