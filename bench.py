@@ -45,7 +45,7 @@ WORKLOADS = {
 
 # HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
 # over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {'gdn-int8-g128': 192143449}
 
 
 def state_bytes_per_slot(bits, group, hv, dk, dv, m):
@@ -142,6 +142,23 @@ def cpu_baseline(workload, m, budget_s=20.0):
                       f'torch CPU oracle, {cores} threads'}
 
 
+def calibrate_copy(dev, nbytes=1 << 30, reps=20):
+    """`reps` plain copies of `nbytes` (reads nbytes, writes nbytes each): the reference point for the HBM counters."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    print(json.dumps({'calibrate_copy': True, 'bytes_read': nbytes, 'bytes_written': nbytes, 'copies': reps + 1,
+                      'us_per_copy': round(us, 2), 'gbs_read_plus_write': round(2 * nbytes / us * 1e-3, 1)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -152,6 +169,9 @@ def main():
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-budget', type=float, default=20.0)
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='instead of the workload, run plain device copies of 1 GiB (the known-size kernel that '
+                         'rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by) and print their rate')
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit('bench.py: this build measures one GPU; the decode step has no cross-GPU exchange (slots shard '
@@ -160,6 +180,8 @@ def main():
         sys.exit('bench.py: no GPU visible; the packed decode step only runs as HIP kernels')
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
+    if a.calibrate_copy:
+        return calibrate_copy(dev)
     m = a.m
     fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
     fam, lay, views, idx = build(a.workload, m, dev)
