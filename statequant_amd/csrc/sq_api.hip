@@ -42,8 +42,21 @@ int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
     key->hk = L.hk;
     key->dk = L.dk;
     key->dv = L.dv;
+    key->gqa = L.hv / L.hk;
+    key->hv_shift = pow2(L.hv) ? __builtin_ctz(unsigned(L.hv)) : -1;
+    key->gqa_shift = pow2(key->gqa) ? __builtin_ctz(unsigned(key->gqa)) : -1;
+    key->per_xcd = 0;
     return SQ_OK;
 }
+
+// Tiles per XCD for the launch's tile -> XCD mapping (0: tile count not a multiple of 8, workgroup id = tile id).
+void set_rows(sq::LayoutKey* key, int rows) {
+    const int64_t tiles = int64_t(rows) * key->hv;
+    key->per_xcd = (tiles % 8 == 0) ? int(tiles / 8) : 0;
+}
+
+// A per-sequence or per-row stride as the kernels take it: non-negative, below 2^31.
+bool stride_ok(int64_t s) { return s >= 0 && s < (int64_t(1) << 31); }
 
 // Pointers, strides and alignment of the stored state.  The kernels read a lane's piece of a code row with one
 // 128-bit (int8) or 64-bit (int4) load and a piece of a buffered int8 key with one 128-bit load.
@@ -61,15 +74,18 @@ int check_state(const sq_state& s, const sq_layout& L, const char* who, sq::Stat
         return fail(SQ_E_ARG, "%s: scales and value buffer must be 16-byte aligned (base and per-sequence stride)", who);
     if (!aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
         return fail(SQ_E_ARG, "%s: misaligned decay / counter pointer", who);
-    st->S = static_cast<uint8_t*>(s.S);         st->sS = s.sS;
-    st->SC = static_cast<uint16_t*>(s.SC);      st->sSC = s.sSC;
-    st->KB = static_cast<uint8_t*>(s.KB);       st->sKB = s.sKB;
-    st->KBS = static_cast<uint16_t*>(s.KBS);    st->sKBS = s.sKBS;
-    st->UB = static_cast<uint8_t*>(s.UB);       st->sUB = s.sUB;
-    st->UBS = static_cast<uint16_t*>(s.UBS);    st->sUBS = s.sUBS;
-    st->GB = s.GB;                              st->sGB = s.sGB;
-    st->GCUR = s.GCUR;                          st->sGC = s.sGC;
-    st->NPTR = s.NPTR;                          st->sN = s.sN;
+    if (!stride_ok(s.sS) || !stride_ok(s.sSC) || !stride_ok(s.sKB) || !stride_ok(s.sKBS) || !stride_ok(s.sUB) ||
+        !stride_ok(s.sUBS) || !stride_ok(s.sGB) || !stride_ok(s.sGC) || !stride_ok(s.sN))
+        return fail(SQ_E_ARG, "%s: per-sequence strides must be in [0, 2^31)", who);
+    st->S = static_cast<uint8_t*>(s.S);         st->sS = uint32_t(s.sS);
+    st->SC = static_cast<uint16_t*>(s.SC);      st->sSC = uint32_t(s.sSC);
+    st->KB = static_cast<uint8_t*>(s.KB);       st->sKB = uint32_t(s.sKB);
+    st->KBS = static_cast<uint16_t*>(s.KBS);    st->sKBS = uint32_t(s.sKBS);
+    st->UB = static_cast<uint8_t*>(s.UB);       st->sUB = uint32_t(s.sUB);
+    st->UBS = static_cast<uint16_t*>(s.UBS);    st->sUBS = uint32_t(s.sUBS);
+    st->GB = s.GB;                              st->sGB = uint32_t(s.sGB);
+    st->GCUR = s.GCUR;                          st->sGC = uint32_t(s.sGC);
+    st->NPTR = s.NPTR;                          st->sN = uint32_t(s.sN);
     return SQ_OK;
 }
 
@@ -146,21 +162,25 @@ int sq_gdn_step(const sq_gdn_args* a, void* stream) {
         if (!a->g || !a->beta) return fail(SQ_E_ARG, "%s: neither g / beta nor a gate", who);
         if (!dtype_ok(a->g_dtype) || !dtype_ok(a->beta_dtype)) return fail(SQ_E_ARG, "%s: bad g / beta dtype code", who);
     }
+    if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) ||
+        !stride_ok(a->gate ? a->s_a : a->s_g) || !stride_ok(a->gate ? a->s_b : a->s_beta))
+        return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
     p.rows = a->rows;
+    set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.q = a->q; p.s_q = a->s_q; p.q_dt = a->q_dtype;
-    p.k = a->k; p.s_k = a->s_k; p.k_dt = a->k_dtype;
-    p.v = a->v; p.s_v = a->s_v; p.v_dt = a->v_dtype;
+    p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
+    p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
+    p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
     p.qk_per_key_head = a->qk_per_key_head != 0;
     p.gate = a->gate != 0;
     if (p.gate) {
-        p.a = a->a; p.s_a = a->s_a; p.a_dt = a->a_dtype;
-        p.bt = a->b; p.s_bt = a->s_b; p.bt_dt = a->b_dtype;
+        p.a = a->a; p.s_a = uint32_t(a->s_a); p.a_dt = a->a_dtype;
+        p.bt = a->b; p.s_bt = uint32_t(a->s_b); p.bt_dt = a->b_dtype;
         p.A_log = a->A_log; p.A_log_dt = a->A_log_dtype;
         p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
     } else {                  // the kernel reads the same four operands either way: g, beta, and g twice as dummies
-        p.a = a->g; p.s_a = a->s_g; p.a_dt = a->g_dtype;
-        p.bt = a->beta; p.s_bt = a->s_beta; p.bt_dt = a->beta_dtype;
+        p.a = a->g; p.s_a = uint32_t(a->s_g); p.a_dt = a->g_dtype;
+        p.bt = a->beta; p.s_bt = uint32_t(a->s_beta); p.bt_dt = a->beta_dtype;
         p.A_log = a->g; p.A_log_dt = a->g_dtype;
         p.dt_bias = a->g; p.dt_bias_dt = a->g_dtype;
     }
@@ -184,14 +204,18 @@ int sq_kda_step(const sq_kda_args* a, void* stream) {
     if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->g_dtype) ||
         !dtype_ok(a->beta_dtype) || !dtype_ok(a->out_dtype))
         return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) || !stride_ok(a->s_g) ||
+        !stride_ok(a->s_beta) || !stride_ok(a->s_out))
+        return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
     p.rows = a->rows;
+    set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.q = a->q; p.s_q = a->s_q; p.q_dt = a->q_dtype;
-    p.k = a->k; p.s_k = a->s_k; p.k_dt = a->k_dtype;
-    p.v = a->v; p.s_v = a->s_v; p.v_dt = a->v_dtype;
-    p.g = a->g; p.s_g = a->s_g; p.g_dt = a->g_dtype;
-    p.beta = a->beta; p.s_beta = a->s_beta; p.beta_dt = a->beta_dtype;
-    p.out = a->out; p.s_out = a->s_out; p.out_dt = a->out_dtype;
+    p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
+    p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
+    p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
+    p.g = a->g; p.s_g = uint32_t(a->s_g); p.g_dt = a->g_dtype;
+    p.beta = a->beta; p.s_beta = uint32_t(a->s_beta); p.beta_dt = a->beta_dtype;
+    p.out = a->out; p.s_out = uint32_t(a->s_out); p.out_dt = a->out_dtype;
     p.scale = a->scale;
     return finish(sq::dispatch_kda(p, static_cast<hipStream_t>(stream), true), who, a->lay);
 }
@@ -209,12 +233,15 @@ int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
         !dtype_ok(a->A_dtype) || !dtype_ok(a->out_dtype) || (a->D && !dtype_ok(a->D_dtype)) ||
         (a->dt_bias && !dtype_ok(a->dt_bias_dtype)))
         return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    if (!stride_ok(a->s_x) || !stride_ok(a->s_dt) || !stride_ok(a->s_B) || !stride_ok(a->s_C) || !stride_ok(a->s_out))
+        return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
     p.rows = a->rows;
+    set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.x = a->x; p.s_x = a->s_x; p.x_dt = a->x_dtype;
-    p.dt = a->dt; p.s_dt = a->s_dt; p.dt_dt = a->dt_dtype;
-    p.B = a->B; p.s_B = a->s_B; p.B_dt = a->B_dtype;
-    p.C = a->C; p.s_C = a->s_C; p.C_dt = a->C_dtype;
+    p.x = a->x; p.s_x = uint32_t(a->s_x); p.x_dt = a->x_dtype;
+    p.dt = a->dt; p.s_dt = uint32_t(a->s_dt); p.dt_dt = a->dt_dtype;
+    p.B = a->B; p.s_B = uint32_t(a->s_B); p.B_dt = a->B_dtype;
+    p.C = a->C; p.s_C = uint32_t(a->s_C); p.C_dt = a->C_dtype;
     p.A = a->A; p.A_dt = a->A_dtype;
     p.has_D = a->D != nullptr;
     p.has_dt_bias = a->dt_bias != nullptr;
@@ -225,7 +252,7 @@ int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
     p.dt_softplus = a->dt_softplus != 0;
     p.dt_clamp = a->dt_clamp != 0;
     p.dt_min = a->dt_min; p.dt_max = a->dt_max;
-    p.out = a->out; p.s_out = a->s_out; p.out_dt = a->out_dtype;
+    p.out = a->out; p.s_out = uint32_t(a->s_out); p.out_dt = a->out_dtype;
     return finish(sq::dispatch_mamba2(p, static_cast<hipStream_t>(stream), true), who, a->lay);
 }
 

@@ -43,23 +43,30 @@ __device__ __forceinline__ uint16_t f32_to_f16(float f) { return __builtin_bit_c
 // A scalar of a float tensor of run-time dtype (inputs come as fp32, bf16 or fp16), in two steps so that a kernel can
 // issue all its loads first and convert later: a conversion right behind a load, inside the dtype branch, makes
 // the compiler wait for memory in every branch and serializes the loads.
-__device__ __forceinline__ uint32_t load_raw(const void* p, int dt, int64_t i) {
+// `p` carries the wave-uniform part of the address (see `advance`), `i` the lane's 32-bit element index: the load
+// then needs no 64-bit vector arithmetic.
+__device__ __forceinline__ uint32_t load_raw(const void* p, int dt, uint32_t i) {
     if (dt == F32) return reinterpret_cast<const uint32_t*>(p)[i];
     return reinterpret_cast<const uint16_t*>(p)[i];
+}
+__device__ __forceinline__ const void* advance(const void* p, int dt, uint64_t elems) {
+    return reinterpret_cast<const uint8_t*>(p) + (elems << (dt == F32 ? 2 : 1));
+}
+__device__ __forceinline__ void* advance(void* p, int dt, uint64_t elems) {
+    return reinterpret_cast<uint8_t*>(p) + (elems << (dt == F32 ? 2 : 1));
 }
 // The same for a wave-uniform address (a per-head scalar).  The offset is laundered through a vector register so
 // that the load stays a vector load: as a scalar load its result would have to be moved into a VGPR right away, and
 // the wait for that move also waits for every vector load issued before it.
-__device__ __forceinline__ uint32_t load_raw_uniform(const void* p, int dt, int64_t i) {
-    int32_t z = 0;
+__device__ __forceinline__ uint32_t load_raw_uniform(const void* p, int dt, uint64_t i) {
+    uint32_t z = 0;
     asm volatile("" : "+v"(z));
-    return load_raw(p, dt, i + z);
+    return load_raw(advance(p, dt, i), dt, z);
 }
 __device__ __forceinline__ float raw_to_f(uint32_t r, int dt) {
     return dt == F32 ? as_f32(r) : dt == BF16 ? bf16_to_f32(uint16_t(r)) : f16_to_f32(uint16_t(r));
 }
-__device__ __forceinline__ float load_f(const void* p, int dt, int64_t i) { return raw_to_f(load_raw(p, dt, i), dt); }
-__device__ __forceinline__ void store_f(void* p, int dt, int64_t i, float v) {
+__device__ __forceinline__ void store_f(void* p, int dt, uint32_t i, float v) {
     if (dt == F32) reinterpret_cast<float*>(p)[i] = v;
     else reinterpret_cast<uint16_t*>(p)[i] = dt == BF16 ? f32_to_bf16(v) : f32_to_f16(v);
 }
@@ -240,14 +247,6 @@ template <int BITS>
 __device__ __forceinline__ void store_row(uint8_t* p, const RawRow<BITS>& r) {
     if constexpr (BITS == 8) *reinterpret_cast<uint4*>(p) = r.v;
     else *reinterpret_cast<uint2*>(p) = r.v;
-}
-
-// Workgroup id -> tile id.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs; this makes every XCD walk
-// a contiguous range of tiles, so the tiles of one sequence (shared key buffer, neighbouring counters) meet in one L2.
-__device__ __forceinline__ int xcd_tile(int wg, int n) {
-    constexpr int XCDS = 8;
-    if (n % XCDS) return wg;
-    return (wg % XCDS) * (n / XCDS) + wg / XCDS;
 }
 
 }  // namespace sq

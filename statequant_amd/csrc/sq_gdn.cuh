@@ -23,7 +23,7 @@ template <class T>
 struct GdnAddr {
     int b, h, hk;
     bool live;                         // false: padding row (slot index <= 0)
-    int64_t obase;
+    uint64_t obase;
     uint8_t* Sh;
     uint16_t* SCh;
     BufAddr<T> buf;
@@ -32,24 +32,24 @@ struct GdnAddr {
     int32_t* np;
 };
 template <class T>
-__device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p, int tile) {
+__device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p) {
     GdnAddr<T> a;
-    a.b = tile / p.hv;
-    a.h = tile - a.b * p.hv;
-    a.hk = a.h / (p.hv / p.hk);
-    const int64_t seq = p.idx ? int64_t(p.idx[a.b]) : int64_t(a.b);
-    a.live = !(p.idx && seq <= 0);
-    a.obase = (int64_t(a.b) * p.hv + a.h) * T::DV;
-    const int m = p.m;
-    a.Sh = p.st.S + seq * p.st.sS + int64_t(a.h) * (T::DV * T::ROW_BYTES);
-    a.SCh = p.st.SC + seq * p.st.sSC + int64_t(a.h) * (T::DV * T::NG);
-    a.buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(a.hk) * m * T::DK) * T::BE;
-    a.buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(a.h) * m * T::DV) * T::BE;
-    a.buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(a.hk) * m;
-    a.buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(a.h) * m;
-    a.GBh = p.st.GB + seq * p.st.sGB + int64_t(a.h) * m;
-    a.gcp = p.st.GCUR + seq * p.st.sGC + a.h;
-    a.np = p.st.NPTR + seq * p.st.sN + a.h;
+    const TileId t = tile_id(p);
+    a.b = t.b; a.h = t.h; a.hk = t.hk;
+    const int32_t slot = p.idx ? p.idx[a.b] : a.b;
+    a.live = !(p.idx && slot <= 0);
+    const uint32_t seq = a.live ? uint32_t(slot) : 0u;
+    const uint32_t m = p.m, h = a.h, hk = a.hk;
+    a.obase = (uint64_t(uint32_t(a.b)) * uint32_t(p.hv) + h) * T::DV;
+    a.Sh = field(p.st.S, seq, p.st.sS, h * (T::DV * T::ROW_BYTES));
+    a.SCh = field(p.st.SC, seq, p.st.sSC, h * (T::DV * T::NG));
+    a.buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * m * T::DK) * T::BE;
+    a.buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * m * T::DV) * T::BE;
+    a.buf.KBS = field(p.st.KBS, seq, p.st.sKBS, hk * m);
+    a.buf.UBS = field(p.st.UBS, seq, p.st.sUBS, h * m);
+    a.GBh = field(p.st.GB, seq, p.st.sGB, h * m);
+    a.gcp = field(p.st.GCUR, seq, p.st.sGC, h);
+    a.np = field(p.st.NPTR, seq, p.st.sN, h);
     return a;
 }
 
@@ -75,7 +75,7 @@ template <class T>
 __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& a, const LaneId& l, GdnFront<T>& f) {
     constexpr int DK = T::DK, DV = T::DV;
     const int m = p.m;
-    const int gqa = p.hv / p.hk;
+    const int gqa = p.gqa;
     const int hq = p.qk_per_key_head ? a.hk : a.h;
     const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
     f.n = *a.np & (m - 1);
@@ -89,25 +89,30 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     load_keybuf<T>(a.buf, m, l, f.kbuf);
 #pragma unroll
     for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < m ? i : m - 1]; }
+    const uint32_t b = a.b, h = a.h;
+    const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(hq) * DK);
+    const void* kb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(hq) * DK);
+    const void* kxb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(a.hk * gqa) * DK);
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
-        int e = l.lane + WAVE * t;
+        uint32_t e = l.lane + WAVE * t;
         e = e < DK ? e : DK - 1;
-        f.qr[t] = load_raw(p.q, p.q_dt, int64_t(a.b) * p.s_q + int64_t(hq) * DK + e);
-        f.kr[t] = load_raw(p.k, p.k_dt, int64_t(a.b) * p.s_k + int64_t(hq) * DK + e);
-        f.kxr[t] = own_key ? load_raw(p.k, p.k_dt, int64_t(a.b) * p.s_k + int64_t(a.hk * gqa) * DK + e) : 0u;
+        f.qr[t] = load_raw(qb, p.q_dt, e);
+        f.kr[t] = load_raw(kb, p.k_dt, e);
+        f.kxr[t] = own_key ? load_raw(kxb, p.k_dt, e) : 0u;
     }
     // gate: a, b [rows, hv], A_log, dt_bias [hv];  no gate: the same four slots carry g, beta and two dummies
     // (the C ABI points them at g), so the loads need no branch
-    f.g0 = load_raw_uniform(p.a, p.a_dt, int64_t(a.b) * p.s_a + a.h);
-    f.g1 = load_raw_uniform(p.bt, p.bt_dt, int64_t(a.b) * p.s_bt + a.h);
-    f.g2 = load_raw_uniform(p.A_log, p.A_log_dt, a.h);
-    f.g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, a.h);
+    f.g0 = load_raw_uniform(p.a, p.a_dt, uint64_t(b) * p.s_a + h);
+    f.g1 = load_raw_uniform(p.bt, p.bt_dt, uint64_t(b) * p.s_bt + h);
+    f.g2 = load_raw_uniform(p.A_log, p.A_log_dt, h);
+    f.g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);
+    const void* vb = advance(p.v, p.v_dt, uint64_t(b) * p.s_v + h * DV);
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = owned_row<T>(l, t);
+        uint32_t r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        f.vr[t] = load_raw(p.v, p.v_dt, int64_t(a.b) * p.s_v + int64_t(a.h) * DV + r);
+        f.vr[t] = load_raw(vb, p.v_dt, r);
     }
     window_init<T>(lane_codes<T>(a.Sh, l), f.win);
 }
@@ -128,16 +133,16 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);          // the fold's operands overlay the above
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
-    const int gqa = p.hv / p.hk;
+    const int gqa = p.gqa;
     const int m = p.m;
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
     const bool own_key = !p.qk_per_key_head && gqa > 1;
     const LaneId l = lane_id<T>();
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const GdnAddr<T> A = gdn_addr<T>(p, tile);
+    const GdnAddr<T> A = gdn_addr<T>(p);
+    void* const outp = advance(p.out, p.out_dt, A.obase);
     if (!A.live) {                                                // padding row: zero output, touch nothing else
-        for (int r = l.lane; r < DV; r += WAVE) store_f(p.out, p.out_dt, A.obase + r, 0.0f);
+        for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
     GdnFront<T> F;
@@ -242,7 +247,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * __builtin_fmaf(-a, sk, vt);
         const float o = __builtin_fmaf(kq, u[t], a * sq);
-        if (valid) store_f(p.out, p.out_dt, A.obase + r, o);
+        if (valid) store_f(outp, p.out_dt, r, o);
         else u[t] = 0.0f;
         amax = fmaxf(amax, fabsf(u[t]));
     }
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     }
     float ur[T::NOWN], kr[T::NE];                         // value / key as stored, dequantized
     append_values<T>(u, us, A.buf, n, l, ur);
-    append_key<T>(kxe, ks, A.buf, n, (h % gqa) == 0, l, kr);
+    append_key<T>(kxe, ks, A.buf, n, int(h) == A.hk * gqa, l, kr);
     if (l.lane == 0) A.GBh[n] = gnew;
 
     // ---- fold ----

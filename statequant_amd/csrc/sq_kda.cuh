@@ -33,30 +33,31 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     float* lds_c = reinterpret_cast<float*>(lds + L::FC);
 
     const LaneId l = lane_id<T>();
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int b = tile / p.hv;
-    const int h = tile - b * p.hv;
+    const TileId tid = tile_id(p);
+    const uint32_t b = tid.b, h = tid.h;
     const int m = p.m;
+    const uint32_t um = m;
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int64_t seq = p.idx ? int64_t(p.idx[b]) : int64_t(b);
-    const int64_t obase = int64_t(b) * p.s_out + int64_t(h) * DV;
-    if (p.idx && seq <= 0) {
-        for (int r = l.lane; r < DV; r += WAVE) store_f(p.out, p.out_dt, obase + r, 0.0f);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
+    void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
+    if (p.idx && slot <= 0) {
+        for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
+    const uint32_t seq = slot;
 
-    uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
-    uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
+    uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
+    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * (DV * T::NG));
     BufAddr<T> buf;
-    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(h) * m * DK) * T::BE;
-    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * T::BE;
-    buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(h) * m;
-    buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
-    float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m * DK;
-    float* gch = p.st.GCUR + seq * p.st.sGC + int64_t(h) * DK;
-    int32_t* np = p.st.NPTR + seq * p.st.sN + h;
+    buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + h * um * DK) * T::BE;
+    buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
+    buf.KBS = field(p.st.KBS, seq, p.st.sKBS, h * um);
+    buf.UBS = field(p.st.UBS, seq, p.st.sUBS, h * um);
+    float* GBh = field(p.st.GB, seq, p.st.sGB, h * um * DK);
+    float* gch = field(p.st.GCUR, seq, p.st.sGC, h * DK);
+    int32_t* np = field(p.st.NPTR, seq, p.st.sN, h);
     const uint8_t* lane_base = lane_codes<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
@@ -80,23 +81,26 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     }
     uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     float gc[T::NE];
+    const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
+    const void* kb_ = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + h * DK);
+    const void* gb_ = advance(p.g, p.g_dt, uint64_t(b) * p.s_g + h * DK);
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
-        int e = l.lane + WAVE * t;
+        uint32_t e = l.lane + WAVE * t;
         e = e < DK ? e : DK - 1;
-        const int64_t off = int64_t(h) * DK + e;
-        qr[t] = load_raw(p.q, p.q_dt, int64_t(b) * p.s_q + off);
-        kr_[t] = load_raw(p.k, p.k_dt, int64_t(b) * p.s_k + off);
-        gr[t] = load_raw(p.g, p.g_dt, int64_t(b) * p.s_g + off);
+        qr[t] = load_raw(qb, p.q_dt, e);
+        kr_[t] = load_raw(kb_, p.k_dt, e);
+        gr[t] = load_raw(gb_, p.g_dt, e);
         gc[t] = gch[e];
     }
-    const uint32_t betar = load_raw_uniform(p.beta, p.beta_dt, int64_t(b) * p.s_beta + h);
+    const uint32_t betar = load_raw_uniform(p.beta, p.beta_dt, uint64_t(b) * p.s_beta + h);
     uint32_t vr[T::NOWN];
+    const void* vb = advance(p.v, p.v_dt, uint64_t(b) * p.s_v + h * DV);
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = owned_row<T>(l, t);
+        uint32_t r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        vr[t] = load_raw(p.v, p.v_dt, int64_t(b) * p.s_v + int64_t(h) * DV + r);
+        vr[t] = load_raw(vb, p.v_dt, r);
     }
     Window<T> win;
     window_init<T>(lane_base, win);
@@ -203,7 +207,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
         const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * (vt - sk);
         const float o = __builtin_fmaf(kq, u[t], sq);
-        if (valid) store_f(p.out, p.out_dt, obase + r, o);
+        if (valid) store_f(outp, p.out_dt, r, o);
         else u[t] = 0.0f;
         amax = fmaxf(amax, fabsf(u[t]));
     }

@@ -28,32 +28,32 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
     const LaneId l = lane_id<T>();
-    const int tile = xcd_tile(blockIdx.x, gridDim.x);
-    const int b = tile / p.hv;
-    const int h = tile - b * p.hv;
-    const int gqa = p.hv / p.hk;
-    const int hk = h / gqa;
+    const TileId tid = tile_id(p);
+    const uint32_t b = tid.b, h = tid.h, hk = tid.hk;
+    const int gqa = p.gqa;
     const int m = p.m;
+    const uint32_t um = m;
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int64_t seq = p.idx ? int64_t(p.idx[b]) : int64_t(b);
-    const int64_t obase = int64_t(b) * p.s_out + int64_t(h) * DV;
-    if (p.idx && seq <= 0) {
-        for (int r = l.lane; r < DV; r += WAVE) store_f(p.out, p.out_dt, obase + r, 0.0f);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
+    void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
+    if (p.idx && slot <= 0) {
+        for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
+    const uint32_t seq = slot;
 
-    uint8_t* Sh = p.st.S + seq * p.st.sS + int64_t(h) * (DV * T::ROW_BYTES);
-    uint16_t* SCh = p.st.SC + seq * p.st.sSC + int64_t(h) * (DV * T::NG);
+    uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
+    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * (DV * T::NG));
     BufAddr<T> buf;
-    buf.KB = p.st.KB + (seq * p.st.sKB + int64_t(hk) * m * DK) * T::BE;
-    buf.UB = p.st.UB + (seq * p.st.sUB + int64_t(h) * m * DV) * T::BE;
-    buf.KBS = p.st.KBS + seq * p.st.sKBS + int64_t(hk) * m;
-    buf.UBS = p.st.UBS + seq * p.st.sUBS + int64_t(h) * m;
-    float* GBh = p.st.GB + seq * p.st.sGB + int64_t(h) * m;
-    float* gcp = p.st.GCUR + seq * p.st.sGC + h;
-    int32_t* np = p.st.NPTR + seq * p.st.sN + h;
+    buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
+    buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
+    buf.KBS = field(p.st.KBS, seq, p.st.sKBS, hk * um);
+    buf.UBS = field(p.st.UBS, seq, p.st.sUBS, h * um);
+    float* GBh = field(p.st.GB, seq, p.st.sGB, h * um);
+    float* gcp = field(p.st.GCUR, seq, p.st.sGC, h);
+    int32_t* np = field(p.st.NPTR, seq, p.st.sN, h);
     const uint8_t* lane_base = lane_codes<T>(Sh, l);
 
     // ---- issue every load ----
@@ -73,23 +73,26 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
 #pragma unroll
     for (int t = 0; t < KT; ++t) { const int i = l.rg + T::RG * t; gb[t] = GBh[i < m ? i : m - 1]; }
     uint32_t cr[T::NE], br[T::NE];
+    const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
+    const void* bb = advance(p.B, p.B_dt, uint64_t(b) * p.s_B + hk * DK);
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
-        int e = l.lane + WAVE * t;
+        uint32_t e = l.lane + WAVE * t;
         e = e < DK ? e : DK - 1;
-        cr[t] = load_raw(p.C, p.C_dt, int64_t(b) * p.s_C + int64_t(hk) * DK + e);
-        br[t] = load_raw(p.B, p.B_dt, int64_t(b) * p.s_B + int64_t(hk) * DK + e);
+        cr[t] = load_raw(cb, p.C_dt, e);
+        br[t] = load_raw(bb, p.B_dt, e);
     }
-    const uint32_t dtr = load_raw_uniform(p.dt, p.dt_dt, int64_t(b) * p.s_dt + h);
+    const uint32_t dtr = load_raw_uniform(p.dt, p.dt_dt, uint64_t(b) * p.s_dt + h);
     const uint32_t ar = load_raw_uniform(p.A, p.A_dt, h);
     const uint32_t dbr = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);     // absent: the C ABI points them at A,
     const uint32_t ddr = load_raw_uniform(p.D, p.D_dt, h);                 // so the loads need no branch
     uint32_t xr_raw[T::NOWN];
+    const void* xb = advance(p.x, p.x_dt, uint64_t(b) * p.s_x + h * DV);
 #pragma unroll
     for (int t = 0; t < T::NOWN; ++t) {
-        int r = owned_row<T>(l, t);
+        uint32_t r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        xr_raw[t] = load_raw(p.x, p.x_dt, int64_t(b) * p.s_x + int64_t(h) * DV + r);
+        xr_raw[t] = load_raw(xb, p.x_dt, r);
     }
     Window<T> win;
     window_init<T>(lane_base, win);
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         u[t] = dt * xr;
         float y = __builtin_fmaf(bc, u[t], a * sq);
         if (p.has_D) y = __builtin_fmaf(dd, xr, y);
-        if (valid) store_f(p.out, p.out_dt, obase + r, y);
+        if (valid) store_f(outp, p.out_dt, r, y);
         amax = fmaxf(amax, fabsf(u[t]));
     }
 
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     }
     float ur[T::NOWN], kr[T::NE];
     append_values<T>(u, us, buf, n, l, ur);
-    append_key<T>(kxe, ks, buf, n, (h % gqa) == 0, l, kr);
+    append_key<T>(kxe, ks, buf, n, int(h) == hk * gqa, l, kr);
     if (l.lane == 0) GBh[n] = gnew;
 
     // ---- fold ----

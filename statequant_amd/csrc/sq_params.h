@@ -6,20 +6,25 @@
 
 namespace sq {
 
+// Per-sequence strides are below 2^31 (checked by the C ABI): sequence x stride is then one 32 x 32 -> 64 bit
+// multiply on the scalar unit instead of a full 64-bit one.
 struct StatePtrs {
-    uint8_t* S;      int64_t sS;     // bytes of codes per sequence step (int8: elements = bytes; int4: packed bytes)
-    uint16_t* SC;    int64_t sSC;
-    uint8_t* KB;     int64_t sKB;    // strides of KB / UB in ELEMENTS (int8 or bf16)
-    uint16_t* KBS;   int64_t sKBS;
-    uint8_t* UB;     int64_t sUB;
-    uint16_t* UBS;   int64_t sUBS;
-    float* GB;       int64_t sGB;
-    float* GCUR;     int64_t sGC;
-    int32_t* NPTR;   int64_t sN;
+    uint8_t* S;      uint32_t sS;     // bytes of codes per sequence (int8: elements = bytes; int4: packed bytes)
+    uint16_t* SC;    uint32_t sSC;
+    uint8_t* KB;     uint32_t sKB;    // strides of KB / UB in ELEMENTS (int8 or bf16)
+    uint16_t* KBS;   uint32_t sKBS;
+    uint8_t* UB;     uint32_t sUB;
+    uint16_t* UBS;   uint32_t sUBS;
+    float* GB;       uint32_t sGB;
+    float* GCUR;     uint32_t sGC;
+    int32_t* NPTR;   uint32_t sN;
 };
 
 struct LayoutKey {
     int bits, group, qbuf, m, hv, hk, dk, dv;
+    // launch geometry helpers, filled by the C ABI: gqa = hv / hk; log2 of hv and of gqa where those are powers of two (else
+    // -1: the kernel divides), and tiles per XCD when the tile count is a multiple of 8 (else 0: no XCD mapping)
+    int gqa, hv_shift, gqa_shift, per_xcd;
 };
 
 struct GdnParams : LayoutKey {
@@ -27,12 +32,12 @@ struct GdnParams : LayoutKey {
     int rows;
     const int32_t* idx;
     const void *q, *k, *v;
-    int64_t s_q, s_k, s_v;
+    uint32_t s_q, s_k, s_v;
     int q_dt, k_dt, v_dt;
     int qk_per_key_head, gate;
     // gate: a, b, A_log, dt_bias;  no gate: a = g, bt = beta, A_log = dt_bias = g (never used, always readable)
     const void *a, *bt, *A_log, *dt_bias;
-    int64_t s_a, s_bt;
+    uint32_t s_a, s_bt;
     int a_dt, bt_dt, A_log_dt, dt_bias_dt;
     void* out;
     int out_dt;
@@ -44,10 +49,10 @@ struct KdaParams : LayoutKey {
     int rows;
     const int32_t* idx;
     const void *q, *k, *v, *g, *beta;
-    int64_t s_q, s_k, s_v, s_g, s_beta;
+    uint32_t s_q, s_k, s_v, s_g, s_beta;
     int q_dt, k_dt, v_dt, g_dt, beta_dt;
     void* out;
-    int64_t s_out;
+    uint32_t s_out;
     int out_dt;
     float scale;
 };
@@ -57,12 +62,12 @@ struct Mamba2Params : LayoutKey {
     int rows;
     const int32_t* idx;
     const void *x, *dt, *B, *C, *A, *D, *dt_bias;
-    int64_t s_x, s_dt, s_B, s_C;
+    uint32_t s_x, s_dt, s_B, s_C;
     int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
     int dt_softplus, dt_clamp, has_D, has_dt_bias;      // absent D / dt_bias: pointers alias A (readable, unused)
     float dt_min, dt_max;
     void* out;
-    int64_t s_out;
+    uint32_t s_out;
     int out_dt;
 };
 

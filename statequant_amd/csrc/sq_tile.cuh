@@ -103,6 +103,28 @@ __device__ __forceinline__ LaneId lane_id() {
 template <class T>
 __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG + l.rg; }
 
+// Which (batch row, value head, key head) a workgroup works on.  Consecutive workgroup ids are dealt round-robin to
+// the 8 XCDs; with `per_xcd` set every XCD walks a contiguous range of tiles, so the heads of one sequence (shared key
+// buffer, neighbouring counters) meet in one L2.
+struct TileId {
+    int b, h, hk;
+};
+template <class K>
+__device__ __forceinline__ TileId tile_id(const K& k) {
+    const int wg = blockIdx.x;
+    const int tile = k.per_xcd ? (wg & 7) * k.per_xcd + (wg >> 3) : wg;
+    TileId t;
+    t.b = k.hv_shift >= 0 ? tile >> k.hv_shift : tile / k.hv;
+    t.h = tile - t.b * k.hv;
+    t.hk = k.gqa_shift >= 0 ? t.h >> k.gqa_shift : t.h / k.gqa;
+    return t;
+}
+// Address of a per-sequence field: base + sequence x stride + offset inside the sequence, in elements of E.
+template <class E>
+__device__ __forceinline__ E* field(E* base, uint32_t seq, uint32_t stride, uint32_t off) {
+    return base + (uint64_t(seq) * stride + off);
+}
+
 // The head rows a lane owns after the state pass (epilogue, append, fold staging): lane + 64 t.
 template <class T>
 __device__ __forceinline__ int owned_row(const LaneId& l, int t) { return l.lane + WAVE * t; }
