@@ -81,6 +81,7 @@ struct LdsPlan {
     static constexpr int FC = FU + T::MMAX * T::UROW * 4;
     static constexpr int FOLD = FC + T::KROW * 4;
     static constexpr int BYTES = FRONT > FOLD ? FRONT : FOLD;
+    static_assert(T::MMAX * T::KROW * 4 >= T::A_BYTES, "the fold reuses the key region as its row-block buffer");
 };
 
 // LDS position of element e of a d_k vector stored piecewise.
@@ -550,65 +551,137 @@ __device__ __forceinline__ void fold_stage_key(const float (&kr)[T::NE], int slo
 //   lds_u   [m][UROW]   the folded values du_i (GDN / Mamba2: decay ratio x delta value; KDA: delta value)
 //   lds_c   [KROW]      COLVEC: per-column factors on the dequantized old state (KDA);  else the scalar `cmul`
 //                       (GDN / Mamba2: exp(G_m))
-// The codes and scales are read again from memory, four rows per lane at a time.  Each lane rewrites exactly the codes
-// it read; the lowest lane of a key group stores the group's scale.  Codes are rint(S x (1/scale)) with the correctly
-// rounded reciprocal: against rint(S / scale) that moves a code by one step only where the quotient lies within
-// |q| 2^-24 of a rounding boundary (a few codes per million, the same order as the accumulation-order mismatches).
+// The m rank-1 updates run on the matrix core in fp32 (v_mfma_f32_32x32x2_f32: two slots per issue, accumulating on
+// the dequantized old state, slot pairs in order), one 32-row x 32-column block of the state at a time.  The block is
+// held "rows across lanes": lane (j = lane % 32, kb = lane / 32) owns row j's columns 16 kb .. 16 kb + 15 of the
+// block -- accumulator element 4a + b is output row 8a + 4 kb + b of the instruction, and the keys are fed with
+// operand row i = 8a + 4 kb' + b carrying column 16 kb' + 4a + b, so element e of a lane IS column e of its piece.
+// That is the operand shape of the state pass: the codes are read again from memory row-shaped (coalesced), turned
+// into that shape through LDS (the region of lds_k, free once the keys sit in registers), and the new codes go back
+// the same way.  A row's scale group lies in one lane pair (j, 0), (j, 1): absmax = per-lane max + one exchange.
+// Codes are rint(S x (1/scale)) with the correctly rounded reciprocal: against rint(S / scale) that moves a code by
+// one step only where the quotient lies within |q| 2^-24 of a rounding boundary (a few codes per million, the same
+// order as the accumulation-order mismatches).
+typedef float v16f __attribute__((ext_vector_type(16)));
+
 template <class T, bool COLVEC>
-__device__ __forceinline__ void fold_tile(const float* lds_k, const float* lds_u, const float* lds_c, float cmul, int m,
+__device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, const float* lds_c, float cmul, int m,
                                           uint8_t* head, uint16_t* sc_head, const LaneId& l) {
-    constexpr int FR = 4;
+    constexpr int NCS = T::NKS;                              // 32-column steps
+    constexpr int MT = (T::MMAX + 1) / 2;                    // slot pairs
+    constexpr int NL = Window<T>::NL;
+    const int j = l.lane % T::MR, kb = l.lane / T::MR;
     const bool live = l.cg < T::LPR;
-    int gi = (l.cg * CPL) / T::GROUP;
-    const bool has_group = gi < T::NG;
-    gi = has_group ? gi : T::NG - 1;
-    const bool lead = live && (l.cg % T::LPG) == 0 && has_group;
-    uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
-    float colmul[COLVEC ? CPL : 1];
-    if constexpr (COLVEC) lds_piece<T>(lds_c, l.cg, colmul);
-    else colmul[0] = cmul;
-#pragma unroll 1
-    for (int j0 = 0; j0 < T::RPL; j0 += FR) {
-        RawRow<T::BITS> raw[FR];
-        uint16_t scr[FR];
+
+    // keys as matrix operands, for the whole tile: aop[cs][t] = kx_{2t + kb}[32 cs + 16 ((j >> 2) & 1) + 4 (j >> 3) + (j & 3)]
+    float aop[NCS][MT];
+    {
+        const int col = 16 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3);
 #pragma unroll
-        for (int jj = 0; jj < FR; ++jj) {
-            raw[jj] = load_row<T::BITS>(lane_base + (j0 + jj) * (T::RG * T::ROW_BYTES));
-            scr[jj] = sc_head[row_of<T>(l, j0 + jj) * T::NG + gi];
-        }
-        float acc[FR][CPL];
+        for (int cs = 0; cs < NCS; ++cs)
 #pragma unroll
-        for (int jj = 0; jj < FR; ++jj) {
-            float c[CPL];
-            decode_row<T::BITS>(raw[jj], c);
-            const float s = (live && has_group) ? f16_to_f32(scr[jj]) : 0.0f;
-#pragma unroll
-            for (int t = 0; t < CPL; ++t) acc[jj][t] = (c[t] * s) * colmul[COLVEC ? t : 0];
-        }
-#pragma unroll 1
-        for (int i = 0; i < m; ++i) {
-            float kx[CPL];
-            lds_piece<T>(lds_k + i * T::KROW, l.cg, kx);
-#pragma unroll
-            for (int jj = 0; jj < FR; ++jj) {
-                const float du = lds_u[i * T::UROW + row_of<T>(l, j0 + jj)];
-#pragma unroll
-                for (int t = 0; t < CPL; ++t) acc[jj][t] = __builtin_fmaf(du, kx[t], acc[jj][t]);
+            for (int t = 0; t < MT; ++t) {
+                const int slot = 2 * t + kb;
+                const float v = lds_k[(slot < m ? slot : 0) * T::KROW + kpos<T>(32 * cs + col)];
+                aop[cs][t] = slot < m ? v : 0.0f;
             }
+    }
+    __syncthreads();                                         // lds_k becomes the block buffer
+    uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
+    uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
+
+    RawRow<T::BITS> nxt[NL];                                 // the next row block and its scales, requested a block ahead
+    uint16_t scn[T::NG];
+#pragma unroll
+    for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
+#pragma unroll
+    for (int g = 0; g < T::NG; ++g) scn[g] = sc_head[j * T::NG + g];
+
+#pragma unroll 1
+    for (int rb = 0; rb < T::NRB; ++rb) {
+        const int row = rb * T::MR + j;
+        uint16_t scr[T::NG];
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) scr[g] = scn[g];
+        if (live) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                store_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES, nxt[t]);
+        }
+        if (rb + 1 < T::NRB) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                nxt[t] = load_row<T::BITS>(lane_base + ((rb + 1) * T::MR + t * T::RG) * T::ROW_BYTES);
+#pragma unroll
+            for (int g = 0; g < T::NG; ++g) scn[g] = sc_head[(row + T::MR) * T::NG + g];
+        }
+        float bop[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int slot = 2 * t + kb;
+            const float v = lds_u[(slot < m ? slot : 0) * T::UROW + row];
+            bop[t] = slot < m ? v : 0.0f;
+        }
+        __syncthreads();
+
+        v16f acc[NCS];
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) {
+            const int piece = 2 * cs + kb;
+            const RawRow<T::BITS> r = load_row<T::BITS>(blk + j * T::A_PITCH + piece * T::LANE_BYTES);
+            float c[CPL];
+            decode_row<T::BITS>(r, c);
+            const float s = f16_to_f32(scr[(piece * CPL) / T::GROUP]);
+            if constexpr (COLVEC) {
+                float cm[CPL];
+                lds_piece<T>(lds_c, piece, cm);
+#pragma unroll
+                for (int e = 0; e < CPL; ++e) acc[cs][e] = (c[e] * s) * cm[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < CPL; ++e) acc[cs][e] = (c[e] * s) * cmul;
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[cs] = __builtin_amdgcn_mfma_f32_32x32x2f32(aop[cs][t], bop[t], acc[cs], 0, 0, 0);
+        }
+
+        // absmax per scale group: the lane's pieces, then the other half of the row
+        float gmax[T::NG];
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) gmax[g] = 0.0f;
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) {
+            float mx = 0.0f;
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) mx = fmaxf(mx, fabsf(acc[cs][e]));
+            const int g = (cs * T::MK) / T::GROUP;
+            gmax[g] = fmaxf(gmax[g], mx);
+        }
+        float rs[T::NG];
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) {
+            const float other = __shfl_xor(gmax[g], 32);
+            const float sc = fp16_scale(fmaxf(gmax[g], other), T::QMAX);
+            rs[g] = 1.0f / sc;
+            if (kb == 0) sc_head[row * T::NG + g] = f32_to_f16(sc);
         }
 #pragma unroll
-        for (int jj = 0; jj < FR; ++jj) {
-            float amax = 0.0f;
+        for (int cs = 0; cs < NCS; ++cs) {
+            float a16[CPL];
 #pragma unroll
-            for (int t = 0; t < CPL; ++t) amax = fmaxf(amax, fabsf(acc[jj][t]));
-            amax = block_max<T::LPG>(amax);
-            const float s = fp16_scale(amax, T::QMAX);
-            const float r = 1.0f / s;
-            const int row = row_of<T>(l, j0 + jj);
-            if (lead) sc_head[row * T::NG + gi] = f32_to_f16(s);
-            if (live)
-                store_row<T::BITS>(lane_base + (j0 + jj) * (T::RG * T::ROW_BYTES), quantize_row<T::BITS>(acc[jj], r));
+            for (int e = 0; e < CPL; ++e) a16[e] = acc[cs][e];
+            store_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES,
+                               quantize_row<T::BITS>(a16, rs[(cs * T::MK) / T::GROUP]));
         }
+        __syncthreads();
+        if (live) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                store_row<T::BITS>(lane_base + (rb * T::MR + t * T::RG) * T::ROW_BYTES,
+                                   load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
+        }
+        __syncthreads();
     }
 }
 
