@@ -70,11 +70,16 @@ struct LdsPlan {
     static constexpr int X = 0;
     static constexpr int UB = X + NX * T::KROW * 4;
     static constexpr int SC = UB + T::UB_BYTES;
-    static constexpr int B = SC + T::SC_BYTES;
-    static constexpr int XS = B + T::B_BYTES;
-    static constexpr int A = XS + round_up(NV * T::NG * 4, 16);
-    static constexpr int C = A + T::A_BYTES;
-    static constexpr int OWN = C + T::NG * T::PLANES * NV * T::MR * 4;
+    static constexpr int XS = SC + T::SC_BYTES;
+    // one region, three tenants in turn: the digit planes (until the pass has them in registers), then per row block
+    // the codes on their way to operand shape and, once the block's products are issued, its integer sums
+    static constexpr int B = XS + round_up(NV * T::NG * 4, 16);
+    static constexpr int A = B;
+    static constexpr int C = B;
+    static constexpr int C_BYTES = T::NG * T::PLANES * NV * T::MR * 4;
+    static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
+                                                    : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
+    static constexpr int OWN = B + BAC;
     static constexpr int FRONT = OWN + NV * T::UROW * 4;
     static constexpr int FK = 0;
     static constexpr int FU = FK + T::MMAX * T::KROW * 4;
@@ -278,15 +283,24 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
                                            const float* lds_xs, const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c,
                                            float* lds_own, const LaneId& l, float (&own)[NV][T::NOWN]) {
     constexpr int NPL = T::PLANES * NV;
-    static_assert(NPL <= 8 && NV <= 2, "digit planes fill at most 8 operand columns");
+    constexpr int NCOL = NPL * T::NG;                        // result columns in use: (scale group, vector, digit)
+    static_assert(NCOL <= T::MR && NV <= 2, "groups x digit planes must fit the instruction's 32 result columns");
     const int j = l.lane % T::MR, kb = l.lane / T::MR;
+    // second operand, per column step: result column j = g NPL + p takes digit plane p, but only on the column steps
+    // that belong to scale group g (zero elsewhere), so ONE accumulation over all steps leaves every group's sums in
+    // its own columns
+    const int colg = j / NPL, colp = j - colg * NPL;
     v4i bop[T::NKS];
 #pragma unroll
-    for (int ks = 0; ks < T::NKS; ++ks)
-        bop[ks] = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (j & 7)) * CPL);
+    for (int ks = 0; ks < T::NKS; ++ks) {
+        const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (colp & 7)) * CPL);
+        const bool mine = colg == (ks * T::MK) / T::GROUP;
+        bop[ks] = mine ? d : v4i{0, 0, 0, 0};
+    }
     float xs[T::NG];
 #pragma unroll
     for (int g = 0; g < T::NG; ++g) xs[g] = lds_xs[(kb < NV ? kb : 0) * T::NG + g];
+    __syncthreads();                                         // the planes' region now carries the row blocks
 
 #pragma unroll
     for (int rb = 0; rb < T::NRB; ++rb) {
@@ -297,20 +311,17 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
         }
         if (rb + 2 < T::NRB) window_load<T>(lane_base, rb + 2, w);
         __syncthreads();
+        v16i acc = {0};
 #pragma unroll
-        for (int g = 0; g < T::NG; ++g) {
-            v16i acc = {0};
+        for (int ks = 0; ks < T::NKS; ++ks) {
+            const RawRow<T::BITS> r = load_row<T::BITS>(lds_a + j * T::A_PITCH + (2 * ks + kb) * T::LANE_BYTES);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), bop[ks], acc, 0, 0, 0);
+        }
+        __syncthreads();                                     // every lane has its codes: the sums may take their place
+        if (j < NCOL) {
+            int4* dst = reinterpret_cast<int4*>(lds_c + j * T::MR + 4 * kb);
 #pragma unroll
-            for (int ks = 0; ks < T::NKS; ++ks)
-                if ((ks * T::MK) / T::GROUP == g) {
-                    const RawRow<T::BITS> r = load_row<T::BITS>(lds_a + j * T::A_PITCH + (2 * ks + kb) * T::LANE_BYTES);
-                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), bop[ks], acc, 0, 0, 0);
-                }
-            if (j < NPL) {
-                int4* dst = reinterpret_cast<int4*>(lds_c + (g * NPL + j) * T::MR + 4 * kb);
-#pragma unroll
-                for (int a = 0; a < 4; ++a) dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
-            }
+            for (int a = 0; a < 4; ++a) dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
         }
         __syncthreads();
         if (kb < NV) {
