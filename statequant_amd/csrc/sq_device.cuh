@@ -162,8 +162,12 @@ __device__ __forceinline__ RawRow<BITS> zero_row() {
 }
 __device__ __forceinline__ float s8_to_f(uint32_t w, int byte) { return float(int32_t(w << (24 - 8 * byte)) >> 24); }
 
+// fp32 value of a lane's 16 codes, times `unit`.  int4: a stored nibble is code + 8; with bit 3 flipped and moved to
+// the high half of a byte it reads, as a signed byte, 16 x code -- one byte-to-float conversion per code instead of
+// extract, subtract, convert -- and DECODE_UNIT = 1/16 (exact) goes into whatever factor the caller applies next.
+template <int BITS> constexpr float DECODE_UNIT = BITS == 4 ? 0.0625f : 1.0f;
 template <int BITS>
-__device__ __forceinline__ void decode_row(const RawRow<BITS>& r, float (&c)[CPL]) {
+__device__ __forceinline__ void decode_row_scaled(const RawRow<BITS>& r, float (&c)[CPL]) {
     if constexpr (BITS == 8) {
         const uint32_t w[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
 #pragma unroll
@@ -171,11 +175,24 @@ __device__ __forceinline__ void decode_row(const RawRow<BITS>& r, float (&c)[CPL
 #pragma unroll
             for (int b = 0; b < 4; ++b) c[4 * d + b] = s8_to_f(w[d], b);
     } else {
-        const uint32_t w[2] = {r.v.x, r.v.y};
+        const uint32_t w[2] = {r.v.x ^ 0x88888888u, r.v.y ^ 0x88888888u};
 #pragma unroll
-        for (int d = 0; d < 2; ++d)
+        for (int d = 0; d < 2; ++d) {
+            const uint32_t lo = (w[d] << 4) & 0xF0F0F0F0u, hi = w[d] & 0xF0F0F0F0u;     // columns 0,2,4,6 / 1,3,5,7
 #pragma unroll
-            for (int nb = 0; nb < 8; ++nb) c[8 * d + nb] = float(int32_t((w[d] >> (4 * nb)) & 0xFu) - 8);
+            for (int b = 0; b < 4; ++b) {
+                c[8 * d + 2 * b] = s8_to_f(lo, b);
+                c[8 * d + 2 * b + 1] = s8_to_f(hi, b);
+            }
+        }
+    }
+}
+template <int BITS>
+__device__ __forceinline__ void decode_row(const RawRow<BITS>& r, float (&c)[CPL]) {
+    decode_row_scaled<BITS>(r, c);
+    if constexpr (BITS == 4) {
+#pragma unroll
+        for (int t = 0; t < CPL; ++t) c[t] = c[t] * 0.0625f;
     }
 }
 

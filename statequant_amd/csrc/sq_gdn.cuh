@@ -234,16 +234,9 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         const bool valid = owned_valid<T>(l, t);
         int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        float sq = alpha * own[0][t];
-        float sk = alpha * own[1][t];
-#pragma unroll
-        for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
-            if constexpr (T::QBUF) uv = uv * ubs[i];
-            uv = i < n ? uv : 0.0f;                       // dead slots may hold anything: discard
-            sq = __builtin_fmaf(uv, c[0][i], sq);
-            sk = __builtin_fmaf(uv, c[1][i], sk);
-        }
+        float sqk[2] = {alpha * own[0][t], alpha * own[1][t]};
+        buffer_term<T, 2>(lds_ub, ubs, c, n, m, r, sqk);
+        const float sq = sqk[0], sk = sqk[1];
         const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * __builtin_fmaf(-a, sk, vt);
         const float o = __builtin_fmaf(kq, u[t], a * sq);

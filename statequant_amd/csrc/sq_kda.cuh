@@ -149,7 +149,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     __syncthreads();
 
     // ---- buffer coefficients with the per-channel decay ratio folded into the buffered key ----
-    float cq[T::MMAX], ck[T::MMAX];
+    float cqk[2][T::MMAX];
     {
         float xn[2][CPL], gp[CPL];
         lds_piece<T>(lds_q, l.cg, xn[0]);
@@ -179,8 +179,8 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
         }
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) {
-            cq[i] = lane_bcast(cq_l[i / T::RG], (i % T::RG) * T::LPRP);
-            ck[i] = lane_bcast(ck_l[i / T::RG], (i % T::RG) * T::LPRP);
+            cqk[0][i] = lane_bcast(cq_l[i / T::RG], (i % T::RG) * T::LPRP);
+            cqk[1][i] = lane_bcast(ck_l[i / T::RG], (i % T::RG) * T::LPRP);
         }
     }
 
@@ -194,16 +194,9 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
         const bool valid = owned_valid<T>(l, t);
         int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        float sq = own[0][t];
-        float sk = own[1][t];
-#pragma unroll
-        for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
-            if constexpr (T::QBUF) uv = uv * ubs[i];
-            uv = i < n ? uv : 0.0f;
-            sq = __builtin_fmaf(uv, cq[i], sq);
-            sk = __builtin_fmaf(uv, ck[i], sk);
-        }
+        float sqk[2] = {own[0][t], own[1][t]};
+        buffer_term<T, 2>(lds_ub, ubs, cqk, n, m, r, sqk);
+        const float sq = sqk[0], sk = sqk[1];
         const float vt = raw_to_f(vr[t], p.v_dt);
         u[t] = beta * (vt - sk);
         const float o = __builtin_fmaf(kq, u[t], sq);

@@ -149,14 +149,9 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         const bool valid = owned_valid<T>(l, t);
         int r = owned_row<T>(l, t);
         r = r < DV ? r : DV - 1;
-        float sq = alpha * own[0][t];
-#pragma unroll
-        for (int i = 0; i < T::MMAX; ++i) {
-            float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
-            if constexpr (T::QBUF) uv = uv * ubs[i];
-            uv = i < n ? uv : 0.0f;
-            sq = __builtin_fmaf(uv, c[0][i], sq);
-        }
+        float sq1[1] = {alpha * own[0][t]};
+        buffer_term<T, 1>(lds_ub, ubs, c, n, m, r, sq1);
+        const float sq = sq1[0];
         const float xr = valid ? raw_to_f(xr_raw[t], p.x_dt) : 0.0f;
         u[t] = dt * xr;
         float y = __builtin_fmaf(bc, u[t], a * sq);

@@ -471,6 +471,26 @@ __device__ __forceinline__ void buffer_coefs(const KeyBuf<T>& kbuf, const float 
         for (int i = 0; i < T::MMAX; ++i) c[v][i] = lane_bcast(cl[v][i / T::RG], (i % T::RG) * T::LPRP);
 }
 
+// Buffer term of one owned row r: acc[v] += sum_i U_i[r] c[v][i] as an fma chain in slot order (the reference's
+// `_acc`, _fold_triton.py:239-257).  c[v][i] is zero for dead slots (i >= n).  int8 buffer: the slot's scale is folded
+// into the coefficient once per tile (wave-uniform; zero for a dead slot, whose scale may be anything), so a slot
+// costs one conversion and one fma per vector; dead slots hold finite bytes, times zero.  bf16 buffer: dead slots may
+// hold NaNs, so their values are discarded first.
+template <class T, int NV>
+__device__ __forceinline__ void buffer_term(const uint8_t* lds_ub, const float (&ubs)[T::MMAX],
+                                            const float (&c)[NV][T::MMAX], int n, int m, int r, float (&acc)[NV]) {
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) {
+        float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
+        if constexpr (!T::QBUF) uv = i < n ? uv : 0.0f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const float cu = !T::QBUF ? c[v][i] : i < n ? c[v][i] * ubs[i] : 0.0f;       // (a dead slot's scale: anything)
+            acc[v] = __builtin_fmaf(uv, cu, acc[v]);
+        }
+    }
+}
+
 // Append the current token's value row: int8 with one absmax scale over the whole row (`us`, stored by lane 0), or
 // bf16.  ur = the value as stored, dequantized (what the fold must use for slot n).
 template <class T>
@@ -641,16 +661,17 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             const int piece = 2 * cs + kb;
             const RawRow<T::BITS> r = load_row<T::BITS>(blk + j * T::A_PITCH + piece * T::LANE_BYTES);
             float c[CPL];
-            decode_row<T::BITS>(r, c);
-            const float s = f16_to_f32(scr[(piece * CPL) / T::GROUP]);
+            decode_row_scaled<T::BITS>(r, c);
+            const float s = f16_to_f32(scr[(piece * CPL) / T::GROUP]) * DECODE_UNIT<T::BITS>;     // exact
             if constexpr (COLVEC) {
                 float cm[CPL];
                 lds_piece<T>(lds_c, piece, cm);
 #pragma unroll
                 for (int e = 0; e < CPL; ++e) acc[cs][e] = (c[e] * s) * cm[e];
             } else {
+                const float sm = s * cmul;                   // one rounding more than (code x scale) x decay
 #pragma unroll
-                for (int e = 0; e < CPL; ++e) acc[cs][e] = (c[e] * s) * cmul;
+                for (int e = 0; e < CPL; ++e) acc[cs][e] = c[e] * sm;
             }
 #pragma unroll
             for (int t = 0; t < MT; ++t)
