@@ -11,6 +11,8 @@
  *                   slots.py:178-187 (slot-addressed)
  *   sq_kda_step     _kda_triton.py:38 `_kda_step`, launched from kda.py:192-205
  *   sq_mamba2_step  _mamba2_triton.py:48 `_m2_step`, launched from mamba2.py:223-241
+ *   sq_pack_vk      fold.py:123-147 `pack_vk` / slots.py:236-252 `write` (torch in the reference)
+ *   sq_read         slots.py:210-233, kda.py:351-372 `read` (torch in the reference)
  * The argument convention is the reference's (_fold_triton.py:30-36): every per-sequence tensor comes as a base
  * pointer plus its per-sequence stride IN ELEMENTS of that tensor's type; batch row b works on sequence idx[b]
  * (idx == NULL: sequence b); rows with idx[b] <= 0 are padding: their output row is zeroed, nothing else is touched.
@@ -24,7 +26,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 1
+#define SQ_ABI_VERSION 2
 
 enum { SQ_F32 = 0, SQ_BF16 = 1, SQ_F16 = 2 };                /* dtype codes of float tensors */
 
@@ -129,6 +131,34 @@ typedef struct sq_mamba2_args {
     void* out;          int64_t s_out;   int32_t out_dtype;
 } sq_mamba2_args;
 
+/* Store fp32 states in the packed format (fold.py:123-147 `pack_vk`; with idx, GCUR and NPTR given this is
+ * slots.py:236-252 `SlotLayout.write`: the states go into sequences idx[b] and those sequences' buffers are emptied).
+ * src [rows, hv, dv, dk] value-major fp32, row stride s_src in elements; codes / scales as in sq_state.
+ * Uses lay.bits, axis_k, group, hv, dk, dv.  GCUR / NPTR may be NULL (left alone); gcur_per_head = 1 (GDN, Mamba2)
+ * or dk (KDA).  Rows with idx[b] <= 0 are skipped. */
+typedef struct sq_pack_args {
+    sq_layout lay;
+    int32_t rows;
+    const int32_t* idx;
+    const float* src;   int64_t s_src;
+    void* S;            int64_t sS;
+    void* SC;           int64_t sSC;
+    float* GCUR;        int64_t sGC;     int32_t gcur_per_head;
+    int32_t* NPTR;      int64_t sN;
+} sq_pack_args;
+
+/* The current state of sequences idx[b] as fp32 value-major [rows, hv, dv, dk] (row stride s_out in elements): the
+ * stored state advanced across its pending buffer, a_n S_0 + sum_{i<n} (a_n / a_i) u_i k_i^T (slots.py:210-233;
+ * kda = 1: decays per key channel, kda.py:351-372).  Nothing is modified.  Rows with idx[b] <= 0 are skipped. */
+typedef struct sq_read_args {
+    sq_state st;
+    sq_layout lay;
+    int32_t kda;
+    int32_t rows;
+    const int32_t* idx;
+    float* out;         int64_t s_out;
+} sq_read_args;
+
 int sq_abi_version(void);
 const char* sq_strerror(int code);
 const char* sq_last_error(void);
@@ -139,6 +169,8 @@ int sq_supported(int family, const sq_layout* lay);
 int sq_gdn_step(const sq_gdn_args* args, void* stream);
 int sq_kda_step(const sq_kda_args* args, void* stream);
 int sq_mamba2_step(const sq_mamba2_args* args, void* stream);
+int sq_pack_vk(const sq_pack_args* args, void* stream);
+int sq_read(const sq_read_args* args, void* stream);
 
 #ifdef __cplusplus
 }

@@ -71,9 +71,30 @@ struct Mamba2Params : LayoutKey {
     int out_dt;
 };
 
+struct PackParams {
+    int bits, group, hv, dk, dv;
+    int rows;
+    const int32_t* idx;
+    const float* src;  uint32_t s_src;            // [rows, hv, dv, dk] fp32, row stride in elements
+    uint8_t* S;        uint32_t sS;
+    uint16_t* SC;      uint32_t sSC;
+    float* GCUR;       uint32_t sGC;  int gcur_per_head;      // optional (null: leave)
+    int32_t* NPTR;     uint32_t sN;
+};
+
+struct ReadParams : LayoutKey {
+    StatePtrs st;
+    int kda;                                      // decays per key channel (GB [hv, m, dk], GCUR [hv, dk])
+    int rows;
+    const int32_t* idx;
+    float* out;        uint32_t s_out;            // [rows, hv, dv, dk] fp32, row stride in elements
+};
+
 // hipError_t of the launch (0 = enqueued), or -1 if no kernel is compiled for the layout.  run = false: probe only.
 int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
 int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
 int dispatch_mamba2(const Mamba2Params& p, hipStream_t stream, bool run);
+int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
+int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
 
 }  // namespace sq

@@ -13,14 +13,15 @@ import torch
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, 'libsqhip.so')
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 F32, BF16, F16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 FAMILY = {'gdn': 0, 'kda': 1, 'mamba2': 2}
 
 SYMBOLS = ('sq_abi_version', 'sq_strerror', 'sq_last_error', 'sq_supported', 'sq_gdn_step', 'sq_kda_step',
-           'sq_mamba2_step')
+           'sq_mamba2_step', 'sq_pack_vk', 'sq_read')
+E_UNSUPPORTED = -2
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
 
@@ -73,6 +74,17 @@ class SqMamba2Args(C.Structure):
                 ('out', _vp), ('s_out', _i64), ('out_dtype', _i32)]
 
 
+class SqPackArgs(C.Structure):
+    _fields_ = [('lay', SqLayout), ('rows', _i32), ('idx', _vp), ('src', _vp), ('s_src', _i64),
+                ('S', _vp), ('sS', _i64), ('SC', _vp), ('sSC', _i64),
+                ('GCUR', _vp), ('sGC', _i64), ('gcur_per_head', _i32), ('NPTR', _vp), ('sN', _i64)]
+
+
+class SqReadArgs(C.Structure):
+    _fields_ = [('st', SqState), ('lay', SqLayout), ('kda', _i32), ('rows', _i32), ('idx', _vp),
+                ('out', _vp), ('s_out', _i64)]
+
+
 _lib = None
 
 
@@ -90,7 +102,8 @@ def lib():
         L.sq_last_error.restype = C.c_char_p
         L.sq_supported.restype = C.c_int
         L.sq_supported.argtypes = [C.c_int, C.POINTER(SqLayout)]
-        for name, T in (('sq_gdn_step', SqGdnArgs), ('sq_kda_step', SqKdaArgs), ('sq_mamba2_step', SqMamba2Args)):
+        for name, T in (('sq_gdn_step', SqGdnArgs), ('sq_kda_step', SqKdaArgs), ('sq_mamba2_step', SqMamba2Args),
+                        ('sq_pack_vk', SqPackArgs), ('sq_read', SqReadArgs)):
             f = getattr(L, name)
             f.restype = C.c_int
             f.argtypes = [C.POINTER(T), C.c_void_p]
@@ -138,6 +151,36 @@ def check(rc):
     if rc != 0:
         L = lib()
         raise RuntimeError(f'libsqhip: {L.sq_strerror(rc).decode()}: {L.sq_last_error().decode()}')
+
+
+def pack_into(lay, src, S, sS, SC, sSC, idx=None, GCUR=None, sGC=0, gcur_per_head=1, NPTR=None, sN=0):
+    """``sq_pack_vk``: fp32 value-major ``src`` [rows, hv, dv, dk] (contiguous) -> codes ``S`` / scales ``SC`` of the
+    sequences ``idx`` (int32; None: sequence b), optionally emptying their buffers.  Returns False when the library has
+    no instance for the format (the caller then packs with torch), raises on any other error."""
+    assert src.dtype == torch.float32 and src.is_contiguous()
+    rows = src.shape[0]
+    a = SqPackArgs(lay=lay, rows=rows, idx=ptr(idx), src=src.data_ptr(), s_src=src.stride(0) if rows else 0,
+                   S=S.data_ptr(), sS=sS, SC=SC.data_ptr(), sSC=sSC, GCUR=ptr(GCUR), sGC=sGC,
+                   gcur_per_head=gcur_per_head, NPTR=ptr(NPTR), sN=sN)
+    rc = lib().sq_pack_vk(C.byref(a), current_stream(src.device))
+    if rc == E_UNSUPPORTED:
+        return False
+    check(rc)
+    return True
+
+
+def read_state(lay, T, strides, nptr_stride, idx, out, kda):
+    """``sq_read``: the current state of sequences ``idx`` (int32) into fp32 ``out`` [rows, hv, dv, dk] (contiguous).
+    Returns False when the library has no instance for the layout."""
+    assert out.dtype == torch.float32 and out.is_contiguous()
+    rows = out.shape[0]
+    a = SqReadArgs(st=make_state(T, strides, nptr_stride), lay=lay, kda=int(kda), rows=rows, idx=ptr(idx),
+                   out=out.data_ptr(), s_out=out.stride(0) if rows else 0)
+    rc = lib().sq_read(C.byref(a), current_stream(out.device))
+    if rc == E_UNSUPPORTED:
+        return False
+    check(rc)
+    return True
 
 
 def require_gpu(t, what):

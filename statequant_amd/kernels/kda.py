@@ -195,6 +195,9 @@ class KDASlotLayout(SlotLayout):
     def read(self, views, idx):
         """The current state of slots ``idx`` as fp32 [P, H, d_v, d_k]: diag(alpha_n) S_0 +
         sum_{i<n} diag(alpha_n / alpha_i) k_i u_i^T (value-major) (kda.py:351-372)."""
+        out = self._read_hip(views, idx, kda=True)
+        if out is not None:
+            return out
         idx = idx.long()
         m = self.m
         S0 = self._stored(views, idx)

@@ -189,7 +189,7 @@ class SlotLayout:
         _hip.check(_hip.lib().sq_gdn_step(ctypes.byref(a), _hip.current_stream(out.device)))
         return out
 
-    # -- prefill side (torch, as in the reference) --------------------------------------------------------------
+    # -- prefill side: HIP kernels for the formats the step supports, else torch as in the reference -------------
     def _buffer(self, views, idx):
         """Dequantized buffer of slots idx: keys [P, HK, m, DK], values [P, HV, m, DV], fill counts [P]."""
         V = views
@@ -207,11 +207,28 @@ class SlotLayout:
         sc = V['SC'][idx].reshape(P * self.HV, *V['SC'].shape[2:]) if 'SC' in V else None
         return unpack_vk(codes, sc, self.fmt, self.DK).view(P, self.HV, self.DV, self.DK)
 
+    def _hip_format(self, views):
+        """Key-axis int4 / int8 states on the GPU go through the HIP pack / read kernels; the unpacked and value-axis
+        formats (layout-only here) keep the reference's torch formulation."""
+        return self.fmt is not None and self.axk and views['S'].is_cuda
+
+    def _read_hip(self, views, idx, kda):
+        if not self._hip_format(views) or idx.shape[0] == 0:
+            return None
+        P = idx.shape[0]
+        out = torch.empty(P, self.HV, self.DV, self.DK, device=idx.device, dtype=torch.float32)
+        T, strides, sN = slot_state(views)
+        ok = _hip.read_state(_hip.make_layout(self), T, strides, sN, idx.to(torch.int32).contiguous(), out, kda)
+        return out if ok else None
+
     @torch.no_grad()
     def read(self, views, idx):
         """The current state of slots ``idx`` as fp32 [P, HV, d_v, d_k]: the stored state advanced across its
         pending buffer, S_n = a_n S_0 + sum_{i<n} (a_n/a_i) u_i k_i^T (slots.py:210-233).  Entries of dead buffer
         slots are discarded with ``where`` (they may hold anything)."""
+        out = self._read_hip(views, idx, kda=False)
+        if out is not None:
+            return out
         idx = idx.long()
         m = self.m
         S0 = self._stored(views, idx)
@@ -229,9 +246,16 @@ class SlotLayout:
     def write(self, views, idx, S):
         """Store states S [P, HV, d_v, d_k] (value-major) packed into slots ``idx`` and empty their buffers
         (n = 0, running decay 0) (slots.py:236-252)."""
-        idx = idx.long()
         P = idx.shape[0]
         V = views
+        if self._hip_format(views) and P:
+            src = S.reshape(P, self.HV, self.DV, self.DK).float().contiguous()
+            gc = V['GCUR']
+            if _hip.pack_into(_hip.make_layout(self), src, V['S'], V['S'].stride(0), V['SC'], V['SC'].stride(0),
+                              idx=idx.to(torch.int32).contiguous(), GCUR=gc, sGC=gc.stride(0),
+                              gcur_per_head=gc[0].numel() // self.HV, NPTR=V['NPTR'], sN=V['NPTR'].stride(0)):
+                return
+        idx = idx.long()
         if self.fmt is None and self.state_dtype == torch.float32:
             V['S'][idx] = S.reshape(P, *V['S'].shape[1:]).float()
         else:

@@ -1,0 +1,124 @@
+"""The HIP pack (`sq_pack_vk`: ``pack_vk`` / ``SlotLayout.write``) and read (`sq_read`: ``SlotLayout.read``) kernels
+against the CPU oracle.  pack / write: bit-exact (same IEEE divisions and rounding as the reference's torch code,
+fold.py:123-147, slots.py:236-252).  read: fp32 sums in another order than torch's einsum -> 1e-5 relative.
+"""
+import pytest
+import torch
+
+import statequant_amd as sq
+from oracle import formats as OF
+from oracle import slots as OS
+from statequant_amd.kernels import KDASlotLayout, Mamba2SlotLayout, SlotLayout, pack_vk
+from tests._util import gdn_token, quantizer
+from tests.test_kda_gpu import kda_token
+from tests.test_mamba2_gpu import m2_token, params
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32)])
+@pytest.mark.parametrize('dv,dk', [(128, 128), (64, 64), (192, 96), (96, 96)])
+def test_pack_matches_oracle(fmt, dv, dk):
+    if fmt[2] > (1 << (dk - 1).bit_length()):
+        pytest.skip('group longer than the padded row')
+    gen = torch.Generator().manual_seed(dv + dk + fmt[0] + fmt[2])
+    x = torch.randn(37, dv, dk, generator=gen)
+    x[0] = 0.0                                             # all-zero heads: scale floor, codes 0
+    x[1, :, : dk // 2] = 0.0                               # zero groups next to live ones
+    x[2] *= 1e-6                                           # scales in the fp16 subnormal range
+    x[3] *= 1e4
+    x[4, 5] = 65504.0 * 127                                # scale at the top of fp16
+    codes, sc = pack_vk(x.to(DEV), quantizer(fmt))
+    want_c, want_s = OF.pack_vk(x, fmt)
+    assert codes.dtype == want_c.dtype and codes.shape == want_c.shape and sc.shape == want_s.shape
+    assert torch.equal(sc.cpu(), want_s)
+    assert torch.equal(codes.cpu(), want_c)
+
+
+def _blob_pair(lay, table_args, n_slots, seed):
+    gen = torch.Generator().manual_seed(seed)
+    table, nbytes = OS.layout(*table_args)
+    assert nbytes == lay.nbytes
+    raw = torch.randint(0, 256, (n_slots, lay.nbytes), dtype=torch.uint8, generator=gen)
+    dev = raw.to(DEV)
+    return gen, table, raw, dev
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 64), (4, 'k', 32)])
+def test_write_matches_oracle_whole_blob(fmt):
+    HV, HK, D, m = 4, 2, 128, 8
+    lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=8)
+    gen, table, raw, dev = _blob_pair(lay, ('gdn', fmt, HV, HK, D, D, m, 8), 9, 1)
+    idx = torch.tensor([7, 2, 5])
+    S = torch.randn(3, HV, D, D, generator=gen)
+    lay.write(lay.views(dev), idx.to(DEV), S.to(DEV))
+    OS.write(OS.views(table, raw), idx, S, fmt, HV, D, D)
+    assert torch.equal(dev.cpu(), raw)                    # codes, scales, counters, decays -- and nothing else
+
+
+def _advance(lay, views, step_fn, schedule):
+    """Run decode steps so that the slots end with different buffer fills (schedule: list of slot lists)."""
+    for live in schedule:
+        step_fn(torch.tensor(live, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize('fmt,bb', [((8, 'k', 128), 8), ((4, 'k', 32), 16)])
+def test_gdn_read_matches_oracle(fmt, bb):
+    HV, HK, D, m = 4, 2, 128, 8
+    lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=bb)
+    gen, table, raw, dev = _blob_pair(lay, ('gdn', fmt, HV, HK, D, D, m, bb), 6, 2)
+    views = lay.views(dev)
+    slots = torch.tensor([1, 3, 4, 5])
+    lay.write(views, slots.to(DEV), (torch.randn(4, HV, D, D, generator=gen) * 0.5).to(DEV))
+
+    def step(idx):
+        B = idx.shape[0]
+        q, k, v, g, beta = (x.to(DEV) for x in gdn_token(gen, B, HV, HK, D, D))
+        lay.step(views, idx, q, k, v, torch.empty(B, HV, D, device=DEV), D ** -0.5, g=g, beta=beta)
+
+    _advance(lay, views, step, [[1, 3, 4]] * 3 + [[3, 4]] * 2 + [[4]] * 5)         # fills 3, 5, 10 % 8 = 2, 0
+    got = lay.read(views, slots.to(DEV)).cpu()
+    want = OS.read(OS.views(table, dev.cpu()), slots, fmt, HV, HK, D, D, m)
+    assert (views['NPTR'][slots.to(DEV), 0].cpu() & (m - 1)).tolist() == [3, 5, 2, 0]
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())
+
+
+def test_kda_read_matches_oracle():
+    H, DK, DV, m, fmt = 4, 128, 128, 8, (4, 'k', 32)
+    lay = KDASlotLayout(quantizer(fmt), H, DK, DV, m=m, buffer_bits=8)
+    gen, table, raw, dev = _blob_pair(lay, ('kda', fmt, H, H, DK, DV, m, 8), 5, 3)
+    views = lay.views(dev)
+    slots = torch.tensor([2, 4, 1])
+    lay.write(views, slots.to(DEV), (torch.randn(3, H, DV, DK, generator=gen) * 0.5).to(DEV))
+    assert torch.equal(views['GCUR'][slots.to(DEV)].cpu(), torch.zeros(3, H, DK))
+
+    def step(idx):
+        B = idx.shape[0]
+        q, k, v, g, beta = (x.to(DEV) for x in kda_token(gen, B, H, DK, DV))
+        lay.step(views, idx, q, k, v, g, beta, torch.empty(B, H, DV, device=DEV))
+
+    _advance(lay, views, step, [[2, 4]] * 4 + [[4]] * 3)
+    got = lay.read(views, slots.to(DEV)).cpu()
+    want = OS.read(OS.views(table, dev.cpu()), slots, fmt, H, H, DK, DV, m, per_channel=True)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())
+
+
+def test_mamba2_read_matches_oracle():
+    H, G, DK, DV, m, fmt = 8, 2, 128, 64, 8, (8, 'k', 128)
+    lay = Mamba2SlotLayout(quantizer(fmt), H, G, DK, DV, m=m, buffer_bits=8)
+    gen, table, raw, dev = _blob_pair(lay, ('mamba2', fmt, H, G, DK, DV, m, 8), 5, 4)
+    views = lay.views(dev)
+    slots = torch.tensor([3, 1])
+    lay.write(views, slots.to(DEV), (torch.randn(2, H, DV, DK, generator=gen) * 0.5).to(DEV))
+    A, D, dtb = (t.to(DEV) for t in params(gen, H))
+
+    def step(idx):
+        B = idx.shape[0]
+        x, dt, Bm, C = (t.to(DEV) for t in m2_token(gen, B, H, G, DK, DV))
+        lay.step(views, idx, x, dt, Bm, C, torch.empty(B, H, DV, device=DEV), A, D, dtb)
+
+    _advance(lay, views, step, [[3, 1]] * 2 + [[1]] * 4)
+    got = lay.read(views, slots.to(DEV)).cpu()
+    want = OS.read(OS.views(table, dev.cpu()), slots, fmt, H, G, DK, DV, m)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())

@@ -148,7 +148,7 @@ def test_library_exports_every_declared_symbol():
     L = _hip.lib()
     for name in declared:
         assert hasattr(L, name), name
-    assert L.sq_abi_version() == 1
+    assert L.sq_abi_version() == _hip.ABI_VERSION == 2
     assert L.sq_strerror(0) == b'ok'
     lay = _hip.SqLayout(bits=8, axis_k=1, group=128, buffer_bits=8, m=8, hv=32, hk=16, dk=128, dv=128)
     assert L.sq_supported(0, ctypes.byref(lay)) == 1
@@ -164,7 +164,8 @@ def test_ctypes_structs_match_the_header():
     """Field order of the ctypes mirrors == the C structs (a reordering would silently shift every pointer)."""
     header = open(os.path.join(ROOT, 'include', 'statequant_hip.h')).read()
     for cname, S in (('sq_state', _hip.SqState), ('sq_layout', _hip.SqLayout), ('sq_gdn_args', _hip.SqGdnArgs),
-                     ('sq_kda_args', _hip.SqKdaArgs), ('sq_mamba2_args', _hip.SqMamba2Args)):
+                     ('sq_kda_args', _hip.SqKdaArgs), ('sq_mamba2_args', _hip.SqMamba2Args),
+                     ('sq_pack_args', _hip.SqPackArgs), ('sq_read_args', _hip.SqReadArgs)):
         body = re.search(r'typedef struct %s \{(.*?)\} %s;' % (cname, cname), header, flags=re.S).group(1)
         body = re.sub(r'/\*.*?\*/', '', body, flags=re.S)
         names = []
