@@ -159,6 +159,50 @@ def calibrate_copy(dev, nbytes=1 << 30, reps=20):
                       'us_per_copy': round(us, 2), 'gbs_read_plus_write': round(2 * nbytes / us * 1e-3, 1)}))
 
 
+def bench_convert(a, lay, views, idx, dev):
+    """`SlotLayout.write` (fp32 state -> codes + scales, buffers emptied) or `.read` (stored state advanced across
+    the pending buffer -> fp32) over all slots of every layer blob; one launch per layer.  Algorithmic bytes: the fp32
+    state on one side (4 bytes per code) plus codes and scales on the other."""
+    fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
+    S = torch.randn(slots, hv, dv, dk, device=dev) * 0.3
+    idl = idx.long()
+    for V in views:                                         # a defined state with a partly filled buffer
+        lay.write(V, idl, S)
+        V['NPTR'][idl] = 3
+        V['GB'][idl] = -torch.rand_like(V['GB'][idl])
+        V['GCUR'][idl] = -torch.rand_like(V['GCUR'][idl]) - 1.0
+        V['KB'][idl] = torch.randint(-100, 100, V['KB'][idl].shape, device=dev).to(V['KB'].dtype)
+        V['UB'][idl] = torch.randint(-100, 100, V['UB'][idl].shape, device=dev).to(V['UB'].dtype)
+        V['KBS'][idl] = 0.01
+        V['UBS'][idl] = 0.01
+    run = (lambda V: lay.write(V, idl, S)) if a.op == 'write' else (lambda V: lay.read(V, idl))
+    reps = max(a.steps // 64, 4)
+    for V in views:
+        run(V)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(reps):
+        for V in views:
+            run(V)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    n = reps * layers
+    us = e0.elapsed_time(e1) * 1e3 / n
+    codes = hv * dv * dk * bits // 8 + hv * dv * (-(-dk // group)) * 2
+    alg = slots * (hv * dv * dk * 4 + codes)
+    print(json.dumps({
+        'metric': f'us_per_layer_{a.op}', 'value': round(wall * 1e6 / n, 3), 'unit': 'us', 'n_gpus': 1, 'steps': reps,
+        'warmup': 1, 'higher_is_better': False, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': a.workload, 'op': a.op, 'slots': slots, 'layers': layers,
+                   'includes': 'host-side index conversion and output allocation of SlotLayout.' + a.op},
+        'roofline': {'bound': 'hbm', 'achieved': round(alg / us * 1e-3, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                     'frac': round(alg / us * 1e-3 / HBM_PEAK_GBS, 4), 'traffic': None, 'kernel_us': round(us, 3),
+                     'algorithmic_bytes_per_launch': alg}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -169,6 +213,9 @@ def main():
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-budget', type=float, default=20.0)
+    ap.add_argument('--op', default='step', choices=['step', 'write', 'read'],
+                    help="step: the decode step (the headline); write / read: the prefill-side pack and read kernels "
+                         "on the same slots (SlotLayout.write / .read)")
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='instead of the workload, run plain device copies of 1 GiB (the known-size kernel that '
                          'rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by) and print their rate')
@@ -185,6 +232,8 @@ def main():
     m = a.m
     fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
     fam, lay, views, idx = build(a.workload, m, dev)
+    if a.op != 'step':
+        return bench_convert(a, lay, views, idx, dev)
     inputs, extra = make_inputs(fam, lay, slots, layers, m, dev)
     out = torch.empty(slots, hv, dv, device=dev, dtype=torch.bfloat16)
 

@@ -133,27 +133,38 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     int gi = (l.cg * CPL) / GROUP;
     const bool has_group = gi < T::NG;
     gi = has_group ? gi : T::NG - 1;
-    for (uint32_t r0 = 0; r0 < dv; r0 += T::RG) {
-        const uint32_t row = r0 + l.rg;
-        const uint32_t rc = row < dv ? row : dv - 1;
-        float c[CPL];
-        decode_row<BITS>(load_row<BITS>(Sh + rc * T::ROW_BYTES + cc * T::LANE_BYTES), c);
-        const float s = has_group ? f16_to_f32(SCh[rc * T::NG + gi]) : 0.0f;
-        float acc[CPL];
+    constexpr int RR = 2;                                         // rows per pass over the buffered keys
+    for (uint32_t r0 = 0; r0 < dv; r0 += RR * T::RG) {
+        uint32_t row[RR], rc[RR];
+        float acc[RR][CPL];
 #pragma unroll
-        for (int t = 0; t < CPL; ++t) acc[t] = alpha_p[t] * (c[t] * s);
-        for (int i = 0; i < m; ++i) {
+        for (int k = 0; k < RR; ++k) {
+            row[k] = r0 + k * T::RG + l.rg;
+            rc[k] = row[k] < dv ? row[k] : dv - 1;
+            float c[CPL];
+            decode_row<BITS>(load_row<BITS>(Sh + rc[k] * T::ROW_BYTES + cc * T::LANE_BYTES), c);
+            const float s = has_group ? f16_to_f32(SCh[rc[k] * T::NG + gi]) : 0.0f;
+#pragma unroll
+            for (int t = 0; t < CPL; ++t) acc[k][t] = alpha_p[t] * (c[t] * s);
+        }
+        for (int i = 0; i < n; ++i) {                             // live slots only
             float kx[CPL];
             lds_piece<T>(lds_k + i * T::KROW, l.cg, kx);
-            const float du = lds_u[i * dv + rc];
 #pragma unroll
-            for (int t = 0; t < CPL; ++t) acc[t] = __builtin_fmaf(du, kx[t], acc[t]);
-        }
-        if (row < dv && live) {
-            float4* o4 = reinterpret_cast<float4*>(out + row * DK + l.cg * CPL);
+            for (int k = 0; k < RR; ++k) {
+                const float du = lds_u[i * dv + rc[k]];
 #pragma unroll
-            for (int t = 0; t < CPL / 4; ++t) o4[t] = make_float4(acc[4 * t], acc[4 * t + 1], acc[4 * t + 2], acc[4 * t + 3]);
+                for (int t = 0; t < CPL; ++t) acc[k][t] = __builtin_fmaf(du, kx[t], acc[k][t]);
+            }
         }
+#pragma unroll
+        for (int k = 0; k < RR; ++k)
+            if (row[k] < dv && live) {
+                float4* o4 = reinterpret_cast<float4*>(out + row[k] * DK + l.cg * CPL);
+#pragma unroll
+                for (int t = 0; t < CPL / 4; ++t)
+                    o4[t] = make_float4(acc[k][4 * t], acc[k][4 * t + 1], acc[k][4 * t + 2], acc[k][4 * t + 3]);
+            }
     }
 }
 
