@@ -71,7 +71,8 @@ int check_state(const sq_state& s, const sq_layout& L, const char* who, sq::Stat
         return fail(SQ_E_ARG, "%s: int8 key buffer must be 16-byte aligned (base and per-sequence stride)", who);
     // scales and buffered values are staged into LDS with 128-bit loads
     if (!aligned(s.SC, 16) || (s.sSC % 8) || !aligned(s.UB, 16) || ((s.sUB * (L.buffer_bits / 8)) % 16))
-        return fail(SQ_E_ARG, "%s: scales and value buffer must be 16-byte aligned (base and per-sequence stride)", who);
+        return fail(SQ_E_ARG, "%s: scales and value buffer must be 16-byte aligned (base and per-sequence stride)",
+                    who);
     if (!aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
         return fail(SQ_E_ARG, "%s: misaligned decay / counter pointer", who);
     if (!stride_ok(s.sS) || !stride_ok(s.sSC) || !stride_ok(s.sKB) || !stride_ok(s.sKBS) || !stride_ok(s.sUB) ||
@@ -155,12 +156,14 @@ int sq_gdn_step(const sq_gdn_args* a, void* stream) {
     if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->out_dtype))
         return fail(SQ_E_ARG, "%s: bad dtype code", who);
     if (a->gate) {
-        if (!a->a || !a->b || !a->A_log || !a->dt_bias) return fail(SQ_E_ARG, "%s: gate without a / b / A_log / dt_bias", who);
+        if (!a->a || !a->b || !a->A_log || !a->dt_bias)
+            return fail(SQ_E_ARG, "%s: gate without a / b / A_log / dt_bias", who);
         if (!dtype_ok(a->a_dtype) || !dtype_ok(a->b_dtype) || !dtype_ok(a->A_log_dtype) || !dtype_ok(a->dt_bias_dtype))
             return fail(SQ_E_ARG, "%s: bad gate dtype code", who);
     } else {
         if (!a->g || !a->beta) return fail(SQ_E_ARG, "%s: neither g / beta nor a gate", who);
-        if (!dtype_ok(a->g_dtype) || !dtype_ok(a->beta_dtype)) return fail(SQ_E_ARG, "%s: bad g / beta dtype code", who);
+        if (!dtype_ok(a->g_dtype) || !dtype_ok(a->beta_dtype))
+            return fail(SQ_E_ARG, "%s: bad g / beta dtype code", who);
     }
     if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) ||
         !stride_ok(a->gate ? a->s_a : a->s_g) || !stride_ok(a->gate ? a->s_b : a->s_beta))
@@ -194,7 +197,8 @@ int sq_kda_step(const sq_kda_args* a, void* stream) {
     if (!a) return fail(SQ_E_ARG, "%s: null args", who);
     sq::KdaParams p{};
     SQ_TRY(check_layout(a->lay, who, &p));
-    if (a->lay.hk != a->lay.hv) return fail(SQ_E_ARG, "%s: KDA has no grouped keys (hk %d != hv %d)", who, a->lay.hk, a->lay.hv);
+    if (a->lay.hk != a->lay.hv)
+        return fail(SQ_E_ARG, "%s: KDA has no grouped keys (hk %d != hv %d)", who, a->lay.hk, a->lay.hv);
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;
     SQ_TRY(check_state(a->st, a->lay, who, &p.st));
@@ -294,7 +298,8 @@ int sq_read(const sq_read_args* a, void* stream) {
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;
     SQ_TRY(check_state(a->st, a->lay, who, &p.st));
-    if (a->kda && (!aligned(a->st.GB, 4) || !aligned(a->st.GCUR, 4))) return fail(SQ_E_ARG, "%s: misaligned decay", who);
+    if (a->kda && (!aligned(a->st.GB, 4) || !aligned(a->st.GCUR, 4)))
+        return fail(SQ_E_ARG, "%s: misaligned decay", who);
     if (!a->out || !aligned(a->out, 16) || (a->s_out % 4) || !stride_ok(a->s_out))
         return fail(SQ_E_ARG, "%s: out must be 16-byte aligned with a row stride in [0, 2^31)", who);
     p.kda = a->kda != 0;

@@ -171,7 +171,10 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
                 for (int e = 0; e < 4; ++e) {
                     const float kd = alive ? kb[4 * k + e] * expf(gp[4 * k + e] - gv[e]) : 0.0f;
                     if (k == 0 && e == 0) { pq = kd * xn[0][0]; pk = kd * xn[1][0]; }
-                    else { pq = __builtin_fmaf(kd, xn[0][4 * k + e], pq); pk = __builtin_fmaf(kd, xn[1][4 * k + e], pk); }
+                    else {
+                        pq = __builtin_fmaf(kd, xn[0][4 * k + e], pq);
+                        pk = __builtin_fmaf(kd, xn[1][4 * k + e], pk);
+                    }
                 }
             }
             cq_l[t] = block_sum<T::LPRP>(pq);

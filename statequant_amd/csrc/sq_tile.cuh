@@ -13,10 +13,11 @@
 // accumulation error.
 //
 // Resource plan (what keeps four wavefronts per SIMD resident): the codes stream through a window of two 32-row
-// blocks per wavefront (32 VGPRs for int8), refilled block by block; the small operands (buffered values, scales)
-// are fetched with one coalesced 128-bit load per lane and parked in LDS until needed; the fold reads the codes a
-// second time (from L2 / Infinity Cache: they were read microseconds earlier) instead of pinning them in registers;
-// the fold's LDS operands overlay the front end's.
+// blocks per wavefront (32 VGPRs for int8), loaded row-shaped (whole rows per instruction) and turned into matrix
+// operands through one 4.6 KB LDS block, refilled block by block; the small operands (buffered values, scales) are
+// fetched with one coalesced 128-bit load per lane and parked in LDS until needed; the fold reads the codes a second
+// time instead of pinning them on chip (16 KB per wavefront, more than registers or LDS can spare at this occupancy)
+// and runs its rank-1 updates on the matrix core in fp32; the fold's LDS operands overlay the front end's.
 #pragma once
 #include "sq_device.cuh"
 
@@ -64,7 +65,8 @@ struct Tile {
 
 // LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
 // vectors, the raw buffered values, the raw scales, the digit planes with their exponents, one row block of codes,
-// its integer sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
+// its integer sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay
+// each other.
 template <class T, int NX, int NV = 2>
 struct LdsPlan {
     static constexpr int X = 0;
@@ -235,7 +237,8 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
                 at[0] = uint8_t(d);
                 at[CPL] = uint8_t(d >> 8);
                 at[2 * CPL] = uint8_t(d >> 16);
-                if (e % T::GROUP == 0) lds_xs[v * T::NG + e / T::GROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
+                if (e % T::GROUP == 0)
+                    lds_xs[v * T::NG + e / T::GROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
             }
         }
     }
@@ -321,7 +324,8 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
         if (j < NCOL) {
             int4* dst = reinterpret_cast<int4*>(lds_c + j * T::MR + 4 * kb);
 #pragma unroll
-            for (int a = 0; a < 4; ++a) dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+            for (int a = 0; a < 4; ++a)
+                dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
         }
         __syncthreads();
         if (kb < NV) {
@@ -330,7 +334,8 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 #pragma unroll
             for (int g = 0; g < T::NG; ++g) {
                 const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
-                const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f, __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
+                const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
+                                               __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
                 const float term = (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
                 s = g == 0 ? term : s + term;
             }
@@ -485,7 +490,7 @@ __device__ __forceinline__ void buffer_term(const uint8_t* lds_ub, const float (
         if constexpr (!T::QBUF) uv = i < n ? uv : 0.0f;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const float cu = !T::QBUF ? c[v][i] : i < n ? c[v][i] * ubs[i] : 0.0f;       // (a dead slot's scale: anything)
+            const float cu = !T::QBUF ? c[v][i] : i < n ? c[v][i] * ubs[i] : 0.0f;    // (dead slot: any scale)
             acc[v] = __builtin_fmaf(uv, cu, acc[v]);
         }
     }
@@ -604,7 +609,8 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
     const int j = l.lane % T::MR, kb = l.lane / T::MR;
     const bool live = l.cg < T::LPR;
 
-    // keys as matrix operands, for the whole tile: aop[cs][t] = kx_{2t + kb}[32 cs + 16 ((j >> 2) & 1) + 4 (j >> 3) + (j & 3)]
+    // keys as matrix operands, for the whole tile:
+    // aop[cs][t] = kx_{2t + kb}[32 cs + 16 ((j >> 2) & 1) + 4 (j >> 3) + (j & 3)]
     float aop[NCS][MT];
     {
         const int col = 16 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3);
@@ -621,7 +627,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
     uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
     uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
 
-    RawRow<T::BITS> nxt[NL];                                 // the next row block and its scales, requested a block ahead
+    RawRow<T::BITS> nxt[NL];                                 // the next row block and its scales, a block ahead
     uint16_t scn[T::NG];
 #pragma unroll
     for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
