@@ -80,15 +80,8 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
     f.n = *a.np & (m - 1);
     f.gcur = *a.gcp;
-    const int lm = l.lane < m ? l.lane : m - 1;
-    f.ubs_raw = 0;
-    if constexpr (T::QBUF) f.ubs_raw = a.buf.UBS[lm];
-    f.gb_lane = a.GBh[lm];                                       // lane i: slot i's cumulative decay
-    stage_load(a.buf.UB, m * DV * T::BE, l.lane, f.st_ub);
+    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
     stage_load(reinterpret_cast<const uint8_t*>(a.SCh), DV * T::NG * 2, l.lane, f.st_sc);
-    load_keybuf<T>(a.buf, m, l, f.kbuf);
-#pragma unroll
-    for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < m ? i : m - 1]; }
     const uint32_t b = a.b, h = a.h;
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(hq) * DK);
     const void* kb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(hq) * DK);
@@ -114,7 +107,16 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
         r = r < DV ? r : DV - 1;
         f.vr[t] = load_raw(vb, p.v_dt, r);
     }
-    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
+    // the buffer last, and only its live slots (the fill count is a scalar load issued first: by now it is here)
+    const int nl = f.n > 0 ? f.n : 1;
+    const int lm = l.lane < nl ? l.lane : nl - 1;
+    f.ubs_raw = 0;
+    if constexpr (T::QBUF) f.ubs_raw = a.buf.UBS[lm];
+    f.gb_lane = a.GBh[lm];                                       // lane i: slot i's cumulative decay
+    stage_load(a.buf.UB, nl * DV * T::BE, l.lane, f.st_ub);
+    load_keybuf<T>(a.buf, nl, l, f.kbuf);
+#pragma unroll
+    for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < nl ? i : nl - 1]; }
 }
 
 template <class T>

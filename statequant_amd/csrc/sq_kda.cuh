@@ -61,24 +61,13 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     const uint8_t* lane_base = lane_codes<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
-    // ---- issue every load ----
+    // ---- issue every load: the state and the inputs first, the buffer last and only its live slots (the fill
+    // count is a scalar load issued first; by then it is here) ----
     const int n = *np & (m - 1);
-    uint16_t ubs_raw = 0;
-    if constexpr (T::QBUF) ubs_raw = buf.UBS[l.lane < m ? l.lane : m - 1];
-    Staged<T::UB_BYTES> st_ub;
-    stage_load(buf.UB, m * DV * T::BE, l.lane, st_ub);
+    Window<T> win;
+    window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
     stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
-    KeyBuf<T> kbuf;
-    load_keybuf<T>(buf, m, l, kbuf);
-    float4 gbp[KT][CPL / 4];                                      // the lane's piece of G_i of its slot(s)
-#pragma unroll
-    for (int t = 0; t < KT; ++t) {
-        const int i = l.rg + T::RG * t;
-        const float4* g4 = reinterpret_cast<const float4*>(GBh + (i < m ? i : m - 1) * DK + cc * CPL);
-#pragma unroll
-        for (int k = 0; k < CPL / 4; ++k) gbp[t][k] = g4[k];
-    }
     uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     float gc[T::NE];
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
@@ -102,8 +91,21 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
         r = r < DV ? r : DV - 1;
         vr[t] = load_raw(vb, p.v_dt, r);
     }
-    Window<T> win;
-    window_init<T>(lane_base, win);
+    const int nl = n > 0 ? n : 1;
+    uint16_t ubs_raw = 0;
+    if constexpr (T::QBUF) ubs_raw = buf.UBS[l.lane < nl ? l.lane : nl - 1];
+    Staged<T::UB_BYTES> st_ub;
+    stage_load(buf.UB, nl * DV * T::BE, l.lane, st_ub);
+    KeyBuf<T> kbuf;
+    load_keybuf<T>(buf, nl, l, kbuf);
+    float4 gbp[KT][CPL / 4];                                      // the lane's piece of G_i of its slot(s)
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+        const int i = l.rg + T::RG * t;
+        const float4* g4 = reinterpret_cast<const float4*>(GBh + (i < nl ? i : nl - 1) * DK + cc * CPL);
+#pragma unroll
+        for (int k = 0; k < CPL / 4; ++k) gbp[t][k] = g4[k];
+    }
 
     // ---- prep: q, k normalised, the running decay per channel ----
     const bool full = n == m - 1;

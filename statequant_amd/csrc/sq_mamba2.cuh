@@ -56,22 +56,14 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     int32_t* np = field(p.st.NPTR, seq, p.st.sN, h);
     const uint8_t* lane_base = lane_codes<T>(Sh, l);
 
-    // ---- issue every load ----
+    // ---- issue every load: the state and the inputs first, the buffer last and only its live slots (the fill
+    // count is a scalar load issued first; by then it is here) ----
     const int n = *np & (m - 1);
     const float gcur = *gcp;
-    const int lm = l.lane < m ? l.lane : m - 1;
-    uint16_t ubs_raw = 0;
-    if constexpr (T::QBUF) ubs_raw = buf.UBS[lm];
-    const float gb_lane = GBh[lm];
-    Staged<T::UB_BYTES> st_ub;
-    stage_load(buf.UB, m * DV * T::BE, l.lane, st_ub);
+    Window<T> win;
+    window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
     stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
-    KeyBuf<T> kbuf;
-    load_keybuf<T>(buf, m, l, kbuf);
-    float gb[KT];
-#pragma unroll
-    for (int t = 0; t < KT; ++t) { const int i = l.rg + T::RG * t; gb[t] = GBh[i < m ? i : m - 1]; }
     uint32_t cr[T::NE], br[T::NE];
     const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
     const void* bb = advance(p.B, p.B_dt, uint64_t(b) * p.s_B + hk * DK);
@@ -94,8 +86,18 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         r = r < DV ? r : DV - 1;
         xr_raw[t] = load_raw(xb, p.x_dt, r);
     }
-    Window<T> win;
-    window_init<T>(lane_base, win);
+    const int nl = n > 0 ? n : 1;
+    const int lm = l.lane < nl ? l.lane : nl - 1;
+    uint16_t ubs_raw = 0;
+    if constexpr (T::QBUF) ubs_raw = buf.UBS[lm];
+    const float gb_lane = GBh[lm];
+    Staged<T::UB_BYTES> st_ub;
+    stage_load(buf.UB, nl * DV * T::BE, l.lane, st_ub);
+    KeyBuf<T> kbuf;
+    load_keybuf<T>(buf, nl, l, kbuf);
+    float gb[KT];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) { const int i = l.rg + T::RG * t; gb[t] = GBh[i < nl ? i : nl - 1]; }
 
     // ---- prep: B, C of the group, dt, decay ----
     const bool full = n == m - 1;
