@@ -68,15 +68,20 @@ int launch_pack(const PackParams& p, hipStream_t stream) {
     return int(hipGetLastError());
 }
 
-// LDS (dynamic): keys x decay ratio [m][KROW] fp32, values [m][dv] fp32
+// LDS (dynamic): keys x decay ratio [m][DK] fp32, values [m][dv] fp32.
+// Column split of the output pass: a lane takes NCH chunks of 4 columns, chunk t = columns 4 LPR t + 4 cg .. + 3, so
+// that the LPR lanes of a row write 16 LPR consecutive bytes with every store instruction (whole 128-byte lines for
+// d_k = 128) -- with 16 consecutive columns per lane each store would scatter 16-byte pieces 64 bytes apart.
 template <int BITS, int DK, int GROUP, bool QBUF, bool KDA>
 __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     using T = RowTile<BITS, DK, GROUP, QBUF>;
+    constexpr int NCH = CPL / 4;
+    constexpr int CSTEP = 4 * T::LPR;                             // columns between a lane's chunks
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int m = p.m;
     const uint32_t um = m, dv = p.dv;
     float* lds_k = reinterpret_cast<float*>(lds);
-    float* lds_u = lds_k + m * T::KROW;
+    float* lds_u = lds_k + m * DK;
     const LaneId l = lane_id<T>();
     const uint32_t b = blockIdx.x / uint32_t(p.hv), h = blockIdx.x - b * uint32_t(p.hv);
     const uint32_t hk = h / uint32_t(p.gqa);
@@ -96,74 +101,89 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     const bool live = l.cg < T::LPR;
     const int cc = live ? l.cg : T::LPR - 1;
 
-    // keys, times their decay ratio, dead slots as zeros
-    float alpha_p[CPL];                                           // this lane's columns of a_n
-    float gcp[CPL];
-#pragma unroll
-    for (int t = 0; t < CPL; ++t) {
-        gcp[t] = KDA ? gch[cc * CPL + t] : gch[0];
-        alpha_p[t] = expf(gcp[t]);
-    }
-    BufAddr<T> ba;
-    ba.KB = const_cast<uint8_t*>(KB);
-    for (int i0 = 0; i0 < m; i0 += T::RG) {
+    // keys of the live slots, times their decay ratio (slot = row group + RG x pass, 16 consecutive columns per lane)
+    for (int i0 = 0; i0 < n; i0 += T::RG) {
         const int i = i0 + l.rg;
-        const int ic = i < m ? i : m - 1;
-        const KPiece<QBUF> kp = load_kpiece<T>(ba.KB, ic, m, l);
+        const int ic = i < n ? i : n - 1;
+        const KPiece<QBUF> kp = load_kpiece<T>(KB, ic, n, l);
         const float ks = QBUF ? f16_to_f32(KBS[ic]) : 1.0f;
         float kb[CPL];
         decode_kpiece<T>(kp, ks, l, kb);
-        const bool alive = i < n;
 #pragma unroll
         for (int t = 0; t < CPL; ++t) {
             const float gi = KDA ? GBh[ic * DK + cc * CPL + t] : GBh[ic];
-            kb[t] = alive ? kb[t] * expf(gcp[t] - gi) : 0.0f;
+            const float gc = KDA ? gch[cc * CPL + t] : gch[0];
+            kb[t] = kb[t] * expf(gc - gi);
         }
-        if (i < m) stage_kpiece<T>(lds_k, i, l, kb);
+        if (i < n && live) {
+            float4* d4 = reinterpret_cast<float4*>(lds_k + i * DK + l.cg * CPL);
+#pragma unroll
+            for (int c = 0; c < CPL / 4; ++c) d4[c] = make_float4(kb[4 * c], kb[4 * c + 1], kb[4 * c + 2], kb[4 * c + 3]);
+        }
     }
-    for (uint32_t e = l.lane; e < um * dv; e += WAVE) {
+    for (uint32_t e = l.lane; e < uint32_t(n) * dv; e += WAVE) {
         const uint32_t i = e / dv;
         float u;
         if constexpr (QBUF) u = float(reinterpret_cast<const int8_t*>(UB)[e]) * f16_to_f32(UBS[i]);
         else u = bf16_to_f32(reinterpret_cast<const uint16_t*>(UB)[e]);
-        lds_u[e] = int(i) < n ? u : 0.0f;
+        lds_u[e] = u;
     }
+    float alpha_p[NCH][4];                                        // a_n at this lane's columns
+#pragma unroll
+    for (int t = 0; t < NCH; ++t)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) alpha_p[t][c] = expf(KDA ? gch[t * CSTEP + 4 * cc + c] : gch[0]);
     __syncthreads();
 
-    int gi = (l.cg * CPL) / GROUP;
-    const bool has_group = gi < T::NG;
-    gi = has_group ? gi : T::NG - 1;
     constexpr int RR = 2;                                         // rows per pass over the buffered keys
     for (uint32_t r0 = 0; r0 < dv; r0 += RR * T::RG) {
         uint32_t row[RR], rc[RR];
-        float acc[RR][CPL];
+        float acc[RR][NCH][4];
 #pragma unroll
         for (int k = 0; k < RR; ++k) {
             row[k] = r0 + k * T::RG + l.rg;
             rc[k] = row[k] < dv ? row[k] : dv - 1;
-            float c[CPL];
-            decode_row<BITS>(load_row<BITS>(Sh + rc[k] * T::ROW_BYTES + cc * T::LANE_BYTES), c);
-            const float s = has_group ? f16_to_f32(SCh[rc[k] * T::NG + gi]) : 0.0f;
 #pragma unroll
-            for (int t = 0; t < CPL; ++t) acc[k][t] = alpha_p[t] * (c[t] * s);
+            for (int t = 0; t < NCH; ++t) {
+                const int col = t * CSTEP + 4 * cc;
+                const float s = f16_to_f32(SCh[rc[k] * T::NG + col / GROUP]);
+                float c4[4];
+                if constexpr (BITS == 8) {
+                    const uint32_t w = *reinterpret_cast<const uint32_t*>(Sh + rc[k] * T::ROW_BYTES + col);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) c4[c] = s8_to_f(w, c);
+                } else {
+                    const uint32_t w = *reinterpret_cast<const uint16_t*>(Sh + rc[k] * T::ROW_BYTES + col / 2);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) c4[c] = float(int32_t((w >> (4 * c)) & 0xFu) - 8);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[k][t][c] = alpha_p[t][c] * (c4[c] * s);
+            }
         }
         for (int i = 0; i < n; ++i) {                             // live slots only
-            float kx[CPL];
-            lds_piece<T>(lds_k + i * T::KROW, l.cg, kx);
+            float4 kx[NCH];
+#pragma unroll
+            for (int t = 0; t < NCH; ++t) kx[t] = *reinterpret_cast<const float4*>(lds_k + i * DK + t * CSTEP + 4 * cc);
 #pragma unroll
             for (int k = 0; k < RR; ++k) {
                 const float du = lds_u[i * dv + rc[k]];
 #pragma unroll
-                for (int t = 0; t < CPL; ++t) acc[k][t] = __builtin_fmaf(du, kx[t], acc[k][t]);
+                for (int t = 0; t < NCH; ++t) {
+                    acc[k][t][0] = __builtin_fmaf(du, kx[t].x, acc[k][t][0]);
+                    acc[k][t][1] = __builtin_fmaf(du, kx[t].y, acc[k][t][1]);
+                    acc[k][t][2] = __builtin_fmaf(du, kx[t].z, acc[k][t][2]);
+                    acc[k][t][3] = __builtin_fmaf(du, kx[t].w, acc[k][t][3]);
+                }
             }
         }
 #pragma unroll
         for (int k = 0; k < RR; ++k)
             if (row[k] < dv && live) {
-                float4* o4 = reinterpret_cast<float4*>(out + row[k] * DK + l.cg * CPL);
 #pragma unroll
-                for (int t = 0; t < CPL / 4; ++t)
-                    o4[t] = make_float4(acc[k][4 * t], acc[k][4 * t + 1], acc[k][4 * t + 2], acc[k][4 * t + 3]);
+                for (int t = 0; t < NCH; ++t)
+                    *reinterpret_cast<float4*>(out + row[k] * DK + t * CSTEP + 4 * l.cg) =
+                        make_float4(acc[k][t][0], acc[k][t][1], acc[k][t][2], acc[k][t][3]);
             }
     }
 }
@@ -171,7 +191,7 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
 template <int BITS, int DK, int GROUP, bool QBUF, bool KDA>
 int launch_read(const ReadParams& p, hipStream_t stream) {
     using T = RowTile<BITS, DK, GROUP, QBUF>;
-    const size_t lds = size_t(p.m) * (T::KROW + p.dv) * sizeof(float);
+    const size_t lds = size_t(p.m) * (DK + p.dv) * sizeof(float);
     hipLaunchKernelGGL((read_kernel<BITS, DK, GROUP, QBUF, KDA>), dim3(p.rows * p.hv), dim3(WAVE), lds, stream, p);
     return int(hipGetLastError());
 }
