@@ -77,9 +77,11 @@ def test_decode_vs_oracle(name, m, bb):
 
 @pytest.mark.parametrize('D,DV,HV,HK,fmt', [(64, 64, 4, 2, (8, 'k', 64)), (64, 64, 4, 4, (4, 'k', 32)),
                                             (96, 192, 3, 3, (4, 'k', 64)), (96, 192, 2, 1, (8, 'k', 32)),
-                                            (96, 96, 2, 2, (8, 'k', 128))])
+                                            (96, 96, 2, 2, (8, 'k', 128)), (128, 128, 6, 2, (8, 'k', 128)),
+                                            (128, 128, 12, 12, (4, 'k', 64))])
 def test_other_head_shapes(D, DV, HV, HK, fmt):
-    """d = 64 (the CPU-reference config's head), OLMo-Hybrid's 96 x 192 with a ragged last key group, 96 x 96."""
+    """d = 64 (the CPU-reference config's head), OLMo-Hybrid's 96 x 192 with a ragged last key group, 96 x 96; head
+    counts and GQA factors that are not powers of two (6 / 2, 12 / 12: the tile split divides instead of shifting)."""
     T, m = 20, 4
     check(run_decode(fmt, m, 8, B=3, HV=HV, HK=HK, D=D, DV=DV, T=T), f'{D}x{DV} {fmt}', T, m)
 

@@ -80,7 +80,8 @@ def test_decode_vs_oracle(fmt, m, bb):
     check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
 
 
-@pytest.mark.parametrize('DK,DV,H,G', [(128, 128, 4, 1), (64, 64, 4, 4)])
+# 14 / 2: seven heads per group, as in Nemotron-H (112 / 8); neither count is a power of two
+@pytest.mark.parametrize('DK,DV,H,G', [(128, 128, 4, 1), (64, 64, 4, 4), (128, 64, 14, 2)])
 def test_other_head_shapes(DK, DV, H, G):
     check(run_decode((8, 'k', 64), 4, 8, B=3, H=H, G=G, DK=DK, DV=DV, T=12), f'mamba2 {DK}x{DV}', 12, 4)
 
