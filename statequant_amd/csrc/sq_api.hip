@@ -27,8 +27,9 @@ bool dtype_ok(int d) { return d == SQ_F32 || d == SQ_BF16 || d == SQ_F16; }
 // Geometry / format checks shared by the three families; fills the LayoutKey part of a parameter block.
 int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
     if (L.bits != 4 && L.bits != 8) return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4 or 8, got %d", who, L.bits);
-    if (!L.axis_k) return fail(SQ_E_UNSUPPORTED, "%s: value-axis scale groups are not built", who);
     if (!pow2(L.group)) return fail(SQ_E_ARG, "%s: group %d is not a power of two", who, L.group);
+    if (!L.axis_k && (L.dv <= 0 || L.dv % L.group))
+        return fail(SQ_E_ARG, "%s: value-axis group %d does not divide d_v %d", who, L.group, L.dv);
     if (L.buffer_bits != 8 && L.buffer_bits != 16)
         return fail(SQ_E_ARG, "%s: buffer_bits must be 8 or 16, got %d", who, L.buffer_bits);
     if (!pow2(L.m) || L.m > 32) return fail(SQ_E_ARG, "%s: m must be a power of two <= 32, got %d", who, L.m);
@@ -42,6 +43,7 @@ int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
     key->hk = L.hk;
     key->dk = L.dk;
     key->dv = L.dv;
+    key->axv = L.axis_k ? 0 : 1;
     key->gqa = L.hv / L.hk;
     key->hv_shift = pow2(L.hv) ? __builtin_ctz(unsigned(L.hv)) : -1;
     key->gqa_shift = pow2(key->gqa) ? __builtin_ctz(unsigned(key->gqa)) : -1;
@@ -294,6 +296,7 @@ int sq_read(const sq_read_args* a, void* stream) {
     sq::ReadParams p{};
     SQ_TRY(check_layout(a->lay, who, &p));
     if (a->lay.m > 16) return fail(SQ_E_UNSUPPORTED, "%s: m %d > 16", who, a->lay.m);
+    if (!a->lay.axis_k) return fail(SQ_E_UNSUPPORTED, "%s: value-axis scale groups are not built", who);
     if (a->kda && a->lay.hk != a->lay.hv) return fail(SQ_E_ARG, "%s: KDA has no grouped keys", who);
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;

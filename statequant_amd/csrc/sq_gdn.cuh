@@ -42,7 +42,7 @@ __device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p) {
     const uint32_t m = p.m, h = a.h, hk = a.hk;
     a.obase = (uint64_t(uint32_t(a.b)) * uint32_t(p.hv) + h) * T::DV;
     a.Sh = field(p.st.S, seq, p.st.sS, h * (T::DV * T::ROW_BYTES));
-    a.SCh = field(p.st.SC, seq, p.st.sSC, h * (T::DV * T::NG));
+    a.SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
     a.buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * m * T::DK) * T::BE;
     a.buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * m * T::DV) * T::BE;
     a.buf.KBS = field(p.st.KBS, seq, p.st.sKBS, hk * m);
@@ -81,7 +81,7 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     f.n = *a.np & (m - 1);
     f.gcur = *a.gcp;
     window_init<T>(lane_codes<T>(a.Sh, l), f.win);
-    stage_load(reinterpret_cast<const uint8_t*>(a.SCh), DV * T::NG * 2, l.lane, f.st_sc);
+    stage_load(reinterpret_cast<const uint8_t*>(a.SCh), T::SC_ELEMS * 2, l.lane, f.st_sc);
     const uint32_t b = a.b, h = a.h;
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(hq) * DK);
     const void* kb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(hq) * DK);
@@ -183,10 +183,10 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         float xe[2][T::NE];
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) { xe[0][t] = qe[t]; xe[1][t] = ke[t]; }
-        stage_planes<T, 2>(xe, l, lds_b, lds_xs);
+        if constexpr (!T::AXV) stage_planes<T, 2>(xe, l, lds_b, lds_xs);
     }
     stage_store(lds_ub, m * DV * T::BE, l.lane, F.st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, F.st_sc);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, F.st_sc);
     const float kq = wave_sum(kqp);
     if (own_key) {
         const float nx = sqrtf(wave_sum(ssx) + 1e-6f);
@@ -223,7 +223,10 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
 
     // ---- state pass ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, own);
+    float xe2[2][T::NE];
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) { xe2[0][t] = qe[t]; xe2[1][t] = ke[t]; }
+    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, xe2, own);
 
     const KeyBuf<T>& kbuf = F.kbuf;
     const float gb_lane = F.gb_lane;
@@ -280,7 +283,8 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         }
         fold_stage_key<T>(kr, m - 1, l, lds_k);
         __syncthreads();
-        fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
+        if constexpr (T::AXV) fold_tile_v<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
+        else fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
     }
 
     // ---- advance ----

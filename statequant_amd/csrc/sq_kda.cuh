@@ -49,7 +49,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     const uint32_t seq = slot;
 
     uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
-    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * (DV * T::NG));
+    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
     BufAddr<T> buf;
     buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + h * um * DK) * T::BE;
     buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     Window<T> win;
     window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
-    stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
+    stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
     uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     float gc[T::NE];
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
@@ -140,9 +140,9 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
             lds_g[pos] = gn[t];
         }
     }
-    stage_planes<T, 2>(xa, l, lds_b, lds_xs);
+    if constexpr (!T::AXV) stage_planes<T, 2>(xa, l, lds_b, lds_xs);
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
     const float kq = wave_sum(kqp);
     const float beta = raw_to_f(betar, p.beta_dt);
     float ubs[T::MMAX];
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
 
     // ---- state pass against A*q, A*k ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_ci, lds_own, l, own);
+    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_ci, lds_own, l, xa, own);
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll
@@ -261,7 +261,8 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
             if (e < T::LPRP * CPL) lds_c[kpos<T>(e)] = e < DK ? expf(gn[t]) : 0.0f;     // = A
         }
         __syncthreads();
-        fold_tile<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
+        if constexpr (T::AXV) fold_tile_v<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
+        else fold_tile<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
     }
 
     // ---- advance ----

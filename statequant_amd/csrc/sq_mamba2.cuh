@@ -45,7 +45,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     const uint32_t seq = slot;
 
     uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
-    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * (DV * T::NG));
+    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
     BufAddr<T> buf;
     buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
     buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     Window<T> win;
     window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
-    stage_load(reinterpret_cast<const uint8_t*>(SCh), DV * T::NG * 2, l.lane, st_sc);
+    stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
     uint32_t cr[T::NE], br[T::NE];
     const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
     const void* bb = advance(p.B, p.B_dt, uint64_t(b) * p.s_B + hk * DK);
@@ -115,10 +115,10 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         float xe[1][T::NE];
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) xe[0][t] = ce[t];
-        stage_planes<T, 1>(xe, l, lds_b, lds_xs);
+        if constexpr (!T::AXV) stage_planes<T, 1>(xe, l, lds_b, lds_xs);
     }
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), DV * T::NG * 2, l.lane, st_sc);
+    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
     const float bc = wave_sum(bcp);
     float dt = raw_to_f(dtr, p.dt_dt);
     if (p.has_dt_bias) dt = dt + raw_to_f(dbr, p.dt_bias_dt);
@@ -142,7 +142,10 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
 
     // ---- state pass ----
     float own[1][T::NOWN];
-    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, own);
+    float xe1[1][T::NE];
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) xe1[0][t] = ce[t];
+    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, xe1, own);
 
     // ---- owned rows: y, and the value to buffer ----
     float u[T::NOWN], amax = 0.0f;
@@ -195,7 +198,8 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         }
         fold_stage_key<T>(kr, m - 1, l, lds_k);
         __syncthreads();
-        fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
+        if constexpr (T::AXV) fold_tile_v<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
+        else fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
     }
 
     if (l.lane == 0) {

@@ -22,6 +22,7 @@ struct StatePtrs {
 
 struct LayoutKey {
     int bits, group, qbuf, m, hv, hk, dk, dv;
+    int axv;                                      // scale groups along the value axis (else along d_k)
     // launch geometry helpers, filled by the C ABI: gqa = hv / hk; log2 of hv and of gqa where they are powers of
     // two (else -1: the kernel divides), and tiles per XCD when the tile count is a multiple of 8 (else 0: no XCD
     // mapping)

@@ -27,10 +27,12 @@ namespace sq {
 // power of two) consecutive lanes hold one row, lanes past DK/16 idle (d_k = 96: 6 of 8).  The wavefront therefore
 // covers RG = 64/LPRP rows per load and a lane sees rows rg, rg + RG, rg + 2 RG, ...  (the fold and the buffer passes
 // use this shape; the state pass uses the matrix core's, below).
-template <int BITS_, int DK_, int DV_, int GROUP_, bool QBUF_, int MMAX_>
+// AXV: the scale groups run along the VALUE axis instead (GROUP consecutive rows share one scale per key column;
+// scales [DV / GROUP][DK]); built for GROUP = 32, one row block of the matrix-core passes.
+template <int BITS_, int DK_, int DV_, int GROUP_, bool QBUF_, int MMAX_, bool AXV_ = false>
 struct Tile {
     static constexpr int BITS = BITS_, DK = DK_, DV = DV_, GROUP = GROUP_, MMAX = MMAX_;
-    static constexpr bool QBUF = QBUF_;
+    static constexpr bool QBUF = QBUF_, AXV = AXV_;
     static_assert(BITS == 4 || BITS == 8, "stored codes are int4 or int8");
     static_assert(DK % CPL == 0 && DK >= 32 && DK <= 256, "d_k must be a multiple of 16 in 32..256");
     static constexpr int LPR = DK / CPL;                  // live lanes per row
@@ -39,7 +41,8 @@ struct Tile {
     static_assert(DV % (4 * RG) == 0, "d_v must be a multiple of 4 x the rows one wavefront load covers");
     static constexpr int RPL = DV / RG;                   // rows per lane (fold, buffer passes)
     static constexpr int NOWN = (DV + WAVE - 1) / WAVE;   // rows a lane owns after the state pass: lane + 64 t
-    static constexpr int NG = (DK + GROUP - 1) / GROUP;   // stored key groups per row (last may be ragged)
+    static constexpr int KGROUP = AXV ? pow2_ceil(DK) : GROUP;     // length of a scale group along a row
+    static constexpr int NG = (DK + KGROUP - 1) / KGROUP; // stored key groups per row (last may be ragged); AXV: 1
     static_assert(GROUP % CPL == 0 && GROUP >= CPL, "key group must be a multiple of 16");
     static constexpr int LPG = (GROUP / CPL < LPRP) ? GROUP / CPL : LPRP;   // lanes sharing one scale
     static constexpr int ROW_BYTES = BITS == 4 ? DK / 2 : DK;
@@ -53,6 +56,7 @@ struct Tile {
     // matrix-core pass: blocks of MR rows x MK columns (one lane: one row, 16 columns; lanes 32.. the next 16)
     static constexpr int MR = 32, MK = 32;
     static_assert(DV % MR == 0 && DK % MK == 0 && GROUP % MK == 0, "tile / group must be multiples of 32");
+    static_assert(!AXV || GROUP == MR, "value-axis groups are one row block (32 rows)");
     static constexpr int NRB = DV / MR;                   // row blocks
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
@@ -60,7 +64,8 @@ struct Tile {
     static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
     static constexpr int A_BYTES = MR * A_PITCH;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
-    static constexpr int SC_BYTES = round_up(DV * NG * 2, 16);
+    static constexpr int SC_ELEMS = AXV ? (DV / GROUP) * DK : DV * NG;      // fp16 scales of one head
+    static constexpr int SC_BYTES = round_up(SC_ELEMS * 2, 16);
 };
 
 // LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
@@ -76,12 +81,12 @@ struct LdsPlan {
     // one region, three tenants in turn: the digit planes (until the pass has them in registers), then per row block
     // the codes on their way to operand shape and, once the block's products are issued, its integer sums
     static constexpr int B = XS + round_up(NV * T::NG * 4, 16);
-    static constexpr int A = B;
-    static constexpr int C = B;
+    static constexpr int A = B + (T::AXV ? T::B_BYTES : 0);    // value-axis: planes are rebuilt per row block
+    static constexpr int C = A;
     static constexpr int C_BYTES = T::NG * T::PLANES * NV * T::MR * 4;
     static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
                                                     : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
-    static constexpr int OWN = B + BAC;
+    static constexpr int OWN = A + BAC;
     static constexpr int FRONT = OWN + NV * T::UROW * 4;
     static constexpr int FK = 0;
     static constexpr int FU = FK + T::MMAX * T::KROW * 4;
@@ -216,13 +221,13 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
             float gm[2];                                     // group maximum for the lanes below / from 32
 #pragma unroll
             for (int hf = 0; hf < 2; ++hf) {
-                const int g = (WAVE * t + 32 * hf) / T::GROUP;
+                const int g = (WAVE * t + 32 * hf) / T::KGROUP;
                 float mx = 0.0f;
 #pragma unroll
                 for (int t2 = 0; t2 < T::NE; ++t2)
 #pragma unroll
                     for (int k = 0; k < NBLK; ++k)
-                        if ((WAVE * t2 + 16 * k) / T::GROUP == g && WAVE * t2 + 16 * k < T::DK)
+                        if ((WAVE * t2 + 16 * k) / T::KGROUP == g && WAVE * t2 + 16 * k < T::DK)
                             mx = fmaxf(mx, mb[t2][k]);
                 gm[hf] = mx;
             }
@@ -237,8 +242,8 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
                 at[0] = uint8_t(d);
                 at[CPL] = uint8_t(d >> 8);
                 at[2 * CPL] = uint8_t(d >> 16);
-                if (e % T::GROUP == 0)
-                    lds_xs[v * T::NG + e / T::GROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
+                if (e % T::KGROUP == 0)
+                    lds_xs[v * T::NG + e / T::KGROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
             }
         }
     }
@@ -281,10 +286,12 @@ __device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>&
 // free): operand lane (i = lane % 32, kb = lane / 32) takes, for column step ks, the 16 codes at row i, columns
 // 32 ks + 16 kb.  Result layout of the instruction: lane (j, kb) holds column j (= plane), rows 8 a + 4 kb + b in
 // element 4 a + b.
+// Value-axis scales: the scale belongs to (row block, column), so it goes into the read-out vector instead --
+// x'_k = x_k s[rb][k] -- and the digit planes are rebuilt from `xe` (element lane + 64 t of each vector) per block.
 template <class T, int NV>
-__device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, const uint8_t* lds_b,
-                                           const float* lds_xs, const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c,
-                                           float* lds_own, const LaneId& l, float (&own)[NV][T::NOWN]) {
+__device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, uint8_t* lds_b, float* lds_xs,
+                                           const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c, float* lds_own,
+                                           const LaneId& l, const float (&xe)[NV][T::NE], float (&own)[NV][T::NOWN]) {
     constexpr int NPL = T::PLANES * NV;
     constexpr int NCOL = NPL * T::NG;                        // result columns in use: (scale group, vector, digit)
     static_assert(NCOL <= T::MR && NV <= 2, "groups x digit planes must fit the instruction's 32 result columns");
@@ -294,19 +301,37 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
     // its own columns
     const int colg = j / NPL, colp = j - colg * NPL;
     v4i bop[T::NKS];
-#pragma unroll
-    for (int ks = 0; ks < T::NKS; ++ks) {
-        const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (colp & 7)) * CPL);
-        const bool mine = colg == (ks * T::MK) / T::GROUP;
-        bop[ks] = mine ? d : v4i{0, 0, 0, 0};
-    }
     float xs[T::NG];
+    auto fetch_planes = [&] {
 #pragma unroll
-    for (int g = 0; g < T::NG; ++g) xs[g] = lds_xs[(kb < NV ? kb : 0) * T::NG + g];
-    __syncthreads();                                         // the planes' region now carries the row blocks
+        for (int ks = 0; ks < T::NKS; ++ks) {
+            const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (colp & 7)) * CPL);
+            const bool mine = colg == (ks * T::MK) / T::KGROUP;
+            bop[ks] = mine ? d : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) xs[g] = lds_xs[(kb < NV ? kb : 0) * T::NG + g];
+    };
+    if constexpr (!T::AXV) {
+        fetch_planes();
+        __syncthreads();                                     // the planes' region now carries the row blocks
+    }
 
 #pragma unroll
     for (int rb = 0; rb < T::NRB; ++rb) {
+        if constexpr (T::AXV) {
+            float xr[NV][T::NE];
+#pragma unroll
+            for (int t = 0; t < T::NE; ++t) {
+                const int e = l.lane + WAVE * t;
+                const float s = e < T::DK ? f16_to_f32(lds_sc[rb * T::DK + (e < T::DK ? e : 0)]) : 0.0f;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) xr[v][t] = xe[v][t] * s;
+            }
+            stage_planes<T, NV>(xr, l, lds_b, lds_xs);
+            __syncthreads();
+            fetch_planes();
+        }
         if (l.cg < T::LPR) {
 #pragma unroll
             for (int t = 0; t < Window<T>::NL; ++t)
@@ -336,7 +361,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
                 const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
                 const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
                                                __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
-                const float term = (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
+                const float term = T::AXV ? f * xs[g] : (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
                 s = g == 0 ? term : s + term;
             }
             lds_own[kb * T::UROW + row] = s;
@@ -711,6 +736,131 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             for (int e = 0; e < CPL; ++e) a16[e] = acc[cs][e];
             store_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES,
                                quantize_row<T::BITS>(a16, rs[(cs * T::MK) / T::GROUP]));
+        }
+        __syncthreads();
+        if (live) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                store_row<T::BITS>(lane_base + (rb * T::MR + t * T::RG) * T::ROW_BYTES,
+                                   load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
+        }
+        __syncthreads();
+    }
+}
+
+// The fold for value-axis scale groups: one scale per (32-row block, key column), so the block is held "columns
+// across lanes" -- lane (j = lane % 32, kb = lane / 32) owns column j of a 32-column step and, in accumulator element
+// 4a + b, row 8a + 4 kb + b -- and a column's absmax is again a per-lane maximum plus one lane exchange.  The rank-1
+// updates run as above with the operands' roles swapped (values feed the rows, keys the columns).  The codes arrive in
+// that shape through the matrix core as well: the row block in operand shape times a 32 x 32 identity
+// (v_mfma_i32_32x32x32_i8) is the block itself, one int32 per code, laid out exactly like the accumulators.  The new
+// codes go back to the row-major LDS block byte by byte (int4: even / odd columns paired across neighbouring lanes).
+template <class T, bool COLVEC>
+__device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, const float* lds_c, float cmul, int m,
+                                            uint8_t* head, uint16_t* sc_head, const LaneId& l) {
+    constexpr int NCS = T::NKS;
+    constexpr int MT = (T::MMAX + 1) / 2;
+    constexpr int NL = Window<T>::NL;
+    constexpr float MAGIC = 12582912.0f + (T::BITS == 4 ? 8.0f : 0.0f);
+    const int j = l.lane % T::MR, kb = l.lane / T::MR;
+    const bool live = l.cg < T::LPR;
+
+    float kop[NCS][MT], cm[NCS];
+#pragma unroll
+    for (int cs = 0; cs < NCS; ++cs) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int slot = 2 * t + kb;
+            const float v = lds_k[(slot < m ? slot : 0) * T::KROW + kpos<T>(32 * cs + j)];
+            kop[cs][t] = slot < m ? v : 0.0f;
+        }
+        cm[cs] = COLVEC ? lds_c[kpos<T>(32 * cs + j)] : cmul;
+    }
+    // lane (n, kb) of the identity: byte t is 1 where operand position (kb, t) carries column n
+    v4i ident = {0, 0, 0, 0};
+    {
+        const int t = operand_pos<T::BITS>(j % CPL);
+        const int one = (j / CPL == kb) ? (1 << (8 * (t % 4))) : 0;
+        ident[0] = t / 4 == 0 ? one : 0;
+        ident[1] = t / 4 == 1 ? one : 0;
+        ident[2] = t / 4 == 2 ? one : 0;
+        ident[3] = t / 4 == 3 ? one : 0;
+    }
+    __syncthreads();                                         // lds_k becomes the block buffer
+    uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
+    uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
+
+    RawRow<T::BITS> nxt[NL];
+    uint16_t scn[NCS];
+#pragma unroll
+    for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
+#pragma unroll
+    for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[32 * cs + j];
+
+#pragma unroll 1
+    for (int rb = 0; rb < T::NRB; ++rb) {
+        uint16_t scr[NCS];
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) scr[cs] = scn[cs];
+        if (live) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                store_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES, nxt[t]);
+        }
+        if (rb + 1 < T::NRB) {
+#pragma unroll
+            for (int t = 0; t < NL; ++t)
+                nxt[t] = load_row<T::BITS>(lane_base + ((rb + 1) * T::MR + t * T::RG) * T::ROW_BYTES);
+#pragma unroll
+            for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[(rb + 1) * T::DK + 32 * cs + j];
+        }
+        float dop[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int slot = 2 * t + kb;
+            const float v = lds_u[(slot < m ? slot : 0) * T::UROW + rb * T::MR + j];
+            dop[t] = slot < m ? v : 0.0f;
+        }
+        __syncthreads();
+
+        v16f acc[NCS];
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) {
+            const RawRow<T::BITS> r = load_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES);
+            const v16i ci = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), ident, v16i{0}, 0, 0, 0);
+            const float s = f16_to_f32(scr[cs]) * DECODE_UNIT<T::BITS>;          // exact (int4 operands are 16 x code)
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) acc[cs][e] = COLVEC ? (float(ci[e]) * s) * cm[cs] : float(ci[e]) * (s * cm[cs]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[cs] = __builtin_amdgcn_mfma_f32_32x32x2f32(dop[t], kop[cs][t], acc[cs], 0, 0, 0);
+        }
+        float rs[NCS];
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) {
+            float mx = 0.0f;
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) mx = fmaxf(mx, fabsf(acc[cs][e]));
+            const float sc = fp16_scale(fmaxf(mx, __shfl_xor(mx, 32)), T::QMAX);
+            rs[cs] = 1.0f / sc;
+            if (kb == 0) sc_head[rb * T::DK + 32 * cs + j] = f32_to_f16(sc);
+        }
+        __syncthreads();                                     // every lane has its codes: the block takes the new ones
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs) {
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) {
+                const float f = __builtin_fmaf(acc[cs][e], rs[cs], MAGIC);
+                const uint32_t u = as_u32(__builtin_amdgcn_fmed3f(f, MAGIC - T::QMAX, MAGIC + T::QMAX));
+                const int row = 8 * (e / 4) + 4 * kb + (e % 4);
+                if constexpr (T::BITS == 8) {
+                    blk[row * T::A_PITCH + 32 * cs + j] = uint8_t(u);
+                } else {
+                    const uint32_t nib = u & 0xFu;                       // code + 8
+                    const uint32_t other = as_u32(partner<0>(as_f32(nib)));
+                    if ((j & 1) == 0) blk[row * T::A_PITCH + (32 * cs + j) / 2] = uint8_t(nib | (other << 4));
+                }
+            }
         }
         __syncthreads();
         if (live) {

@@ -19,6 +19,7 @@ DEV = 'cuda'
 
 FORMATS = {'int4-k-g64': (4, 'k', 64), 'int8-k-g32': (8, 'k', 32), 'int8-k-g128': (8, 'k', 128),
            'int4-k-g32': (4, 'k', 32)}
+VALUE_AXIS = {'int8-v-g32': (8, 'v', 32), 'int4-v-g32': (4, 'v', 32)}
 
 
 def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.float32, S0_scale=0.5, DV=None):
@@ -64,7 +65,8 @@ def check(tal, tag, T, m):
     assert tal.worst_o < 2e-5, tal.worst_o
     assert tal.buf_flips <= max(1, 1e-4 * tal.buf_entries), tal.buf_flips
     assert tal.code_mism <= max(1, 1e-4 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)
-    assert tal.scale_mism <= max(1, 1e-4 * tal.code_n / 32)
+    # (a scale differs when the group's absmax lies within an fp32 rounding of an fp16 rounding boundary)
+    assert tal.scale_mism <= max(2, 5e-4 * tal.code_n / 32)
     assert tal.worst_raw < 0.2
 
 
@@ -73,6 +75,16 @@ def check(tal, tag, T, m):
 @pytest.mark.parametrize('bb', [8, 16])
 def test_decode_vs_oracle(name, m, bb):
     check(run_decode(FORMATS[name], m, bb), f'{name} m={m} buf{bb}', 40, m)
+
+
+@pytest.mark.parametrize('fmt', [(4, 'v', 32), (8, 'v', 32)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('D,DV', [(128, 128), (64, 64), (96, 192)])
+def test_value_axis_groups(fmt, m, bb, D, DV):
+    """Scale groups of 32 value rows per key column (the serving presets int4v / int8v): the scales ride on the
+    read-out vectors in the state pass and the fold holds a block columns-across-lanes."""
+    T = 3 * m + 2 if m > 1 else 4
+    check(run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=D, DV=DV, T=T), f'{fmt} {D}x{DV} m{m} bb{bb}', T, m)
 
 
 @pytest.mark.parametrize('D,DV,HV,HK,fmt', [(64, 64, 4, 2, (8, 'k', 64)), (64, 64, 4, 4, (4, 'k', 32)),
@@ -122,7 +134,7 @@ def test_q_k_per_value_head_matches_per_key_head():
     assert torch.equal(a.codes, b.codes) and torch.equal(a.KB, b.KB)
 
 
-@pytest.mark.parametrize('name', ['gdn_c1.pt', 'gdn_int4.pt', 'gdn_int8_m1.pt'])
+@pytest.mark.parametrize('name', ['gdn_c1.pt', 'gdn_int4.pt', 'gdn_int8_m1.pt', 'gdn_int4v.pt'])
 def test_against_reference_golden_vectors(golden, name):
     """The HIP step replayed on the inputs the reference's own ReferenceGDNState was recorded on: outputs, appended
     buffer entries, codes and scales after every fold.  The kernel state is re-seeded from the reference's record
@@ -189,12 +201,12 @@ def _setup(fmt, m, bb, n_slots=8, seed=0):
     return lay, raw, blob, views, slots, refs
 
 
-@pytest.mark.parametrize('name', ['int4-k-g64', 'int8-k-g32'])
+@pytest.mark.parametrize('name', ['int4-k-g64', 'int8-k-g32', 'int8-v-g32'])
 @pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
 def test_slot_step_matches_lockstep_per_sequence(name, m, bb):
     """Slot-addressed step == the lockstep state run per sequence, bit for bit (same kernel, other strides);
     padding rows give zeros; nothing outside the live slots' blobs is written (reference: tests/test_slots.py:54-109)."""
-    fmt = FORMATS[name]
+    fmt = {**FORMATS, **VALUE_AXIS}[name]
     lay, raw, blob, views, slots, refs = _setup(fmt, m, bb)
     for i, r in enumerate(refs):
         assert torch.equal(views['S'][slots[i]], r.codes.view(HV, *r.codes.shape[1:]))
@@ -334,7 +346,8 @@ def test_empty_batch_and_errors():
     e = torch.zeros(0, HK, D, device=DEV)
     assert lay.step(lay.views(blob), torch.zeros(0, dtype=torch.int32, device=DEV), e, e, out, out, 1.0,
                     g=out, beta=out) is out
-    with pytest.raises(NotImplementedError):                     # value-axis groups: layout yes, HIP step not built
-        SlotLayout(quantizer((4, 'v', 32)), HV, HK, D, D)._layout_struct()
+    with pytest.raises(NotImplementedError):                     # value-axis groups of 64: layout yes, no kernel built
+        SlotLayout(quantizer((4, 'v', 64)), HV, HK, D, D)._layout_struct()
+    SlotLayout(quantizer((4, 'v', 32)), HV, HK, D, D)._layout_struct()
     with pytest.raises(RuntimeError):                            # CPU tensors never reach a kernel
         PackedGDNState(torch.zeros(8, D, D), quantizer((4, 'k', 64)), hv=HV, hk=HK)

@@ -65,6 +65,13 @@ def check(tal, tag, T, m):
     assert tal.worst_raw < 0.2
 
 
+@pytest.mark.parametrize('fmt,m,bb', [((4, 'v', 32), 8, 8), ((8, 'v', 32), 4, 16), ((4, 'v', 32), 1, 8)])
+def test_value_axis_groups(fmt, m, bb):
+    """Scale groups of 32 value rows per key column, with KDA's per-channel decay on the stored state."""
+    T = 24 if m > 1 else 4
+    check(run_decode(fmt, m, bb, T=T), f'kda {fmt} m={m} buf{bb}', T, m)
+
+
 @pytest.mark.parametrize('fmt', [(4, 'k', 32), (4, 'k', 64), (8, 'k', 32), (8, 'k', 128)])
 @pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 8)])
 def test_decode_vs_oracle(fmt, m, bb):
