@@ -26,9 +26,12 @@ bool dtype_ok(int d) { return d == SQ_F32 || d == SQ_BF16 || d == SQ_F16; }
 
 // Geometry / format checks shared by the three families; fills the LayoutKey part of a parameter block.
 int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
-    if (L.bits != 4 && L.bits != 8) return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4 or 8, got %d", who, L.bits);
-    if (!pow2(L.group)) return fail(SQ_E_ARG, "%s: group %d is not a power of two", who, L.group);
-    if (!L.axis_k && (L.dv <= 0 || L.dv % L.group))
+    if (L.bits != 4 && L.bits != 8 && L.bits != 16 && L.bits != 32)
+        return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4, 8 (codes), 16 (bf16 state) or 32 (fp32 state), got %d", who,
+                    L.bits);
+    const bool flt = L.bits >= 16;                        // unquantized state: no scales, group / axis ignored
+    if (!flt && !pow2(L.group)) return fail(SQ_E_ARG, "%s: group %d is not a power of two", who, L.group);
+    if (!flt && !L.axis_k && (L.dv <= 0 || L.dv % L.group))
         return fail(SQ_E_ARG, "%s: value-axis group %d does not divide d_v %d", who, L.group, L.dv);
     if (L.buffer_bits != 8 && L.buffer_bits != 16)
         return fail(SQ_E_ARG, "%s: buffer_bits must be 8 or 16, got %d", who, L.buffer_bits);
@@ -36,14 +39,14 @@ int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
     if (L.hv <= 0 || L.hk <= 0 || L.hv % L.hk) return fail(SQ_E_ARG, "%s: hv %d, hk %d", who, L.hv, L.hk);
     if (L.dk <= 0 || L.dv <= 0 || (L.dk & 1)) return fail(SQ_E_ARG, "%s: dk %d, dv %d", who, L.dk, L.dv);
     key->bits = L.bits;
-    key->group = L.group;
+    key->group = flt ? L.dk : L.group;
     key->qbuf = L.buffer_bits == 8;
     key->m = L.m;
     key->hv = L.hv;
     key->hk = L.hk;
     key->dk = L.dk;
     key->dv = L.dv;
-    key->axv = L.axis_k ? 0 : 1;
+    key->axv = (flt || L.axis_k) ? 0 : 1;
     key->gqa = L.hv / L.hk;
     key->hv_shift = pow2(L.hv) ? __builtin_ctz(unsigned(L.hv)) : -1;
     key->gqa_shift = pow2(key->gqa) ? __builtin_ctz(unsigned(key->gqa)) : -1;
@@ -63,24 +66,26 @@ bool stride_ok(int64_t s) { return s >= 0 && s < (int64_t(1) << 31); }
 // Pointers, strides and alignment of the stored state.  The kernels read a lane's piece of a code row with one
 // 128-bit (int8) or 64-bit (int4) load and a piece of a buffered int8 key with one 128-bit load.
 int check_state(const sq_state& s, const sq_layout& L, const char* who, sq::StatePtrs* st) {
-    if (!s.S || !s.SC || !s.KB || !s.UB || !s.GB || !s.GCUR || !s.NPTR)
+    const bool flt = L.bits >= 16;
+    if (!s.S || (!flt && !s.SC) || !s.KB || !s.UB || !s.GB || !s.GCUR || !s.NPTR)
         return fail(SQ_E_ARG, "%s: null state pointer", who);
     if (L.buffer_bits == 8 && (!s.KBS || !s.UBS)) return fail(SQ_E_ARG, "%s: int8 buffer without scales", who);
-    const size_t row_align = L.bits == 8 ? 16 : 8;
-    if (!aligned(s.S, row_align) || (s.sS % int64_t(row_align)))
-        return fail(SQ_E_ARG, "%s: codes must be %zu-byte aligned (base and per-sequence stride)", who, row_align);
+    const size_t row_align = L.bits == 4 ? 8 : 16;
+    const int64_t s_bytes = s.sS * (flt ? L.bits / 8 : 1);          // the kernels address the state in bytes
+    if (!aligned(s.S, row_align) || (s_bytes % int64_t(row_align)))
+        return fail(SQ_E_ARG, "%s: state must be %zu-byte aligned (base and per-sequence stride)", who, row_align);
     if (L.buffer_bits == 8 && (!aligned(s.KB, 16) || (s.sKB % 16)))
         return fail(SQ_E_ARG, "%s: int8 key buffer must be 16-byte aligned (base and per-sequence stride)", who);
     // scales and buffered values are staged into LDS with 128-bit loads
-    if (!aligned(s.SC, 16) || (s.sSC % 8) || !aligned(s.UB, 16) || ((s.sUB * (L.buffer_bits / 8)) % 16))
+    if ((!flt && (!aligned(s.SC, 16) || (s.sSC % 8))) || !aligned(s.UB, 16) || ((s.sUB * (L.buffer_bits / 8)) % 16))
         return fail(SQ_E_ARG, "%s: scales and value buffer must be 16-byte aligned (base and per-sequence stride)",
                     who);
     if (!aligned(s.GB, 4) || !aligned(s.GCUR, 4) || !aligned(s.NPTR, 4))
         return fail(SQ_E_ARG, "%s: misaligned decay / counter pointer", who);
-    if (!stride_ok(s.sS) || !stride_ok(s.sSC) || !stride_ok(s.sKB) || !stride_ok(s.sKBS) || !stride_ok(s.sUB) ||
+    if (!stride_ok(s_bytes) || !stride_ok(s.sSC) || !stride_ok(s.sKB) || !stride_ok(s.sKBS) || !stride_ok(s.sUB) ||
         !stride_ok(s.sUBS) || !stride_ok(s.sGB) || !stride_ok(s.sGC) || !stride_ok(s.sN))
         return fail(SQ_E_ARG, "%s: per-sequence strides must be in [0, 2^31)", who);
-    st->S = static_cast<uint8_t*>(s.S);         st->sS = uint32_t(s.sS);
+    st->S = static_cast<uint8_t*>(s.S);         st->sS = uint32_t(s_bytes);
     st->SC = static_cast<uint16_t*>(s.SC);      st->sSC = uint32_t(s.sSC);
     st->KB = static_cast<uint8_t*>(s.KB);       st->sKB = uint32_t(s.sKB);
     st->KBS = static_cast<uint16_t*>(s.KBS);    st->sKBS = uint32_t(s.sKBS);

@@ -81,7 +81,7 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     f.n = *a.np & (m - 1);
     f.gcur = *a.gcp;
     window_init<T>(lane_codes<T>(a.Sh, l), f.win);
-    stage_load(reinterpret_cast<const uint8_t*>(a.SCh), T::SC_ELEMS * 2, l.lane, f.st_sc);
+    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(a.SCh), T::SC_ELEMS * 2, l.lane, f.st_sc);
     const uint32_t b = a.b, h = a.h;
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(hq) * DK);
     const void* kb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(hq) * DK);
@@ -183,10 +183,10 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         float xe[2][T::NE];
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) { xe[0][t] = qe[t]; xe[1][t] = ke[t]; }
-        if constexpr (!T::AXV) stage_planes<T, 2>(xe, l, lds_b, lds_xs);
+        if constexpr (!T::AXV && !T::FLT) stage_planes<T, 2>(xe, l, lds_b, lds_xs);
     }
     stage_store(lds_ub, m * DV * T::BE, l.lane, F.st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, F.st_sc);
+    if constexpr (!T::FLT) stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, F.st_sc);
     const float kq = wave_sum(kqp);
     if (own_key) {
         const float nx = sqrtf(wave_sum(ssx) + 1e-6f);

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     Window<T> win;
     window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
-    stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
+    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
     uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     float gc[T::NE];
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
@@ -140,9 +140,9 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
             lds_g[pos] = gn[t];
         }
     }
-    if constexpr (!T::AXV) stage_planes<T, 2>(xa, l, lds_b, lds_xs);
+    if constexpr (!T::AXV && !T::FLT) stage_planes<T, 2>(xa, l, lds_b, lds_xs);
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
+    if constexpr (!T::FLT) stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
     const float kq = wave_sum(kqp);
     const float beta = raw_to_f(betar, p.beta_dt);
     float ubs[T::MMAX];

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     Window<T> win;
     window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
-    stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
+    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
     uint32_t cr[T::NE], br[T::NE];
     const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
     const void* bb = advance(p.B, p.B_dt, uint64_t(b) * p.s_B + hk * DK);
@@ -115,10 +115,10 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         float xe[1][T::NE];
 #pragma unroll
         for (int t = 0; t < T::NE; ++t) xe[0][t] = ce[t];
-        if constexpr (!T::AXV) stage_planes<T, 1>(xe, l, lds_b, lds_xs);
+        if constexpr (!T::AXV && !T::FLT) stage_planes<T, 1>(xe, l, lds_b, lds_xs);
     }
     stage_store(lds_ub, m * DV * T::BE, l.lane, st_ub);
-    stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
+    if constexpr (!T::FLT) stage_store(reinterpret_cast<uint8_t*>(lds_sc), T::SC_ELEMS * 2, l.lane, st_sc);
     const float bc = wave_sum(bcp);
     float dt = raw_to_f(dtr, p.dt_dt);
     if (p.has_dt_bias) dt = dt + raw_to_f(dbr, p.dt_bias_dt);

@@ -29,11 +29,16 @@ namespace sq {
 // use this shape; the state pass uses the matrix core's, below).
 // AXV: the scale groups run along the VALUE axis instead (GROUP consecutive rows share one scale per key column;
 // scales [DV / GROUP][DK]); built for GROUP = 32, one row block of the matrix-core passes.
+// BITS = 16 / 32: the unquantized control -- the state kept as bf16 / fp32 [DV][DK], no scales (FLT below).  The front
+// end (vectors, buffer, append) keeps the geometry above; the state rows have their own: a lane's 16 bytes are SPL =
+// 8 / 4 columns, SLPRP lanes hold a row, a wavefront load covers SRG rows, NLD loads the tile.
 template <int BITS_, int DK_, int DV_, int GROUP_, bool QBUF_, int MMAX_, bool AXV_ = false>
 struct Tile {
     static constexpr int BITS = BITS_, DK = DK_, DV = DV_, GROUP = GROUP_, MMAX = MMAX_;
     static constexpr bool QBUF = QBUF_, AXV = AXV_;
-    static_assert(BITS == 4 || BITS == 8, "stored codes are int4 or int8");
+    static_assert(BITS == 4 || BITS == 8 || BITS == 16 || BITS == 32, "int4 / int8 codes, or a bf16 / fp32 state");
+    static constexpr bool FLT = BITS >= 16;
+    static_assert(!FLT || (!AXV && GROUP == DK), "a float state has no scale groups");
     static_assert(DK % CPL == 0 && DK >= 32 && DK <= 256, "d_k must be a multiple of 16 in 32..256");
     static constexpr int LPR = DK / CPL;                  // live lanes per row
     static constexpr int LPRP = pow2_ceil(LPR);           // lanes per row incl. idle ones
@@ -45,9 +50,15 @@ struct Tile {
     static constexpr int NG = (DK + KGROUP - 1) / KGROUP; // stored key groups per row (last may be ragged); AXV: 1
     static_assert(GROUP % CPL == 0 && GROUP >= CPL, "key group must be a multiple of 16");
     static constexpr int LPG = (GROUP / CPL < LPRP) ? GROUP / CPL : LPRP;   // lanes sharing one scale
-    static constexpr int ROW_BYTES = BITS == 4 ? DK / 2 : DK;
+    static constexpr int ROW_BYTES = DK * BITS / 8;
     static constexpr int LANE_BYTES = BITS == 4 ? CPL / 2 : CPL;
-    static constexpr float QMAX = float((1 << (BITS - 1)) - 1);
+    static constexpr float QMAX = float((1 << ((FLT ? 8 : BITS) - 1)) - 1);   // unused for a float state
+    static constexpr int SPL = FLT ? 128 / BITS : CPL;    // float state: columns per 16-byte lane piece
+    static constexpr int SLPR = DK / SPL;
+    static constexpr int SLPRP = pow2_ceil(SLPR);
+    static_assert(SLPRP <= WAVE, "a float-state row must fit one wavefront load");
+    static constexpr int SRG = WAVE / SLPRP;
+    static constexpr int NLD = DV / SRG;
     static constexpr int NE = (DK + WAVE - 1) / WAVE;     // elements of a d_k vector per lane (element = lane + 64 t)
     static constexpr int BE = QBUF ? 1 : 2;               // bytes per buffer element (int8 / bf16)
     static constexpr int KPAD = CPL + 4;                  // LDS stride of a 16-column piece (spreads the banks)
@@ -60,12 +71,13 @@ struct Tile {
     static constexpr int NRB = DV / MR;                   // row blocks
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
-    static constexpr int B_BYTES = (DK / CPL) * 8 * CPL;  // digit planes: [16-column piece][8 planes][16]
+    // digit planes: [16-column piece][8 planes][16]; float state: the read-out vectors themselves (at most two)
+    static constexpr int B_BYTES = FLT ? 2 * KROW * 4 : (DK / CPL) * 8 * CPL;
     static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
-    static constexpr int A_BYTES = MR * A_PITCH;
+    static constexpr int A_BYTES = FLT ? 0 : MR * A_PITCH;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
-    static constexpr int SC_ELEMS = AXV ? (DV / GROUP) * DK : DV * NG;      // fp16 scales of one head
-    static constexpr int SC_BYTES = round_up(SC_ELEMS * 2, 16);
+    static constexpr int SC_ELEMS = FLT ? 0 : AXV ? (DV / GROUP) * DK : DV * NG;      // fp16 scales of one head
+    static constexpr int SC_BYTES = FLT ? 16 : round_up(SC_ELEMS * 2, 16);
 };
 
 // LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
@@ -83,7 +95,7 @@ struct LdsPlan {
     static constexpr int B = XS + round_up(NV * T::NG * 4, 16);
     static constexpr int A = B + (T::AXV ? T::B_BYTES : 0);    // value-axis: planes are rebuilt per row block
     static constexpr int C = A;
-    static constexpr int C_BYTES = T::NG * T::PLANES * NV * T::MR * 4;
+    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::PLANES * NV * T::MR * 4;
     static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
                                                     : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
     static constexpr int OWN = A + BAC;
@@ -252,6 +264,10 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
 // A lane's first row piece in the row-shaped layout (LPRP lanes per row).
 template <class T>
 __device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const LaneId& l) {
+    if constexpr (T::FLT) {
+        const int scg = l.lane % T::SLPRP, srg = l.lane / T::SLPRP;
+        return head + srg * T::ROW_BYTES + (scg < T::SLPR ? scg : T::SLPR - 1) * 16;
+    }
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;       // idle lanes shadow a live one (masked later)
     return head + l.rg * T::ROW_BYTES + cc * T::LANE_BYTES;
 }
@@ -259,10 +275,16 @@ __device__ __forceinline__ const uint8_t* lane_codes(const uint8_t* head, const 
 // Two row blocks of codes in flight per wavefront, loaded row-shaped (LPRP lanes per row, so every load instruction
 // covers whole, consecutive rows and costs the address unit one cycle per 64 bytes; fetched in operand shape -- 32
 // different rows per instruction -- the same bytes cost it 8 x as many cycles and the step became address-bound).
-template <class T>
+template <class T, bool FLT = T::FLT>
 struct Window {
     static constexpr int NL = T::MR / T::RG;              // loads per row block
     RawRow<T::BITS> a[2][NL];
+};
+// Float state: the next FW wavefront loads (SRG rows each), 32 registers as well.
+template <class T>
+struct Window<T, true> {
+    static constexpr int FW = T::NLD < 8 ? T::NLD : 8;
+    uint4 a[FW];
 };
 template <class T>
 __device__ __forceinline__ void window_load(const uint8_t* lane_base, int rb, Window<T>& w) {
@@ -272,8 +294,91 @@ __device__ __forceinline__ void window_load(const uint8_t* lane_base, int rb, Wi
 }
 template <class T>
 __device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
-    window_load<T>(lane_base, 0, w);
-    if constexpr (T::NRB > 1) window_load<T>(lane_base, 1, w);
+    if constexpr (T::FLT) {
+#pragma unroll
+        for (int i = 0; i < Window<T>::FW; ++i)
+            w.a[i] = *reinterpret_cast<const uint4*>(lane_base + i * T::SRG * T::ROW_BYTES);
+    } else {
+        window_load<T>(lane_base, 0, w);
+        if constexpr (T::NRB > 1) window_load<T>(lane_base, 1, w);
+    }
+}
+
+// A lane's SPL state columns of a float-state row piece as fp32.
+template <int BITS>
+__device__ __forceinline__ void float_piece(const uint4& r, float (&s)[128 / BITS]) {
+    if constexpr (BITS == 16) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            s[2 * d] = as_f32(w[d] << 16);
+            s[2 * d + 1] = as_f32(w[d] & 0xFFFF0000u);
+        }
+    } else {
+        s[0] = as_f32(r.x); s[1] = as_f32(r.y); s[2] = as_f32(r.z); s[3] = as_f32(r.w);
+    }
+}
+// A lane's SPL columns of a d_k vector kept piecewise in LDS (kpos layout); zeros in idle lanes.
+template <class T>
+__device__ __forceinline__ void float_cols(const float* vec, int scg, float (&x)[T::SPL]) {
+    const float4* p4 = reinterpret_cast<const float4*>(vec + kpos<T>((scg < T::SLPR ? scg : 0) * T::SPL));
+#pragma unroll
+    for (int t = 0; t < T::SPL / 4; ++t) {
+        const float4 f = p4[t];
+        const bool in = scg < T::SLPR;
+        x[4 * t] = in ? f.x : 0.0f; x[4 * t + 1] = in ? f.y : 0.0f;
+        x[4 * t + 2] = in ? f.z : 0.0f; x[4 * t + 3] = in ? f.w : 0.0f;
+    }
+}
+
+// The pass over a float state: plain fp32 products on the vector ALU (a row piece decodes with a shift or not at all,
+// so there is nothing for the matrix core to save), each row reduced over its SLPRP lanes.
+template <class T, int NV>
+__device__ __forceinline__ void float_pass(const uint8_t* lane_base, Window<T>& w, uint8_t* lds_b, float* lds_own,
+                                           const LaneId& l, const float (&xe)[NV][T::NE], float (&own)[NV][T::NOWN]) {
+    constexpr int FW = Window<T>::FW;
+    static_assert(T::NLD % FW == 0, "whole windows");
+    const int scg = l.lane % T::SLPRP, srg = l.lane / T::SLPRP;
+    float* xf = reinterpret_cast<float*>(lds_b);
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) {
+            const int e = l.lane + WAVE * t;
+            if (e < T::LPRP * CPL) xf[v * T::KROW + kpos<T>(e)] = xe[v][t];
+        }
+    __syncthreads();
+    float xc[NV][T::SPL];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) float_cols<T>(xf + v * T::KROW, scg, xc[v]);
+#pragma unroll 1
+    for (int i0 = 0; i0 < T::NLD; i0 += FW) {
+#pragma unroll
+        for (int j = 0; j < FW; ++j) {
+            const int i = i0 + j;
+            float s[T::SPL];
+            float_piece<T::BITS>(w.a[j], s);
+            if (i + FW < T::NLD)
+                w.a[j] = *reinterpret_cast<const uint4*>(lane_base + (i + FW) * T::SRG * T::ROW_BYTES);
+            const int row = i * T::SRG + srg;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                float d = s[0] * xc[v][0];
+#pragma unroll
+                for (int e = 1; e < T::SPL; ++e) d = __builtin_fmaf(s[e], xc[v][e], d);
+                d = block_sum<(T::SLPRP < 16 ? T::SLPRP : 16)>(d);
+                if constexpr (T::SLPRP >= 32) d += __shfl_xor(d, 16);
+                if constexpr (T::SLPRP >= 64) d += __shfl_xor(d, 32);
+                if (scg == 0) lds_own[v * T::UROW + row] = d;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int t = 0; t < T::NOWN; ++t)
+            own[v][t] = owned_valid<T>(l, t) ? lds_own[v * T::UROW + owned_row<T>(l, t)] : 0.0f;
 }
 
 // Row sums of the whole tile against NV read-out vectors: own[v][t] = (S0 x_v)[lane + 64 t], scales applied.
@@ -292,6 +397,10 @@ template <class T, int NV>
 __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, uint8_t* lds_b, float* lds_xs,
                                            const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c, float* lds_own,
                                            const LaneId& l, const float (&xe)[NV][T::NE], float (&own)[NV][T::NOWN]) {
+    if constexpr (T::FLT) {
+        float_pass<T, NV>(lane_base, w, lds_b, lds_own, l, xe, own);
+        return;
+    } else {
     constexpr int NPL = T::PLANES * NV;
     constexpr int NCOL = NPL * T::NG;                        // result columns in use: (scale group, vector, digit)
     static_assert(NCOL <= T::MR && NV <= 2, "groups x digit planes must fit the instruction's 32 result columns");
@@ -373,6 +482,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 #pragma unroll
         for (int t = 0; t < T::NOWN; ++t)
             own[v][t] = owned_valid<T>(l, t) ? lds_own[v * T::UROW + owned_row<T>(l, t)] : 0.0f;
+    }
 }
 
 // A lane's 16-column piece of a d_k vector kept piecewise in LDS.
@@ -625,9 +735,69 @@ __device__ __forceinline__ void fold_stage_key(const float (&kr)[T::NE], int slo
 // order as the accumulation-order mismatches).
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// The fold of a float state: S = c S0 + sum_i (decayed u_i) k_i^T in slot order on the vector ALU, rounded to the
+// state's type and stored in place (_fused_triton.py:376-382: no scales, no absmax).  A lane keeps its SPL columns of
+// all m keys in registers; the values come from LDS (one broadcast read per row and slot).
+template <class T, bool COLVEC>
+__device__ __forceinline__ void float_fold(const float* lds_k, const float* lds_u, const float* lds_c, float cmul,
+                                           int m, uint8_t* head, const LaneId& l) {
+    constexpr int FW = 4;
+    static_assert(T::NLD % FW == 0, "whole windows");
+    const int scg = l.lane % T::SLPRP, srg = l.lane / T::SLPRP;
+    const bool live = scg < T::SLPR;
+    float kk[T::MMAX][T::SPL], cm[T::SPL];
+#pragma unroll
+    for (int i = 0; i < T::MMAX; ++i) {
+        float_cols<T>(lds_k + (i < m ? i : 0) * T::KROW, scg, kk[i]);
+        if (i >= m) {
+#pragma unroll
+            for (int e = 0; e < T::SPL; ++e) kk[i][e] = 0.0f;
+        }
+    }
+    if constexpr (COLVEC) float_cols<T>(lds_c, scg, cm);
+    uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
+    uint4 w[FW];
+#pragma unroll
+    for (int j = 0; j < FW; ++j) w[j] = *reinterpret_cast<const uint4*>(lane_base + j * T::SRG * T::ROW_BYTES);
+#pragma unroll 1
+    for (int i0 = 0; i0 < T::NLD; i0 += FW) {
+#pragma unroll
+        for (int j = 0; j < FW; ++j) {
+            const int i = i0 + j;
+            float acc[T::SPL];
+            float_piece<T::BITS>(w[j], acc);
+            if (i + FW < T::NLD) w[j] = *reinterpret_cast<const uint4*>(lane_base + (i + FW) * T::SRG * T::ROW_BYTES);
+#pragma unroll
+            for (int e = 0; e < T::SPL; ++e) acc[e] = acc[e] * (COLVEC ? cm[e] : cmul);
+            const int row = i * T::SRG + srg;
+#pragma unroll
+            for (int t = 0; t < T::MMAX; ++t) {
+                const float uv = lds_u[(t < m ? t : 0) * T::UROW + row];
+#pragma unroll
+                for (int e = 0; e < T::SPL; ++e) acc[e] = __builtin_fmaf(uv, kk[t][e], acc[e]);   // dead slots: k = 0
+            }
+            uint4 o;
+            if constexpr (T::BITS == 16) {
+                uint32_t q[4];
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    q[d] = uint32_t(f32_to_bf16(acc[2 * d])) | (uint32_t(f32_to_bf16(acc[2 * d + 1])) << 16);
+                o = make_uint4(q[0], q[1], q[2], q[3]);
+            } else {
+                o = make_uint4(as_u32(acc[0]), as_u32(acc[1]), as_u32(acc[2]), as_u32(acc[3]));
+            }
+            if (live) *reinterpret_cast<uint4*>(lane_base + i * T::SRG * T::ROW_BYTES) = o;
+        }
+    }
+}
+
 template <class T, bool COLVEC>
 __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, const float* lds_c, float cmul, int m,
                                           uint8_t* head, uint16_t* sc_head, const LaneId& l) {
+    if constexpr (T::FLT) {
+        float_fold<T, COLVEC>(lds_k, lds_u, lds_c, cmul, m, head, l);
+        return;
+    } else {
     constexpr int NCS = T::NKS;                              // 32-column steps
     constexpr int MT = (T::MMAX + 1) / 2;                    // slot pairs
     constexpr int NL = Window<T>::NL;
@@ -746,6 +916,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
         }
         __syncthreads();
     }
+}
 }
 
 // The fold for value-axis scale groups: one scale per (32-row block, key column), so the block is held "columns

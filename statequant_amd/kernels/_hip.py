@@ -126,7 +126,10 @@ def ptr(t):
 
 def make_layout(st):
     """``SqLayout`` from a layout / state object with the reference's attribute names (bits, axk, group, ...)."""
-    return SqLayout(bits=st.bits, axis_k=int(st.axk), group=st.group, buffer_bits=st.buffer_bits, m=st.m,
+    bits = st.bits                                        # 16: the unquantized state, bf16 -- or fp32 (slot layouts)
+    if st.fmt is None and getattr(st, 'state_dtype', None) == torch.float32:
+        bits = 32
+    return SqLayout(bits=bits, axis_k=int(st.axk), group=st.group, buffer_bits=st.buffer_bits, m=st.m,
                     hv=st.HV, hk=st.HK, dk=st.DK, dv=st.DV)
 
 

@@ -160,12 +160,11 @@ def _flat(S):
 
 def _require_kernel(family, st):
     """Fail at construction, with the reason, when no HIP kernel exists for a layout."""
-    if st.fmt is None:
-        raise NotImplementedError('the unquantized bf16 / fp32 state control is not built for the HIP step yet')
     if not _hip.supported(family, st):
+        what = 'an unquantized state' if st.fmt is None else \
+            f'int{st.bits} {"key" if st.axk else "value"}-axis group {st.group}'
         raise NotImplementedError(
-            f'no HIP kernel instance for {family}: int{st.bits} {"key" if st.axk else "value"}-axis group {st.group}, '
-            f'd_k {st.DK}, d_v {st.DV}, '
+            f'no HIP kernel instance for {family}: {what}, d_k {st.DK}, d_v {st.DV}, '
             f'm {st.m}, buffer_bits {st.buffer_bits} (see statequant_amd/csrc/build.py: CASES)')
 
 

@@ -12,7 +12,8 @@ import statequant_amd as sq
 
 
 def quantizer(fmt):
-    return sq.Quantizer(*fmt)
+    """(bits, axis, group) -> Quantizer; 'bf16' / 'fp32' (the unquantized state controls) pass through."""
+    return fmt if isinstance(fmt, str) else sq.Quantizer(*fmt)
 
 
 def gdn_token(gen, B, HV, HK, DK, DV, dtype=torch.float32, v_scale=None):
@@ -56,11 +57,10 @@ class Tally:
     def fold(self, codes, scales, ref, bits):
         """codes / scales of the kernel (CPU copies) vs the oracle that has just folded the same buffer."""
         self.folds += 1
-        a, b = unpack_nib(codes, bits), unpack_nib(ref.codes, bits)
-        d = (a.int() - b.int()).abs()
-        self.code_mism += (d != 0).sum().item()
-        self.code_far += (d > 1).sum().item()
-        self.code_n += d.numel()
+        mism, far, n = code_diff(codes, ref.codes, bits)
+        self.code_mism += mism
+        self.code_far += far
+        self.code_n += n
         self.scale_mism += (scales != ref.scales).sum().item()
         from oracle.formats import unpack_vk
         deq = unpack_vk(codes, scales, ref.fmt, ref.DK)
@@ -75,9 +75,25 @@ class Tally:
                 f'{self.worst_raw:.2e}; buffer entries flipped {self.buf_flips} of {self.buf_entries}')
 
 
+def code_diff(got, want, bits):
+    """(codes differing, differing by more than one step, codes compared) of two stored states."""
+    d = (unpack_nib(got, bits).int() - unpack_nib(want, bits).int()).abs()
+    if bits == 16:          # bf16 numbers: "one step" is relative, and across zero it is an absolute matter
+        fa, fb = got.float(), want.float()
+        tol = torch.maximum(fa.abs(), fb.abs()) * 2.0 ** -7 + 1e-6 * fb.abs().max()
+        far = ((fa - fb).abs() > tol).sum().item()
+    else:
+        far = (d > 1).sum().item()
+    return (d != 0).sum().item(), far, d.numel()
+
+
 def unpack_nib(codes, bits):
-    """Stored codes -> one integer per code (int4 bytes split into their two nibbles)."""
+    """Stored codes -> one integer per code (int4 bytes split into their two nibbles).  A bf16 state (bits 16): an
+    integer that orders like the value, so that neighbouring bf16 numbers differ by one."""
     if bits == 8:
         return codes.to(torch.int16)
+    if bits == 16:
+        raw = codes.view(torch.int16).int()
+        return torch.where(raw < 0, -(raw & 0x7FFF), raw)
     c = codes.to(torch.int16)
     return torch.stack(((c & 15) - 8, ((c >> 4) & 15) - 8), -1).flatten(-2)

@@ -195,6 +195,7 @@ if __name__ == '__main__':
     run_gdn('gdn_int4.pt', (4, 'k', 32), 2, 4, 2, 64, 64, 4, 8, 14, seed=2, v_head_scale=True)
     run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 64, 1, 8, 4, seed=3, per_key=False)
     run_gdn('gdn_int4v.pt', (4, 'v', 32), 2, 4, 2, 64, 64, 4, 8, 10, seed=8)      # value-axis scale groups
+    run_gdn('gdn_bf16.pt', 'bf16', 2, 4, 2, 64, 64, 4, 8, 10, seed=9)             # the unquantized bf16 state
     run_kda('kda_int4.pt', (4, 'k', 32), 2, 3, 64, 64, 4, 8, 10, seed=4)
     run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 64, 2, 16, 6, seed=5)
     run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 64, 4, 8, 10, seed=6)

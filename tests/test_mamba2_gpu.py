@@ -58,7 +58,7 @@ def run_decode(fmt, m, bb, B=2, H=8, G=2, DK=128, DV=64, T=24, seed=1, dtype=tor
         assert ker.n == ref.n
         if ref.n == 0:
             codes, scales = ker.codes.cpu(), ker.scales.cpu()
-            tal.fold(codes, scales, ref, fmt[0])
+            tal.fold(codes, scales, ref, 16 if fmt == 'bf16' else fmt[0])
             ref.adopt(codes, scales)
         assert torch.equal(ker.NPTR.cpu(), torch.full((B, H), ref.n, dtype=torch.int32))
     return tal
@@ -77,6 +77,14 @@ def check(tal, tag, T, m):
 def test_value_axis_groups(fmt, m, bb):
     T = 24 if m > 1 else 4
     check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
+
+
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('DK,DV', [(128, 64), (128, 128), (64, 64)])
+def test_unquantized_state_control(m, bb, DK, DV):
+    """The bf16 state (mamba2.py:352: the control for the packed formats) through the same step."""
+    T = 3 * m + 2 if m > 1 else 4
+    check(run_decode('bf16', m, bb, DK=DK, DV=DV, T=T), f'mamba2 bf16 state {DK}x{DV} m={m} buf{bb}', T, m)
 
 
 @pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32)])
@@ -171,7 +179,7 @@ def _setup(fmt, m, bb, seed=0):
     return lay, raw, blob, views, slots, refs, (A, D, dtb)
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32)])
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32), 'bf16'])
 @pytest.mark.parametrize('m,bb', [(8, 8), (2, 16)])
 def test_slot_step_matches_lockstep_per_sequence(fmt, m, bb):
     lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup(fmt, m, bb)
@@ -204,7 +212,8 @@ def test_slot_step_matches_lockstep_per_sequence(fmt, m, bb):
                 assert torch.equal(out[b], want[b].view(H, DV)), (t, b)
                 assert views['NPTR'][slots[r], :H].tolist() == [steps[r] % m] * H
                 assert torch.equal(views['S'][slots[r]], refs[r].codes.view(H, *refs[r].codes.shape[1:]))
-                assert torch.equal(views['SC'][slots[r]], refs[r].scales.view(H, *refs[r].scales.shape[1:]))
+                if 'SC' in views:
+                    assert torch.equal(views['SC'][slots[r]], refs[r].scales.view(H, *refs[r].scales.shape[1:]))
             else:
                 assert torch.equal(out[b], torch.zeros_like(out[b]))
     keep = torch.ones_like(raw, dtype=torch.bool)

@@ -73,7 +73,7 @@ def _replay(rec, make, call):
     return worst, flips
 
 
-@pytest.mark.parametrize('name', ['gdn_c1.pt', 'gdn_int4.pt', 'gdn_int8_m1.pt', 'gdn_int4v.pt'])
+@pytest.mark.parametrize('name', ['gdn_c1.pt', 'gdn_int4.pt', 'gdn_int8_m1.pt', 'gdn_int4v.pt', 'gdn_bf16.pt'])
 def test_gdn_steps_and_folds(golden, name):
     rec = golden(name)
     mk = lambda S: ST.GDNOracle(S, rec['fmt'], m=rec['m'], hv=rec['HV'], hk=rec['HK'],      # noqa: E731
