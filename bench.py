@@ -34,31 +34,53 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 
 WORKLOADS = {
-    # name: (family, bits, group, hv, hk, dk, dv, slots, layers)
+    # name: (family, bits, group, hv, hk, dk, dv, slots, layers); group < 0: value-axis groups of -group rows;
+    # bits 16: the unquantized bf16 state (the reference's control)
     'gdn-int8-g128': ('gdn', 8, 128, 32, 16, 128, 128, 256, 24),
     'gdn-int8-g32': ('gdn', 8, 32, 32, 16, 128, 128, 256, 24),
     'gdn-int4-g64': ('gdn', 4, 64, 32, 16, 128, 128, 256, 24),
     'gdn-int4-g32': ('gdn', 4, 32, 32, 16, 128, 128, 256, 24),
+    'gdn-int4v-g32': ('gdn', 4, -32, 32, 16, 128, 128, 256, 24),
+    'gdn-int8v-g32': ('gdn', 8, -32, 32, 16, 128, 128, 256, 24),
+    'gdn-bf16': ('gdn', 16, 128, 32, 16, 128, 128, 256, 24),
     'mamba2-int8-g128': ('mamba2', 8, 128, 128, 8, 128, 64, 128, 24),
     'kda-int4-g32': ('kda', 4, 32, 32, 32, 128, 128, 256, 24),
 }
 
+
+def workload_format(bits, group):
+    """The oracle's / Quantizer's format triple of a workload, 'bf16' for the unquantized state."""
+    return 'bf16' if bits == 16 else (bits, 'v' if group < 0 else 'k', abs(group))
+
+
+def describe_state(bits, group):
+    if bits == 16:
+        return 'bf16, unquantized'
+    return f'int{bits} {"value" if group < 0 else "key"}-axis group {abs(group)}, fp16 scales'
+
 # HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
 # over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
-MEASURED_TRAFFIC = {'gdn-int8-g128': 185291062}
+MEASURED_TRAFFIC = {'gdn-int8-g128': 185269418}
+
+
+def stored_bytes_per_slot(bits, group, hv, dk, dv):
+    codes = hv * dv * dk * bits // 8
+    if bits == 16:
+        return codes
+    scales = hv * (dv // -group) * dk * 2 if group < 0 else hv * dv * (-(-dk // group)) * 2
+    return codes + scales
 
 
 def state_bytes_per_slot(bits, group, hv, dk, dv, m):
-    codes = hv * dv * dk * bits // 8
-    scales = hv * dv * (-(-dk // group)) * 2
-    return (codes + scales) * (1 + 1 / m)
+    return stored_bytes_per_slot(bits, group, hv, dk, dv) * (1 + 1 / m)
 
 
 def build(workload, m, device):
     import statequant_amd as sq
     from statequant_amd.kernels import KDASlotLayout, Mamba2SlotLayout, SlotLayout
     fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[workload]
-    fmt = sq.Quantizer(bits, 'k', group)
+    fmt = workload_format(bits, group)
+    fmt = fmt if fmt == 'bf16' else sq.Quantizer(*fmt)
     if fam == 'gdn':
         lay = SlotLayout(fmt, hv, hk, dk, dv, m=m, buffer_bits=8)
     elif fam == 'kda':
@@ -113,7 +135,7 @@ def cpu_baseline(workload, m, budget_s=20.0):
     gen = torch.Generator().manual_seed(0)
     r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
     S0 = r(slots * hv, dv, dk) * 0.1
-    fmt = (bits, 'k', group)
+    fmt = workload_format(bits, group)
     if fam == 'gdn':
         st = ST.GDNOracle(S0, fmt, m=m, hv=hv, hk=hk, buffer_bits=8)
     elif fam == 'kda':
@@ -191,8 +213,7 @@ def bench_convert(a, lay, views, idx, dev):
     wall = time.perf_counter() - t0
     n = reps * layers
     us = e0.elapsed_time(e1) * 1e3 / n
-    codes = hv * dv * dk * bits // 8 + hv * dv * (-(-dk // group)) * 2
-    alg = slots * (hv * dv * dk * 4 + codes)
+    alg = slots * (hv * dv * dk * 4 + stored_bytes_per_slot(bits, group, hv, dk, dv))
     print(json.dumps({
         'metric': f'us_per_layer_{a.op}', 'value': round(wall * 1e6 / n, 3), 'unit': 'us', 'n_gpus': 1, 'steps': reps,
         'warmup': 1, 'higher_is_better': False, 'dtype': 'f32', 'data': 'synthetic',
@@ -235,7 +256,7 @@ def main():
     if a.op != 'step':
         return bench_convert(a, lay, views, idx, dev)
     inputs, extra = make_inputs(fam, lay, slots, layers, m, dev)
-    out = torch.empty(slots, hv, dv, device=dev, dtype=torch.bfloat16)
+    out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
 
     def period():                                           # m steps x layers launches
         for s in range(m):
@@ -280,7 +301,7 @@ def main():
         'n_gpus': 1, 'steps': a.steps, 'warmup': a.warmup, 'ms_per_step': round(wall * 1e3 / a.steps, 5),
         'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
         'config': {'workload': a.workload, 'family': fam, 'slots': slots, 'layers': layers, 'value_heads': hv,
-                   'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': f'int{bits} key-axis group {group}, fp16 scales',
+                   'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': describe_state(bits, group),
                    'buffer': f'int8, m={m}', 'inputs': 'bf16', 'launch': 'hip-graph' if use_graph else 'eager',
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),

@@ -38,8 +38,11 @@ enum {
 };
 
 /* The stored state and decode buffer of a set of sequences (slots.py:9-22 for the field meanings and shapes).
- * S     codes: int8 [hv, dv, dk] (bits 8) or uint8 [hv, dv, dk/2] (bits 4, byte j = (c[2j]+8) | (c[2j+1]+8) << 4)
- * SC    fp16 scales [hv, dv, ceil(dk/group)] (key-axis groups)
+ * S     codes: int8 [hv, dv, dk] (bits 8) or uint8 [hv, dv, dk/2] (bits 4, byte j = (c[2j]+8) | (c[2j+1]+8) << 4);
+ *       the unquantized control: bf16 (bits 16) or fp32 (bits 32) [hv, dv, dk] (fold.py:128-129, slots.py:55-56)
+ * SC    fp16 scales [hv, dv, ceil(dk/group)] (key-axis groups) or [hv, dv/group, dk] (value-axis groups);
+ *       ignored (may be NULL) for the unquantized control
+ * Every stride s* counts elements of its own tensor per sequence (sS: codes bytes, or bf16 / fp32 elements).
  * KB    buffered keys [hk, m, dk], int8 (buffer_bits 8) or bf16 (16);  KBS fp16 [hk, m] (int8 buffer only)
  * UB    buffered delta values [hv, m, dv], int8 or bf16;               UBS fp16 [hv, m] (int8 buffer only)
  * GB    fp32 cumulative log decay of each buffered token: [hv, m] (GDN, Mamba2) or [hv, m, dk] (KDA)
@@ -59,9 +62,9 @@ typedef struct sq_state {
 
 /* Layer geometry and storage format (fold.py:91-104 `packed_format`, slots.py:53-74). */
 typedef struct sq_layout {
-    int32_t bits;         /* 4 or 8 */
-    int32_t axis_k;       /* 1: scale groups along d_k (the only axis built so far) */
-    int32_t group;        /* scale group length, a power of two */
+    int32_t bits;         /* 4 or 8: codes; 16 / 32: the state kept as bf16 / fp32, no scales (axis_k, group ignored) */
+    int32_t axis_k;       /* 1: scale groups along d_k; 0: along d_v (group rows of one key column share a scale) */
+    int32_t group;        /* scale group length, a power of two (value-axis: must divide d_v; built for 32) */
     int32_t buffer_bits;  /* 8 (int8 + fp16 scale per vector) or 16 (bf16) */
     int32_t m;            /* buffer length, a power of two */
     int32_t hv, hk;       /* value heads, key heads (groups); hv % hk == 0 */
