@@ -232,6 +232,10 @@ def main():
     ap.add_argument('--workload', default='gdn-int8-g128', choices=list(WORKLOADS))
     ap.add_argument('--m', type=int, default=8)
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
+    ap.add_argument('--mixed-fill', action='store_true',
+                    help='start slot s with s %% m tokens in its buffer, so that every step folds 1/m of the slots '
+                         '(sequences of unequal lengths, as a serving engine has them) instead of all slots folding '
+                         'on the same step; a secondary figure, the headline is the lockstep configuration')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--cpu-budget', type=float, default=20.0)
     ap.add_argument('--op', default='step', choices=['step', 'write', 'read'],
@@ -256,6 +260,10 @@ def main():
     if a.op != 'step':
         return bench_convert(a, lay, views, idx, dev)
     inputs, extra = make_inputs(fam, lay, slots, layers, m, dev)
+    if a.mixed_fill:
+        fill = (torch.arange(slots, device=dev, dtype=torch.int32) % m)[:, None]
+        for V in views:
+            V['NPTR'][idx.long()] = fill.expand(slots, V['NPTR'].shape[1])
     out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
 
     def period():                                           # m steps x layers launches
@@ -303,6 +311,7 @@ def main():
         'config': {'workload': a.workload, 'family': fam, 'slots': slots, 'layers': layers, 'value_heads': hv,
                    'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': describe_state(bits, group),
                    'buffer': f'int8, m={m}', 'inputs': 'bf16', 'launch': 'hip-graph' if use_graph else 'eager',
+                   'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
