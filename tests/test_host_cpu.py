@@ -185,3 +185,21 @@ def test_no_fallback_off_the_gpu():
     with pytest.raises(NotImplementedError):
         lay._layout_struct()
     SlotLayout(sq.Quantizer(4, 'v', 32), 4, 2, 128, 128)._layout_struct()
+
+
+def test_bench_contract_off_the_gpu():
+    """bench.py: more than one GPU is refused with a message (the step has no cross-GPU exchange to measure), and the
+    byte model is the one the target is quoted on: (S + SC)(1 + 1/m) per slot and step."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, 'bench.py'), '--gpus', '2'], capture_output=True, text=True)
+    assert r.returncode != 0 and 'one GPU' in r.stderr
+    sys.path.insert(0, root)
+    import bench
+    per_slot = {'gdn-int8-g128': 599040, 'gdn-int8-g32': 626688, 'gdn-int4-g32': 331776, 'gdn-int4-g64': 313344,
+                'mamba2-int8-g128': 1198080, 'kda-int4-g32': 331776, 'gdn-int4v-g32': 331776}
+    for name, want in per_slot.items():
+        fam, bits, group, hv, hk, dk, dv, slots, layers = bench.WORKLOADS[name]
+        assert bench.state_bytes_per_slot(bits, group, hv, dk, dv, 8) == want, name
+    assert bench.state_bytes_per_slot(8, 128, 32, 128, 128, 8) * 256 == 153354240
