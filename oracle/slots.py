@@ -88,6 +88,11 @@ def write(V, idx, S, fmt, hv, dk, dv):
     stay as they are (slots.py:236-252)."""
     idx = idx.long()
     P = idx.shape[0]
+    if 'SC' not in V and V['S'].dtype == torch.float32:          # fp32 state: stored as is (slots.py:242-243)
+        V['S'][idx] = S.reshape(P, *V['S'].shape[1:]).float()
+        V['NPTR'][idx] = 0
+        V['GCUR'][idx] = 0.
+        return
     codes, sc = pack_vk(S.reshape(P * hv, dv, dk), fmt)
     V['S'][idx] = codes.view(P, *V['S'].shape[1:])
     if 'SC' in V:

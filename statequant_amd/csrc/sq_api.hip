@@ -271,24 +271,30 @@ int sq_pack_vk(const sq_pack_args* a, void* stream) {
     const char* who = "sq_pack_vk";
     if (!a) return fail(SQ_E_ARG, "%s: null args", who);
     const sq_layout& L = a->lay;
-    if (L.bits != 4 && L.bits != 8) return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4 or 8, got %d", who, L.bits);
-    if (!L.axis_k) return fail(SQ_E_UNSUPPORTED, "%s: value-axis scale groups are not built", who);
+    if (L.bits != 4 && L.bits != 8 && L.bits != 16 && L.bits != 32)
+        return fail(SQ_E_UNSUPPORTED, "%s: bits must be 4, 8, 16 or 32, got %d", who, L.bits);
+    const bool flt = L.bits >= 16;
     if (L.hv <= 0 || L.dk <= 0 || L.dv <= 0) return fail(SQ_E_ARG, "%s: hv %d, dk %d, dv %d", who, L.hv, L.dk, L.dv);
+    if (!flt && !L.axis_k && (L.group <= 0 || L.dv % L.group))
+        return fail(SQ_E_ARG, "%s: value-axis group %d does not divide d_v %d", who, L.group, L.dv);
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;
-    if (!a->src || !a->S || !a->SC) return fail(SQ_E_ARG, "%s: null src / S / SC", who);
-    const size_t row_align = L.bits == 8 ? 16 : 8;
-    if (!aligned(a->src, 16) || (a->s_src % 4) || !aligned(a->S, row_align) || (a->sS % int64_t(row_align)) ||
-        !aligned(a->SC, 2))
-        return fail(SQ_E_ARG, "%s: src must be 16-byte aligned, codes %zu-byte aligned", who, row_align);
-    if (!stride_ok(a->s_src) || !stride_ok(a->sS) || !stride_ok(a->sSC) || !stride_ok(a->sGC) || !stride_ok(a->sN))
+    if (!a->src || !a->S || (!flt && !a->SC)) return fail(SQ_E_ARG, "%s: null src / S / SC", who);
+    const size_t row_align = L.bits == 4 ? 8 : 16;
+    const int64_t s_bytes = a->sS * (flt ? L.bits / 8 : 1);          // the kernels address the state in bytes
+    if (!aligned(a->src, 16) || (a->s_src % 4) || !aligned(a->S, row_align) || (s_bytes % int64_t(row_align)) ||
+        (!flt && (!aligned(a->SC, 4) || (a->sSC % 2))))
+        return fail(SQ_E_ARG, "%s: src must be 16-byte aligned, the state %zu-byte, scales 4-byte aligned", who,
+                    row_align);
+    if (!stride_ok(a->s_src) || !stride_ok(s_bytes) || !stride_ok(a->sSC) || !stride_ok(a->sGC) || !stride_ok(a->sN))
         return fail(SQ_E_ARG, "%s: strides must be in [0, 2^31)", who);
     if (a->GCUR && a->gcur_per_head <= 0) return fail(SQ_E_ARG, "%s: gcur_per_head %d", who, a->gcur_per_head);
     sq::PackParams p{};
-    p.bits = L.bits; p.group = L.group; p.hv = L.hv; p.dk = L.dk; p.dv = L.dv;
+    p.bits = L.bits; p.group = flt ? L.dk : L.group; p.axv = (flt || L.axis_k) ? 0 : 1;
+    p.hv = L.hv; p.dk = L.dk; p.dv = L.dv;
     p.rows = a->rows; p.idx = a->idx;
     p.src = a->src; p.s_src = uint32_t(a->s_src);
-    p.S = static_cast<uint8_t*>(a->S); p.sS = uint32_t(a->sS);
+    p.S = static_cast<uint8_t*>(a->S); p.sS = uint32_t(s_bytes);
     p.SC = static_cast<uint16_t*>(a->SC); p.sSC = uint32_t(a->sSC);
     p.GCUR = a->GCUR; p.sGC = uint32_t(a->sGC); p.gcur_per_head = a->gcur_per_head;
     p.NPTR = a->NPTR; p.sN = uint32_t(a->sN);
@@ -301,7 +307,6 @@ int sq_read(const sq_read_args* a, void* stream) {
     sq::ReadParams p{};
     SQ_TRY(check_layout(a->lay, who, &p));
     if (a->lay.m > 16) return fail(SQ_E_UNSUPPORTED, "%s: m %d > 16", who, a->lay.m);
-    if (!a->lay.axis_k) return fail(SQ_E_UNSUPPORTED, "%s: value-axis scale groups are not built", who);
     if (a->kda && a->lay.hk != a->lay.hv) return fail(SQ_E_ARG, "%s: KDA has no grouped keys", who);
     if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
     if (a->rows == 0) return SQ_OK;

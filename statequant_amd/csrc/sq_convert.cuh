@@ -5,7 +5,9 @@
 //          S_n = a_n S_0 + sum_{i<n} (a_n / a_i) u_i k_i^T;  KDA: decays per key channel
 //          (reference: kernels/slots.py:210-233, kernels/kda.py:351-372)
 // Both are plain streaming kernels, one wavefront per (sequence, value head): rows in the row shape of the fold
-// (LPRP lanes per row, 16 columns per lane), d_v and m taken at run time.  They are bound by the fp32 side of the
+// (LPRP lanes per row, 16 columns per lane), d_v and m taken at run time.  Value-axis scale groups (32 rows of one key
+// column share a scale) pack with a column shape instead (a lane owns two neighbouring columns of a 32-row block);
+// the unquantized state (bf16 / fp32) packs as a cast.  They are bound by the fp32 side of the
 // transfer (pack reads 4 bytes per code it writes, read writes 4 bytes per code it reads).
 #pragma once
 #include "sq_tile.cuh"
@@ -14,8 +16,16 @@
 namespace sq {
 
 // geometry carrier: only the d_k-shaped members of Tile are used here
-template <int BITS, int DK, int GROUP, bool QBUF>
-using RowTile = Tile<BITS, DK, 128, GROUP, QBUF, 16>;
+template <int BITS, int DK, int GROUP, bool QBUF, bool AXV = false>
+using RowTile = Tile<BITS, DK, 128, GROUP, QBUF, 16, AXV>;
+
+// Empty a sequence's buffer: this head's counter copy and running decay.
+__device__ __forceinline__ void reset_counters(const PackParams& p, uint32_t seq, uint32_t h, int lane) {
+    if (p.NPTR && lane == 0) *field(p.NPTR, seq, p.sN, h) = 0;
+    if (p.GCUR)
+        for (uint32_t e = lane; e < uint32_t(p.gcur_per_head); e += WAVE)
+            *field(p.GCUR, seq, p.sGC, h * uint32_t(p.gcur_per_head) + e) = 0.0f;
+}
 
 template <int BITS, int DK, int GROUP>
 __global__ __launch_bounds__(WAVE) void pack_kernel(const PackParams p) {
@@ -55,16 +65,82 @@ __global__ __launch_bounds__(WAVE) void pack_kernel(const PackParams p) {
         if (in && live) store_row<BITS>(Sh + row * T::ROW_BYTES + l.cg * T::LANE_BYTES, encode_row<BITS>(q));
         if (in && lead) SCh[row * T::NG + gi] = f32_to_f16(s);
     }
-    // empty the buffer: counter copy of this head, running decay of this head
-    if (p.NPTR && l.lane == 0) *field(p.NPTR, seq, p.sN, h) = 0;
-    if (p.GCUR)
-        for (uint32_t e = l.lane; e < uint32_t(p.gcur_per_head); e += WAVE)
-            *field(p.GCUR, seq, p.sGC, h * uint32_t(p.gcur_per_head) + e) = 0.0f;
+    reset_counters(p, seq, h, l.lane);
 }
 
-template <int BITS, int DK, int GROUP>
+// Value-axis groups of 32 rows (fold.py:139-146): scales [dv / 32][DK].  A lane owns columns 2 lane, 2 lane + 1 and
+// walks the 32 rows of a block twice (absmax, then codes) with the block's 64 values in registers.
+template <int BITS, int DK>
+__global__ __launch_bounds__(WAVE) void pack_v_kernel(const PackParams p) {
+    constexpr int G = 32;
+    constexpr float QMAX = float((1 << (BITS - 1)) - 1);
+    constexpr int ROW_BYTES = DK * BITS / 8;
+    static_assert(DK % 2 == 0 && DK <= 2 * WAVE, "two columns per lane");
+    const int lane = threadIdx.x;
+    const uint32_t b = blockIdx.x / uint32_t(p.hv), h = blockIdx.x - b * uint32_t(p.hv);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
+    if (p.idx && slot <= 0) return;
+    const uint32_t seq = slot, dv = p.dv;
+    const float* src = p.src + (uint64_t(b) * p.s_src + uint64_t(h) * dv * DK);
+    uint8_t* Sh = field(p.S, seq, p.sS, h * (dv * ROW_BYTES));
+    uint16_t* SCh = field(p.SC, seq, p.sSC, h * ((dv / G) * DK));
+    const bool live = 2 * lane < DK;
+    const int c0 = live ? 2 * lane : DK - 2;
+    for (uint32_t r0 = 0; r0 < dv; r0 += G) {
+        float2 x[G];
+#pragma unroll
+        for (int r = 0; r < G; ++r) x[r] = *reinterpret_cast<const float2*>(src + (r0 + r) * DK + c0);
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int r = 0; r < G; ++r) { a0 = fmaxf(a0, fabsf(x[r].x)); a1 = fmaxf(a1, fabsf(x[r].y)); }
+        const float s0 = fp16_scale(a0, QMAX), s1 = fp16_scale(a1, QMAX);
+        if (live)
+            *reinterpret_cast<uint32_t*>(SCh + (r0 / G) * DK + c0) = uint32_t(f32_to_f16(s0)) | (uint32_t(f32_to_f16(s1)) << 16);
+#pragma unroll
+        for (int r = 0; r < G; ++r) {
+            const int q0 = int(fminf(fmaxf(rintf(x[r].x / s0), -QMAX), QMAX));
+            const int q1 = int(fminf(fmaxf(rintf(x[r].y / s1), -QMAX), QMAX));
+            uint8_t* row = Sh + (r0 + r) * ROW_BYTES;
+            if (live) {
+                if constexpr (BITS == 8)
+                    *reinterpret_cast<uint16_t*>(row + c0) = uint16_t((q0 & 0xFF) | ((q1 & 0xFF) << 8));
+                else
+                    row[lane] = uint8_t((q0 + 8) | ((q1 + 8) << 4));
+            }
+        }
+    }
+    reset_counters(p, seq, h, lane);
+}
+
+// The unquantized state: a cast to bf16 (round to nearest even) or a copy (fp32), [dv][DK] per head.
+template <int BITS, int DK>
+__global__ __launch_bounds__(WAVE) void pack_f_kernel(const PackParams p) {
+    static_assert(DK % 4 == 0, "four columns per lane and step");
+    const int lane = threadIdx.x;
+    const uint32_t b = blockIdx.x / uint32_t(p.hv), h = blockIdx.x - b * uint32_t(p.hv);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
+    if (p.idx && slot <= 0) return;
+    const uint32_t seq = slot, n = p.dv * DK;
+    const float* src = p.src + (uint64_t(b) * p.s_src + uint64_t(h) * n);
+    uint8_t* Sh = field(p.S, seq, p.sS, h * (n * (BITS / 8)));
+    for (uint32_t e = 4 * lane; e < n; e += 4 * WAVE) {
+        const float4 f = *reinterpret_cast<const float4*>(src + e);
+        if constexpr (BITS == 16)
+            *reinterpret_cast<uint2*>(Sh + 2 * e) =
+                make_uint2(uint32_t(f32_to_bf16(f.x)) | (uint32_t(f32_to_bf16(f.y)) << 16),
+                           uint32_t(f32_to_bf16(f.z)) | (uint32_t(f32_to_bf16(f.w)) << 16));
+        else
+            *reinterpret_cast<float4*>(Sh + 4 * e) = f;
+    }
+    reset_counters(p, seq, h, lane);
+}
+
+// AXV: value-axis groups (GROUP = 32); BITS 16 / 32: the unquantized state (GROUP = DK).
+template <int BITS, int DK, int GROUP, bool AXV>
 int launch_pack(const PackParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL((pack_kernel<BITS, DK, GROUP>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    if constexpr (BITS >= 16) hipLaunchKernelGGL((pack_f_kernel<BITS, DK>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    else if constexpr (AXV) hipLaunchKernelGGL((pack_v_kernel<BITS, DK>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((pack_kernel<BITS, DK, GROUP>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     return int(hipGetLastError());
 }
 
@@ -72,9 +148,9 @@ int launch_pack(const PackParams& p, hipStream_t stream) {
 // Column split of the output pass: a lane takes NCH chunks of 4 columns, chunk t = columns 4 LPR t + 4 cg .. + 3, so
 // that the LPR lanes of a row write 16 LPR consecutive bytes with every store instruction (whole 128-byte lines for
 // d_k = 128) -- with 16 consecutive columns per lane each store would scatter 16-byte pieces 64 bytes apart.
-template <int BITS, int DK, int GROUP, bool QBUF, bool KDA>
+template <int BITS, int DK, int GROUP, bool QBUF, bool KDA, bool AXV>
 __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
-    using T = RowTile<BITS, DK, GROUP, QBUF>;
+    using T = RowTile<BITS, DK, GROUP, QBUF, AXV>;
     constexpr int NCH = CPL / 4;
     constexpr int CSTEP = 4 * T::LPR;                             // columns between a lane's chunks
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -90,7 +166,7 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     if (p.idx && slot <= 0) return;
     const uint32_t seq = slot;
     const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (dv * T::ROW_BYTES));
-    const uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * (dv * T::NG));
+    const uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, AXV ? h * ((dv / GROUP) * DK) : h * (dv * T::NG));
     const uint8_t* KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
     const uint8_t* UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * dv) * T::BE;
     const uint16_t* KBS = field(p.st.KBS, seq, p.st.sKBS, hk * um);
@@ -146,9 +222,27 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
 #pragma unroll
             for (int t = 0; t < NCH; ++t) {
                 const int col = t * CSTEP + 4 * cc;
-                const float s = f16_to_f32(SCh[rc[k] * T::NG + col / GROUP]);
-                float c4[4];
-                if constexpr (BITS == 8) {
+                float s4[4], c4[4];
+                if constexpr (T::FLT) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) s4[c] = 1.0f;
+                } else if constexpr (AXV) {                       // one scale per (32-row block, column)
+                    const uint2 w = *reinterpret_cast<const uint2*>(SCh + (rc[k] / GROUP) * DK + col);
+                    s4[0] = f16_to_f32(uint16_t(w.x)); s4[1] = f16_to_f32(uint16_t(w.x >> 16));
+                    s4[2] = f16_to_f32(uint16_t(w.y)); s4[3] = f16_to_f32(uint16_t(w.y >> 16));
+                } else {
+                    const float s = f16_to_f32(SCh[rc[k] * T::NG + col / GROUP]);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) s4[c] = s;
+                }
+                if constexpr (BITS == 32) {
+                    const float4 w = *reinterpret_cast<const float4*>(Sh + rc[k] * T::ROW_BYTES + 4 * col);
+                    c4[0] = w.x; c4[1] = w.y; c4[2] = w.z; c4[3] = w.w;
+                } else if constexpr (BITS == 16) {
+                    const uint2 w = *reinterpret_cast<const uint2*>(Sh + rc[k] * T::ROW_BYTES + 2 * col);
+                    c4[0] = as_f32(w.x << 16); c4[1] = as_f32(w.x & 0xFFFF0000u);
+                    c4[2] = as_f32(w.y << 16); c4[3] = as_f32(w.y & 0xFFFF0000u);
+                } else if constexpr (BITS == 8) {
                     const uint32_t w = *reinterpret_cast<const uint32_t*>(Sh + rc[k] * T::ROW_BYTES + col);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) c4[c] = s8_to_f(w, c);
@@ -158,7 +252,7 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
                     for (int c = 0; c < 4; ++c) c4[c] = float(int32_t((w >> (4 * c)) & 0xFu) - 8);
                 }
 #pragma unroll
-                for (int c = 0; c < 4; ++c) acc[k][t][c] = alpha_p[t][c] * (c4[c] * s);
+                for (int c = 0; c < 4; ++c) acc[k][t][c] = alpha_p[t][c] * (c4[c] * s4[c]);
             }
         }
         for (int i = 0; i < n; ++i) {                             // live slots only
@@ -188,11 +282,10 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     }
 }
 
-template <int BITS, int DK, int GROUP, bool QBUF, bool KDA>
+template <int BITS, int DK, int GROUP, bool QBUF, bool KDA, bool AXV>
 int launch_read(const ReadParams& p, hipStream_t stream) {
-    using T = RowTile<BITS, DK, GROUP, QBUF>;
     const size_t lds = size_t(p.m) * (DK + p.dv) * sizeof(float);
-    hipLaunchKernelGGL((read_kernel<BITS, DK, GROUP, QBUF, KDA>), dim3(p.rows * p.hv), dim3(WAVE), lds, stream, p);
+    hipLaunchKernelGGL((read_kernel<BITS, DK, GROUP, QBUF, KDA, AXV>), dim3(p.rows * p.hv), dim3(WAVE), lds, stream, p);
     return int(hipGetLastError());
 }
 

@@ -74,7 +74,7 @@ struct Mamba2Params : LayoutKey {
 };
 
 struct PackParams {
-    int bits, group, hv, dk, dv;
+    int bits, group, axv, hv, dk, dv;              // axv: value-axis scale groups; bits 16 / 32: unquantized state
     int rows;
     const int32_t* idx;
     const float* src;  uint32_t s_src;            // [rows, hv, dv, dk] fp32, row stride in elements

@@ -157,13 +157,14 @@ def check(rc):
 
 
 def pack_into(lay, src, S, sS, SC, sSC, idx=None, GCUR=None, sGC=0, gcur_per_head=1, NPTR=None, sN=0):
-    """``sq_pack_vk``: fp32 value-major ``src`` [rows, hv, dv, dk] (contiguous) -> codes ``S`` / scales ``SC`` of the
-    sequences ``idx`` (int32; None: sequence b), optionally emptying their buffers.  Returns False when the library has
+    """``sq_pack_vk``: fp32 value-major ``src`` [rows, hv, dv, dk] (contiguous) -> codes ``S`` / scales ``SC`` (None
+    for an unquantized state, which is cast) of the sequences ``idx`` (int32; None: sequence b), optionally emptying
+    their buffers.  Returns False when the library has
     no instance for the format (the caller then packs with torch), raises on any other error."""
     assert src.dtype == torch.float32 and src.is_contiguous()
     rows = src.shape[0]
     a = SqPackArgs(lay=lay, rows=rows, idx=ptr(idx), src=src.data_ptr(), s_src=src.stride(0) if rows else 0,
-                   S=S.data_ptr(), sS=sS, SC=SC.data_ptr(), sSC=sSC, GCUR=ptr(GCUR), sGC=sGC,
+                   S=S.data_ptr(), sS=sS, SC=ptr(SC), sSC=sSC, GCUR=ptr(GCUR), sGC=sGC,
                    gcur_per_head=gcur_per_head, NPTR=ptr(NPTR), sN=sN)
     rc = lib().sq_pack_vk(C.byref(a), current_stream(src.device))
     if rc == E_UNSUPPORTED:

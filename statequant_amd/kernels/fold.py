@@ -99,11 +99,13 @@ def pack_vk(x, fmt):
         return x.to(torch.bfloat16).contiguous(), torch.ones(1, device=x.device, dtype=torch.float16)
     g = fmt.group
     qmax = float(2 ** (fmt.bits - 1) - 1)
-    if x.is_cuda and fmt.axis == 'k' and n:               # the HIP pack kernel (same arithmetic, one launch)
+    if x.is_cuda and n and (fmt.axis == 'k' or dv % g == 0):          # the HIP pack kernels (same arithmetic, one launch)
         codes = torch.empty(n, dv, dk if fmt.bits == 8 else dk // 2, device=x.device,
                             dtype=torch.int8 if fmt.bits == 8 else torch.uint8)
-        sc = torch.empty(n, dv, -(-dk // g), device=x.device, dtype=torch.float16)
-        lay = _hip.SqLayout(bits=fmt.bits, axis_k=1, group=g, buffer_bits=8, m=1, hv=1, hk=1, dk=dk, dv=dv)
+        sc = torch.empty((n, dv, -(-dk // g)) if fmt.axis == 'k' else (n, dv // g, dk), device=x.device,
+                         dtype=torch.float16)
+        lay = _hip.SqLayout(bits=fmt.bits, axis_k=int(fmt.axis == 'k'), group=g, buffer_bits=8, m=1, hv=1, hk=1,
+                            dk=dk, dv=dv)
         if _hip.pack_into(lay, x.contiguous().view(n, 1, dv, dk), codes, codes[0].numel(), sc, sc[0].numel()):
             return codes, sc
     if fmt.axis == 'k':

@@ -208,9 +208,9 @@ class SlotLayout:
         return unpack_vk(codes, sc, self.fmt, self.DK).view(P, self.HV, self.DV, self.DK)
 
     def _hip_format(self, views):
-        """Key-axis int4 / int8 states on the GPU go through the HIP pack / read kernels; the unpacked and value-axis
-        formats (layout-only here) keep the reference's torch formulation."""
-        return self.fmt is not None and self.axk and views['S'].is_cuda
+        """States on the GPU go through the HIP pack / read kernels (a layout the library has no instance for falls
+        back to the reference's torch formulation below; CPU tensors always take it)."""
+        return views['S'].is_cuda
 
     def _read_hip(self, views, idx, kda):
         if not self._hip_format(views) or idx.shape[0] == 0:
@@ -251,7 +251,9 @@ class SlotLayout:
         if self._hip_format(views) and P:
             src = S.reshape(P, self.HV, self.DV, self.DK).float().contiguous()
             gc = V['GCUR']
-            if _hip.pack_into(_hip.make_layout(self), src, V['S'], V['S'].stride(0), V['SC'], V['SC'].stride(0),
+            sc = V.get('SC')
+            if _hip.pack_into(_hip.make_layout(self), src, V['S'], V['S'].stride(0), sc,
+                              sc.stride(0) if sc is not None else 0,
                               idx=idx.to(torch.int32).contiguous(), GCUR=gc, sGC=gc.stride(0),
                               gcur_per_head=gc[0].numel() // self.HV, NPTR=V['NPTR'], sN=V['NPTR'].stride(0)):
                 return

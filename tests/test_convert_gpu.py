@@ -1,6 +1,7 @@
 """The HIP pack (`sq_pack_vk`: ``pack_vk`` / ``SlotLayout.write``) and read (`sq_read`: ``SlotLayout.read``) kernels
 against the CPU oracle.  pack / write: bit-exact (same IEEE divisions and rounding as the reference's torch code,
 fold.py:123-147, slots.py:236-252).  read: fp32 sums in another order than torch's einsum -> 1e-5 relative.
+Formats: key-axis groups, value-axis groups of 32 rows, and the unquantized bf16 / fp32 state.
 """
 import pytest
 import torch
@@ -17,10 +18,10 @@ pytestmark = pytest.mark.gpu
 DEV = 'cuda'
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32)])
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32), (8, 'v', 32), (4, 'v', 32)])
 @pytest.mark.parametrize('dv,dk', [(128, 128), (64, 64), (192, 96), (96, 96)])
 def test_pack_matches_oracle(fmt, dv, dk):
-    if fmt[2] > (1 << (dk - 1).bit_length()):
+    if fmt[1] == 'k' and fmt[2] > (1 << (dk - 1).bit_length()):
         pytest.skip('group longer than the padded row')
     gen = torch.Generator().manual_seed(dv + dk + fmt[0] + fmt[2])
     x = torch.randn(37, dv, dk, generator=gen)
@@ -29,6 +30,7 @@ def test_pack_matches_oracle(fmt, dv, dk):
     x[2] *= 1e-6                                           # scales in the fp16 subnormal range
     x[3] *= 1e4
     x[4, 5] = 65504.0 * 127                                # scale at the top of fp16
+    x[5, :32, 7] = 0.0                                     # value-axis: an all-zero group next to live ones
     codes, sc = pack_vk(x.to(DEV), quantizer(fmt))
     want_c, want_s = OF.pack_vk(x, fmt)
     assert codes.dtype == want_c.dtype and codes.shape == want_c.shape and sc.shape == want_s.shape
@@ -45,15 +47,16 @@ def _blob_pair(lay, table_args, n_slots, seed):
     return gen, table, raw, dev
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 64), (4, 'k', 32)])
+@pytest.mark.parametrize('fmt', [(8, 'k', 64), (4, 'k', 32), (4, 'v', 32), (8, 'v', 32), 'bf16', 'fp32'])
 def test_write_matches_oracle_whole_blob(fmt):
     HV, HK, D, m = 4, 2, 128, 8
     lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=8)
-    gen, table, raw, dev = _blob_pair(lay, ('gdn', fmt, HV, HK, D, D, m, 8), 9, 1)
+    ofmt, sdt = ('bf16', torch.float32) if fmt == 'fp32' else (fmt, torch.bfloat16)
+    gen, table, raw, dev = _blob_pair(lay, ('gdn', ofmt, HV, HK, D, D, m, 8, sdt), 9, 1)
     idx = torch.tensor([7, 2, 5])
     S = torch.randn(3, HV, D, D, generator=gen)
     lay.write(lay.views(dev), idx.to(DEV), S.to(DEV))
-    OS.write(OS.views(table, raw), idx, S, fmt, HV, D, D)
+    OS.write(OS.views(table, raw), idx, S, ofmt, HV, D, D)
     assert torch.equal(dev.cpu(), raw)                    # codes, scales, counters, decays -- and nothing else
 
 
@@ -63,11 +66,13 @@ def _advance(lay, views, step_fn, schedule):
         step_fn(torch.tensor(live, dtype=torch.int32, device=DEV))
 
 
-@pytest.mark.parametrize('fmt,bb', [((8, 'k', 128), 8), ((4, 'k', 32), 16)])
+@pytest.mark.parametrize('fmt,bb', [((8, 'k', 128), 8), ((4, 'k', 32), 16), ((4, 'v', 32), 8), ((8, 'v', 32), 16),
+                                    ('bf16', 8), ('fp32', 16)])
 def test_gdn_read_matches_oracle(fmt, bb):
     HV, HK, D, m = 4, 2, 128, 8
     lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=bb)
-    gen, table, raw, dev = _blob_pair(lay, ('gdn', fmt, HV, HK, D, D, m, bb), 6, 2)
+    ofmt, sdt = ('bf16', torch.float32) if fmt == 'fp32' else (fmt, torch.bfloat16)
+    gen, table, raw, dev = _blob_pair(lay, ('gdn', ofmt, HV, HK, D, D, m, bb, sdt), 6, 2)
     views = lay.views(dev)
     slots = torch.tensor([1, 3, 4, 5])
     lay.write(views, slots.to(DEV), (torch.randn(4, HV, D, D, generator=gen) * 0.5).to(DEV))
@@ -79,13 +84,14 @@ def test_gdn_read_matches_oracle(fmt, bb):
 
     _advance(lay, views, step, [[1, 3, 4]] * 3 + [[3, 4]] * 2 + [[4]] * 5)         # fills 3, 5, 10 % 8 = 2, 0
     got = lay.read(views, slots.to(DEV)).cpu()
-    want = OS.read(OS.views(table, dev.cpu()), slots, fmt, HV, HK, D, D, m)
+    want = OS.read(OS.views(table, dev.cpu()), slots, ofmt, HV, HK, D, D, m)
     assert (views['NPTR'][slots.to(DEV), 0].cpu() & (m - 1)).tolist() == [3, 5, 2, 0]
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())
 
 
-def test_kda_read_matches_oracle():
-    H, DK, DV, m, fmt = 4, 128, 128, 8, (4, 'k', 32)
+@pytest.mark.parametrize('fmt', [(4, 'k', 32), (8, 'v', 32), 'bf16'])
+def test_kda_read_matches_oracle(fmt):
+    H, DK, DV, m = 4, 128, 128, 8
     lay = KDASlotLayout(quantizer(fmt), H, DK, DV, m=m, buffer_bits=8)
     gen, table, raw, dev = _blob_pair(lay, ('kda', fmt, H, H, DK, DV, m, 8), 5, 3)
     views = lay.views(dev)
@@ -104,8 +110,9 @@ def test_kda_read_matches_oracle():
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())
 
 
-def test_mamba2_read_matches_oracle():
-    H, G, DK, DV, m, fmt = 8, 2, 128, 64, 8, (8, 'k', 128)
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'v', 32), 'bf16'])
+def test_mamba2_read_matches_oracle(fmt):
+    H, G, DK, DV, m = 8, 2, 128, 64, 8
     lay = Mamba2SlotLayout(quantizer(fmt), H, G, DK, DV, m=m, buffer_bits=8)
     gen, table, raw, dev = _blob_pair(lay, ('mamba2', fmt, H, G, DK, DV, m, 8), 5, 4)
     views = lay.views(dev)
