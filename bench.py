@@ -231,6 +231,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=512)
     ap.add_argument('--workload', default='gdn-int8-g128', choices=list(WORKLOADS))
     ap.add_argument('--m', type=int, default=8)
+    ap.add_argument('--slots', type=int, default=None,
+                    help='number of sequences instead of the workload\'s own (the reference quotes batch 128 and 512)')
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
     ap.add_argument('--mixed-fill', action='store_true',
                     help='start slot s with s %% m tokens in its buffer, so that every step folds 1/m of the slots '
@@ -255,6 +257,9 @@ def main():
     if a.calibrate_copy:
         return calibrate_copy(dev)
     m = a.m
+    if a.slots:
+        w = WORKLOADS[a.workload]
+        WORKLOADS[a.workload] = w[:7] + (a.slots,) + w[8:]
     fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
     fam, lay, views, idx = build(a.workload, m, dev)
     if a.op != 'step':
