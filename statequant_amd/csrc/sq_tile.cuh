@@ -621,12 +621,13 @@ __device__ __forceinline__ void buffer_term(const uint8_t* lds_ub, const float (
                                             const float (&c)[NV][T::MMAX], int n, int m, int r, float (&acc)[NV]) {
 #pragma unroll
     for (int i = 0; i < T::MMAX; ++i) {
-        float uv = ub_lds<T>(lds_ub, i < m ? i : m - 1, r);
-        if constexpr (!T::QBUF) uv = i < n ? uv : 0.0f;
+        if (i < n) {                                     // wave-uniform: a dead slot would add exactly zero
+            const float uv = ub_lds<T>(lds_ub, i, r);
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const float cu = !T::QBUF ? c[v][i] : i < n ? c[v][i] * ubs[i] : 0.0f;    // (dead slot: any scale)
-            acc[v] = __builtin_fmaf(uv, cu, acc[v]);
+            for (int v = 0; v < NV; ++v) {
+                const float cu = !T::QBUF ? c[v][i] : c[v][i] * ubs[i];
+                acc[v] = __builtin_fmaf(uv, cu, acc[v]);
+            }
         }
     }
 }
