@@ -116,13 +116,15 @@ def make_inputs(fam, lay, slots, layers, m, device, seed=1):
     return out, extra
 
 
-def launch(fam, lay, views, idx, inp, extra, out):
+def launch(fam, lay, views, idx, inp, extra, out, order=None):
     if fam == 'gdn':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'])
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'],
+                 order=order)
     elif fam == 'kda':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out)
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out, order=order)
     else:
-        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'])
+        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'],
+                 order=order)
 
 
 def cpu_baseline(workload, m, budget_s=20.0):
@@ -231,6 +233,10 @@ def main():
     ap.add_argument('--warmup', type=int, default=512)
     ap.add_argument('--workload', default='gdn-int8-g128', choices=list(WORKLOADS))
     ap.add_argument('--m', type=int, default=8)
+    ap.add_argument('--fold-first', action='store_true',
+                    help='hand every launch a dispatch order with the rows that fold on this step first '
+                         '(SlotLayout.fold_first, computed once per step from the first layer\'s counters, inside the '
+                         'timed region); meant for --mixed-fill')
     ap.add_argument('--slots', type=int, default=None,
                     help='number of sequences instead of the workload\'s own (the reference quotes batch 128 and 512)')
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
@@ -273,8 +279,9 @@ def main():
 
     def period():                                           # m steps x layers launches
         for s in range(m):
+            order = lay.fold_first(views[0], idx) if a.fold_first else None
             for L in range(layers):
-                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out)
+                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out, order)
 
     use_graph = not a.no_graph and a.steps % m == 0 and a.warmup % m == 0 and a.steps > 0
     stream = torch.cuda.Stream()
@@ -290,8 +297,9 @@ def main():
         else:
             def run(n):
                 for s in range(n):
+                    order = lay.fold_first(views[0], idx) if a.fold_first else None
                     for L in range(layers):
-                        launch(fam, lay, views[L], idx, inputs[(s % m) * layers + L], extra, out)
+                        launch(fam, lay, views[L], idx, inputs[(s % m) * layers + L], extra, out, order)
             done = 0
         run(max(a.warmup - done, 0))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -317,6 +325,7 @@ def main():
                    'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': describe_state(bits, group),
                    'buffer': f'int8, m={m}', 'inputs': 'bf16', 'launch': 'hip-graph' if use_graph else 'eager',
                    'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
+                   'dispatch_order': 'folding rows first' if a.fold_first else 'natural',
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',

@@ -27,12 +27,14 @@ struct LayoutKey {
     // two (else -1: the kernel divides), and tiles per XCD when the tile count is a multiple of 8 (else 0: no XCD
     // mapping)
     int gqa, hv_shift, gqa_shift, per_xcd;
+    int rows_per_xcd;                             // batch rows per XCD range when those ranges hold whole rows, else 0
 };
 
 struct GdnParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;                         // optional dispatch order of the rows (null: natural)
     const void *q, *k, *v;
     uint32_t s_q, s_k, s_v;
     int q_dt, k_dt, v_dt;
@@ -50,6 +52,7 @@ struct KdaParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;
     const void *q, *k, *v, *g, *beta;
     uint32_t s_q, s_k, s_v, s_g, s_beta;
     int q_dt, k_dt, v_dt, g_dt, beta_dt;
@@ -63,6 +66,7 @@ struct Mamba2Params : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;
     const void *x, *dt, *B, *C, *A, *D, *dt_bias;
     uint32_t s_x, s_dt, s_B, s_C;
     int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
@@ -97,6 +101,8 @@ int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
 int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
 int dispatch_mamba2(const Mamba2Params& p, hipStream_t stream, bool run);
 int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
+int launch_fold_first(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,
+                      hipStream_t stream);
 int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
 
 }  // namespace sq

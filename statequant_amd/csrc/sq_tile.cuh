@@ -130,7 +130,7 @@ __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG
 
 // Which (batch row, value head, key head) a workgroup works on.  Consecutive workgroup ids are dealt round-robin to
 // the 8 XCDs; with `per_xcd` set every XCD walks a contiguous range of tiles, so the heads of one sequence (shared key
-// buffer, neighbouring counters) meet in one L2.
+// buffer, neighbouring counters) meet in one L2.  `order` (optional) names the batch row of each position.
 struct TileId {
     int b, h, hk;
 };
@@ -141,6 +141,16 @@ __device__ __forceinline__ TileId tile_id(const K& k) {
     TileId t;
     t.b = k.hv_shift >= 0 ? tile >> k.hv_shift : tile / k.hv;
     t.h = tile - t.b * k.hv;
+    if (k.order) {
+        // the caller's order is a priority list: its entries are dealt round-robin to the XCDs' row ranges, so that
+        // every XCD starts with its share of the first entries
+        int pos = t.b;
+        if (k.rows_per_xcd) {
+            const int x = pos / k.rows_per_xcd;
+            pos = (pos - x * k.rows_per_xcd) * 8 + x;
+        }
+        t.b = k.order[pos];
+    }
     t.hk = k.gqa_shift >= 0 ? t.h >> k.gqa_shift : t.h / k.gqa;
     return t;
 }
