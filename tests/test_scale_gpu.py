@@ -93,6 +93,27 @@ def test_dispatch_order_changes_nothing_but_the_schedule():
         assert torch.equal(blobs[0], blobs[1]), t
 
 
+@pytest.mark.parametrize('rows', [1, 7, 256, 601])
+def test_fold_first_is_a_stable_three_class_order(rows):
+    """`sq_fold_first`: folding rows, then the other live rows, then padding rows, each class in its natural order
+    (more rows than the helper's workgroup has threads: several passes per class)."""
+    m = 8
+    lay = SlotLayout(sq.Quantizer(8, 'k', 128), 4, 2, 128, 128, m=m)
+    gen = torch.Generator().manual_seed(rows)
+    n_slots = rows + 3
+    views = lay.views(lay.alloc(n_slots, DEV))
+    views['NPTR'][:] = torch.randint(0, 4 * m, (n_slots, views['NPTR'].shape[1]), generator=gen).to(torch.int32).to(DEV)
+    idx = (torch.randperm(rows, generator=gen) + 1).to(torch.int32)
+    idx[torch.rand(rows, generator=gen) < 0.2] = 0
+    if rows > 3:
+        idx[2] = -1
+    got = lay.fold_first(views, idx.to(DEV)).cpu()
+    n = views['NPTR'][idx.long().clamp_min(0), 0].cpu() & (m - 1)
+    cls = torch.where(idx <= 0, 2, torch.where(n == m - 1, 0, 1))
+    want = torch.argsort(cls, stable=True).to(torch.int32)
+    assert torch.equal(got, want)
+
+
 def test_graph_replay_matches_eager():
     HV, HK, D, m, slots = 8, 4, 128, 4, 6
     fmt = (8, 'k', 64)
