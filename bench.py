@@ -19,6 +19,11 @@ step kernel against HBM: achieved = algorithmic state bytes per launch / average
 algorithmic bytes are (codes + scales) x (1 + 1/m) per slot (read every step, rewritten once per m steps) x slots.
 ``cpu_baseline`` times the CPU oracle (a torch restatement of the reference's own CPU path) on this box's host cores
 on a bounded sample of the same workload; it is a reported baseline, not a target.
+
+Secondary figures: ``--workload`` (the other formats and families), ``--slots N`` (other batch sizes), ``--op write |
+read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots)
+with or without ``--fold-first`` (the step calls' optional dispatch order, folding rows first), ``--calibrate-copy``
+(the known-size copy that the HBM counters are scaled by).
 """
 import argparse
 import json
