@@ -13,6 +13,10 @@ What is recorded (CPU, fp32, torch.manual_seed per case):
   kda_*.pt       ReferenceKDAState, likewise;   m2_*.pt  ReferenceMamba2State, likewise
   slots_*.pt     SlotLayout / KDASlotLayout / Mamba2SlotLayout: field tables, `write` then `read` on a blob with a
                  partly filled buffer
+  gga.pt         the mixed-width GGA / STEP slot: `step_quant.fit` and `methods_ext.gga.fp8_vec` on seeded inputs (all
+                 widths, zero and tiny vectors), the `GGAPacked` offset tables and bits-per-value figures, and decode
+                 steps of the `PureWrite` / `StepQuant` reference path driven as the reference's tests/test_vllm_gga.py
+                 drives it (per step: tokens, output, stored state, queued pairs), with and without the window
 """
 import os
 import sys
@@ -188,6 +192,93 @@ def golden_slots():
     save('slots.pt', out)
 
 
+def golden_gga():
+    from statequant.families import BY_NAME, Piece
+    from statequant.integrations.vllm_gga import GGAPacked
+    from statequant.methods_ext.gga import fp8_vec
+    from statequant.step_quant import fit
+    GDN = BY_NAME['gdn']
+    out = {}
+    # -- the fit: every width, columns spanning three decades, a zero row, a zero column, a zero head
+    g = torch.Generator().manual_seed(0)
+    bits = torch.tensor([2, 4, 6, 8, 16, 4])
+    w = torch.rand(6, 64, generator=g) + 0.5
+    x = torch.randn(2, 6, 64, 64, generator=g) * torch.logspace(-3, 0, 64)
+    x[0, 1, 5, :] = 0
+    x[0, 3, :, 7] = 0
+    x[1, 5] = 0
+    out['fit'] = dict(x=x, bits=bits, w=w, y=fit(x, bits, w))
+    v = torch.randn(12, 64, generator=g)
+    v[1] = 0
+    v[2] *= 1e-40
+    v[3] *= 1e-30
+    v[4] *= 1e4
+    v[5, 0] = 0
+    out['fp8'] = dict(x=v, y=fp8_vec(v))
+    # -- offset tables and storage accounting (the plan of the reference's tests/test_gga_packed.py)
+    HV, D = 8, 128
+    widths = [[2, 4, 6, 8, 16, 2, 4, 6], [8, 6, 4, 2, 2, 16, 8, 4]]
+    q = sq.GGA(4, pivots=1)
+    q.plan = {i: (torch.tensor(widths[i]), torch.rand(HV, D, generator=g) + 0.5) for i in range(2)}
+    q.masks = {i: b == 16 for i, (b, _) in q.plan.items()}
+    tab = dict(widths=widths, hv=HV, dk=D, dv=D, m=8, step_bits=q.bits_per_value(D, D),
+               pw_bits=sq.pure_write(q).bits_per_value(D, D))
+    for pw in (False, True):
+        pk = GGAPacked(q, HV, 4, D, D, pw=pw)
+        tab[pw] = dict(offs=[pk.tables[i][0] for i in range(2)], bytes_per_layer=[pk.bytes_per_layer[i] for i in range(2)],
+                       QOFF=pk.QOFF, QSZ=pk.QSZ, nbytes=pk.nbytes, bits_per_value=pk.bits_per_value())
+    out['tables'] = tab
+
+    # -- decode steps of the reference path (PureWrite around the plan; without the window the plan's own rounding)
+    def run(pw, m, T, seed):
+        B, HV, HK, D = 2, 4, 2, 32
+        gg = torch.Generator().manual_seed(seed)
+        r = lambda *s: torch.randn(*s, generator=gg)      # noqa: E731
+        qq = sq.GGA(4, pivots=1)
+        qq.plan = {0: (torch.tensor([2, 4, 16, 8]), torch.rand(HV, D, generator=gg) + 0.5)}
+        qq.masks = {0: qq.plan[0][0] == 16}
+        S0 = r(B, HV, D, D) * 0.3
+        O = qq.quantize(S0, 0)
+        rec = dict(pw=pw, m=m, hv=HV, hk=HK, dk=D, dv=D, bits=qq.plan[0][0], w=qq.plan[0][1], S0=S0, O0=O,
+                   scale=D ** -0.5, steps=[])
+        ref = sq.pure_write(qq, m=m) if pw else qq
+        if pw:
+            ref.reset()
+            ref.layers[0] = {'O': O, 'Q': [], 'R': []}
+        for t in range(T):
+            tq, tk, tv, ta, tb = r(B, HK, D), r(B, HK, D), r(B, HV, D), r(B, HV) * 0.5 - 2, r(B, HV)
+            kw = {'q': tq[:, None], 'k': tk[:, None], 'v': tv[:, None], 'g': ta[:, None], 'beta': tb[:, None],
+                  'A_log': torch.zeros(HV), 'dt_bias': torch.zeros(HV), 'use_gate_in_kernel': True,
+                  'use_beta_sigmoid_in_kernel': True, 'use_qk_l2norm_in_kernel': True, 'scale': D ** -0.5}
+            x = GDN.inputs(kw)
+
+            def delta(S):
+                Sa = x['log_decay'][:, 0].exp()[..., None, None] * S
+                u = x['beta'][:, 0][..., None] * (x['v'][:, 0] - torch.einsum('bhkv,bhk->bhv', Sa, x['k'][:, 0]))
+                Sn = Sa + x['k'][:, 0][..., None] * u[:, :, None]
+                return torch.einsum('bhkv,bhk->bhv', Sn, x['q'][:, 0]), Sn
+            pos = torch.full((B,), 3 + t)
+            if pw:
+                S = ref.prepare(ref._logical(ref.layers[0]), 0, Piece(kw, GDN, 0, None, pos))
+                o, Sn = delta(S)
+                d = ref.output_delta(0)
+                o = o if d is None else o + d[:, 0]
+                ref.piece(Sn, 0, Piece(kw, GDN, 0, S, pos, hit=torch.ones(B, dtype=torch.bool)))
+                O = ref.layers[0]['O']
+                Q = ref.layers[0]['Q']
+                P = torch.stack([p for p, _ in Q], 1)                     # [B, n, HV, d_k], oldest first
+                V = torch.stack([v_ for _, v_ in Q], 1)
+            else:
+                o, Sn = delta(O)
+                O = qq.quantize(Sn, 0)
+                P = V = None
+            rec['steps'].append(dict(q=tq, k=tk, v=tv, a=ta, b=tb, o=o.clone(), O=O.clone(), P=P, V=V))
+        return rec
+    out['steps_pw'] = run(True, 4, 11, 5)
+    out['steps_plain'] = run(False, 1, 4, 6)
+    save('gga.pt', out)
+
+
 if __name__ == '__main__':
     golden_pack()
     # config-1 shape (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start) in a 17-step excerpt (two folds)
@@ -201,3 +292,4 @@ if __name__ == '__main__':
     run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 64, 4, 8, 10, seed=6)
     run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 128, 64, 2, 16, 6, seed=7)
     golden_slots()
+    golden_gga()
