@@ -13,6 +13,10 @@
  *   sq_mamba2_step  _mamba2_triton.py:48 `_m2_step`, launched from mamba2.py:223-241
  *   sq_pack_vk      fold.py:123-147 `pack_vk` / slots.py:236-252 `write` (torch in the reference)
  *   sq_read         slots.py:210-233, kda.py:351-372 `read` (torch in the reference)
+ *   sq_gga_step     _gga_triton.py:207 `_gga_step` + :300 `_gga_advance`, launched from
+ *                   ../integrations/vllm_gga.py:240-253 (`GGAPacked.step`)
+ *   sq_gga_store    _gga_triton.py:314 `_gga_store` (vllm_gga.py:305-318, `GGAPacked.write`)
+ *   sq_gga_load     _gga_triton.py:331 `_gga_load` (vllm_gga.py:255-267, `GGAPacked.stored`)
  * The argument convention is the reference's (_fold_triton.py:30-36): every per-sequence tensor comes as a base
  * pointer plus its per-sequence stride IN ELEMENTS of that tensor's type; batch row b works on sequence idx[b]
  * (idx == NULL: sequence b); rows with idx[b] <= 0 are padding: their output row is zeroed, nothing else is touched.
@@ -26,7 +30,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 3
+#define SQ_ABI_VERSION 4
 
 enum { SQ_F32 = 0, SQ_BF16 = 1, SQ_F16 = 2 };                /* dtype codes of float tensors */
 
@@ -170,6 +174,48 @@ typedef struct sq_read_args {
     float* out;         int64_t s_out;
 } sq_read_args;
 
+/* The mixed-width GGA / STEP slot of one layer (../integrations/vllm_gga.py:185-217 `GGAPacked`; byte layout in
+ * _gga_triton.py:3-13).  One blob per slot:
+ *   bytes 0..15     int32 n (queued pairs), head (ring index of the oldest pair), 2 unused
+ *   offs[h]         value head h at its frozen width bits[h]: 16 = fp16 [dk, dv]; 4, 6, 8 = codes [dk, dv*b/8] (u = z +
+ *                   qmax, little-endian along dv), row factors fp16 [dk], column factors fp16 [dv]; 2 = codes
+ *                   [dk, dv/4] (u = (z+3)/2), row factors fp16 [dk, dv/32], column factors fp16 [dv]
+ *   qoff + h*qsz    (pw only) head h's window: P e4m3 [m, dk], V e4m3 [m, dv], PS fp32 [m], VS fp32 [m]
+ * offs, bits [hv] int32 and w [hv, dk] fp32 (row impact factors of the fit) are device arrays of the layer's plan.
+ * blob / slot_stride: base of slot 0 and bytes per slot (both multiples of 16). */
+typedef struct sq_gga_slots {
+    void* blob;         int64_t slot_stride;
+    const int32_t* offs;
+    const int32_t* bits;
+    const float* w;
+    int32_t hv, hk, dk, dv;
+    int32_t m;          /* window length (pw), <= 8 */
+    int32_t pw;         /* 1: the FP8 write window is kept; 0: every token's write goes into the state */
+    int64_t qoff, qsz;
+} sq_gga_slots;
+
+/* One decode token per batch row on slots idx[b] (idx required; <= 0: padding).  q, k [rows, hk, dk] (normalised in
+ * the kernel, q also times `scale`), v [rows, hv, dv] with row strides in elements; out [rows, hv, dv] contiguous.
+ * gate = 1: a, b [rows, hv], A_log, dt_bias [hv] (decay exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b));
+ * gate = 0: g (log decay) and beta [rows, hv].  With pw the slots' counters are advanced by a second small launch. */
+typedef struct sq_gga_args {
+    sq_gga_slots sl;
+    int32_t rows;
+    const int32_t* idx;
+    const void* q;      int64_t s_q;     int32_t q_dtype;
+    const void* k;      int64_t s_k;     int32_t k_dtype;
+    const void* v;      int64_t s_v;     int32_t v_dtype;
+    int32_t gate;
+    const void* g;      int64_t s_g;     int32_t g_dtype;
+    const void* beta;   int64_t s_beta;  int32_t beta_dtype;
+    const void* a;      int64_t s_a;     int32_t a_dtype;
+    const void* b;      int64_t s_b;     int32_t b_dtype;
+    const void* A_log;  int32_t A_log_dtype;
+    const void* dt_bias; int32_t dt_bias_dtype;
+    void* out;          int32_t out_dtype;
+    float scale;
+} sq_gga_args;
+
 int sq_abi_version(void);
 const char* sq_strerror(int code);
 const char* sq_last_error(void);
@@ -188,6 +234,15 @@ int sq_pack_vk(const sq_pack_args* args, void* stream);
 int sq_fold_first(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m, int32_t rows, int32_t* order,
                   void* stream);
 int sq_read(const sq_read_args* args, void* stream);
+int sq_gga_step(const sq_gga_args* args, void* stream);
+/* Fit + pack canonical fp32 states X [rows, hv, dk, dv] (key-major, contiguous) into slots idx[b]; their counters are
+ * zeroed (the window starts empty).  Rows with idx[b] <= 0 are skipped. */
+int sq_gga_store(const sq_gga_slots* slots, const int32_t* idx, int32_t rows, const float* X, void* stream);
+/* The stored states of slots idx[b] (without the window) as canonical fp32 Y [rows, hv, dk, dv]; zeros for
+ * idx[b] <= 0. */
+int sq_gga_load(const sq_gga_slots* slots, const int32_t* idx, int32_t rows, float* Y, void* stream);
+/* 1 if the GGA kernels are built for these head dims and window length. Pure host code. */
+int sq_gga_supported(int32_t dk, int32_t dv, int32_t m);
 
 #ifdef __cplusplus
 }

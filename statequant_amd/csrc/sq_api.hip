@@ -338,4 +338,114 @@ int sq_fold_first(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m
     return SQ_OK;
 }
 
+namespace {
+int check_gga_slots(const sq_gga_slots& s, const char* who, sq::GgaParams* p) {
+    if (!s.blob || !s.offs || !s.bits || !s.w) return fail(SQ_E_ARG, "%s: null blob / offs / bits / w", who);
+    if (!aligned(s.blob, 16) || s.slot_stride <= 0 || (s.slot_stride % 16))
+        return fail(SQ_E_ARG, "%s: blob and slot stride must be multiples of 16 bytes", who);
+    if (s.hv <= 0 || s.hk <= 0 || s.hv % s.hk) return fail(SQ_E_ARG, "%s: hv %d, hk %d", who, s.hv, s.hk);
+    if (s.pw && (s.m < 1 || s.qoff <= 0 || (s.qoff % 16) || s.qsz < int64_t(s.m) * (s.dk + s.dv + 8) ||
+                 s.qoff + int64_t(s.hv) * s.qsz > s.slot_stride || s.qoff >= (int64_t(1) << 31) ||
+                 s.qsz >= (int64_t(1) << 31)))
+        return fail(SQ_E_ARG, "%s: window of m %d at qoff %lld, qsz %lld does not fit the slot", who, s.m,
+                    (long long)s.qoff, (long long)s.qsz);
+    p->blob = static_cast<uint8_t*>(s.blob);
+    p->slot_stride = uint64_t(s.slot_stride);
+    p->offs = s.offs;
+    p->bits = s.bits;
+    p->w = s.w;
+    p->hv = s.hv; p->hk = s.hk; p->gqa = s.hv / s.hk; p->dk = s.dk; p->dv = s.dv;
+    p->pw = s.pw != 0;
+    p->m = p->pw ? s.m : 1;
+    p->qoff = uint32_t(s.pw ? s.qoff : 0);
+    p->qsz = uint32_t(s.pw ? s.qsz : 0);
+    if (sq::dispatch_gga(*p, 0, nullptr, false) != 0)
+        return fail(SQ_E_UNSUPPORTED, "%s: no kernel built for d_k %d, d_v %d, window %d", who, s.dk, s.dv, p->m);
+    return SQ_OK;
+}
+int finish_gga(int rc, const char* who) {
+    if (rc == 0) return SQ_OK;
+    return fail(SQ_E_LAUNCH, "%s: %s", who, hipGetErrorString(hipError_t(rc)));
+}
+}  // namespace
+
+int sq_gga_supported(int32_t dk, int32_t dv, int32_t m) {
+    sq::GgaParams p{};
+    p.dk = dk; p.dv = dv; p.m = m;
+    return sq::dispatch_gga(p, 0, nullptr, false) == 0;
+}
+
+int sq_gga_step(const sq_gga_args* a, void* stream) {
+    const char* who = "sq_gga_step";
+    if (!a) return fail(SQ_E_ARG, "%s: null args", who);
+    if (a->rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, a->rows);
+    if (a->rows == 0) return SQ_OK;
+    sq::GgaParams p{};
+    SQ_TRY(check_gga_slots(a->sl, who, &p));
+    if (!a->idx || !a->q || !a->k || !a->v || !a->out) return fail(SQ_E_ARG, "%s: null idx / q / k / v / out", who);
+    if (!dtype_ok(a->q_dtype) || !dtype_ok(a->k_dtype) || !dtype_ok(a->v_dtype) || !dtype_ok(a->out_dtype))
+        return fail(SQ_E_ARG, "%s: bad dtype code", who);
+    if (a->gate) {
+        if (!a->a || !a->b || !a->A_log || !a->dt_bias)
+            return fail(SQ_E_ARG, "%s: gate without a / b / A_log / dt_bias", who);
+        if (!dtype_ok(a->a_dtype) || !dtype_ok(a->b_dtype) || !dtype_ok(a->A_log_dtype) || !dtype_ok(a->dt_bias_dtype))
+            return fail(SQ_E_ARG, "%s: bad gate dtype code", who);
+    } else {
+        if (!a->g || !a->beta) return fail(SQ_E_ARG, "%s: neither g / beta nor a gate", who);
+        if (!dtype_ok(a->g_dtype) || !dtype_ok(a->beta_dtype))
+            return fail(SQ_E_ARG, "%s: bad g / beta dtype code", who);
+    }
+    if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) ||
+        !stride_ok(a->gate ? a->s_a : a->s_g) || !stride_ok(a->gate ? a->s_b : a->s_beta))
+        return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
+    p.rows = a->rows;
+    p.idx = a->idx;
+    p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
+    p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
+    p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
+    p.gate = a->gate != 0;
+    if (p.gate) {
+        p.a = a->a; p.s_a = uint32_t(a->s_a); p.a_dt = a->a_dtype;
+        p.bt = a->b; p.s_bt = uint32_t(a->s_b); p.bt_dt = a->b_dtype;
+        p.A_log = a->A_log; p.A_log_dt = a->A_log_dtype;
+        p.dt_bias = a->dt_bias; p.dt_bias_dt = a->dt_bias_dtype;
+    } else {
+        p.a = a->g; p.s_a = uint32_t(a->s_g); p.a_dt = a->g_dtype;
+        p.bt = a->beta; p.s_bt = uint32_t(a->s_beta); p.bt_dt = a->beta_dtype;
+        p.A_log = a->g; p.A_log_dt = a->g_dtype;
+        p.dt_bias = a->g; p.dt_bias_dt = a->g_dtype;
+    }
+    p.out = a->out; p.out_dt = a->out_dtype;
+    p.scale = a->scale;
+    return finish_gga(sq::dispatch_gga(p, 0, static_cast<hipStream_t>(stream), true), who);
+}
+
+int sq_gga_store(const sq_gga_slots* s, const int32_t* idx, int32_t rows, const float* X, void* stream) {
+    const char* who = "sq_gga_store";
+    if (!s) return fail(SQ_E_ARG, "%s: null slots", who);
+    if (rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, rows);
+    if (rows == 0) return SQ_OK;
+    sq::GgaParams p{};
+    SQ_TRY(check_gga_slots(*s, who, &p));
+    if (!idx || !X || !aligned(X, 16)) return fail(SQ_E_ARG, "%s: null idx / X, or X not 16-byte aligned", who);
+    p.rows = rows;
+    p.idx = idx;
+    p.X = X;
+    return finish_gga(sq::dispatch_gga(p, 1, static_cast<hipStream_t>(stream), true), who);
+}
+
+int sq_gga_load(const sq_gga_slots* s, const int32_t* idx, int32_t rows, float* Y, void* stream) {
+    const char* who = "sq_gga_load";
+    if (!s) return fail(SQ_E_ARG, "%s: null slots", who);
+    if (rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, rows);
+    if (rows == 0) return SQ_OK;
+    sq::GgaParams p{};
+    SQ_TRY(check_gga_slots(*s, who, &p));
+    if (!idx || !Y || !aligned(Y, 16)) return fail(SQ_E_ARG, "%s: null idx / Y, or Y not 16-byte aligned", who);
+    p.rows = rows;
+    p.idx = idx;
+    p.Y = Y;
+    return finish_gga(sq::dispatch_gga(p, 2, static_cast<hipStream_t>(stream), true), who);
+}
+
 }  // extern "C"

@@ -96,6 +96,31 @@ struct ReadParams : LayoutKey {
     float* out;        uint32_t s_out;            // [rows, hv, dv, dk] fp32, row stride in elements
 };
 
+// The mixed-width GGA / STEP slot (sq_gga.cuh): one blob per slot, per-layer tables on the device.
+struct GgaParams {
+    uint8_t* blob;
+    uint64_t slot_stride;                         // bytes
+    const int32_t* idx;
+    int rows;
+    const int32_t* offs;                          // [hv] byte offset of each head in the slot
+    const int32_t* bits;                          // [hv] width of each head: 2, 4, 6, 8 or 16 (fp16 pivot)
+    const float* w;                               // [hv, dk] row impact factors of the fit
+    int hv, hk, gqa, dk, dv, m, pw;
+    uint32_t qoff, qsz;                           // windows: at qoff + h * qsz
+    const void *q, *k, *v;
+    uint32_t s_q, s_k, s_v;
+    int q_dt, k_dt, v_dt;
+    int gate;                                     // as in GdnParams
+    const void *a, *bt, *A_log, *dt_bias;
+    uint32_t s_a, s_bt;
+    int a_dt, bt_dt, A_log_dt, dt_bias_dt;
+    void* out;
+    int out_dt;
+    float scale;
+    const float* X;                               // store: canonical states [rows, hv, dk, dv]
+    float* Y;                                     // load
+};
+
 // hipError_t of the launch (0 = enqueued), or -1 if no kernel is compiled for the layout.  run = false: probe only.
 int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
 int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
@@ -104,5 +129,6 @@ int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
 int launch_fold_first(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,
                       hipStream_t stream);
 int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
+int dispatch_gga(const GgaParams& p, int op, hipStream_t stream, bool run);      // op: 0 step, 1 store, 2 load
 
 }  // namespace sq

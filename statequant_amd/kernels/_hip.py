@@ -13,14 +13,15 @@ import torch
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, 'libsqhip.so')
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 F32, BF16, F16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 FAMILY = {'gdn': 0, 'kda': 1, 'mamba2': 2}
 
 SYMBOLS = ('sq_abi_version', 'sq_strerror', 'sq_last_error', 'sq_supported', 'sq_gdn_step', 'sq_kda_step',
-           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_fold_first')
+           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_fold_first', 'sq_gga_step', 'sq_gga_store', 'sq_gga_load',
+           'sq_gga_supported')
 E_UNSUPPORTED = -2
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
@@ -85,6 +86,27 @@ class SqReadArgs(C.Structure):
                 ('out', _vp), ('s_out', _i64)]
 
 
+class SqGgaSlots(C.Structure):
+    _fields_ = [('blob', _vp), ('slot_stride', _i64), ('offs', _vp), ('bits', _vp), ('w', _vp),
+                ('hv', _i32), ('hk', _i32), ('dk', _i32), ('dv', _i32), ('m', _i32), ('pw', _i32),
+                ('qoff', _i64), ('qsz', _i64)]
+
+
+class SqGgaArgs(C.Structure):
+    _fields_ = [('sl', SqGgaSlots), ('rows', _i32), ('idx', _vp),
+                ('q', _vp), ('s_q', _i64), ('q_dtype', _i32),
+                ('k', _vp), ('s_k', _i64), ('k_dtype', _i32),
+                ('v', _vp), ('s_v', _i64), ('v_dtype', _i32),
+                ('gate', _i32),
+                ('g', _vp), ('s_g', _i64), ('g_dtype', _i32),
+                ('beta', _vp), ('s_beta', _i64), ('beta_dtype', _i32),
+                ('a', _vp), ('s_a', _i64), ('a_dtype', _i32),
+                ('b', _vp), ('s_b', _i64), ('b_dtype', _i32),
+                ('A_log', _vp), ('A_log_dtype', _i32),
+                ('dt_bias', _vp), ('dt_bias_dtype', _i32),
+                ('out', _vp), ('out_dtype', _i32), ('scale', _f32)]
+
+
 _lib = None
 
 
@@ -107,6 +129,14 @@ def lib():
             f = getattr(L, name)
             f.restype = C.c_int
             f.argtypes = [C.POINTER(T), C.c_void_p]
+        L.sq_gga_step.restype = C.c_int
+        L.sq_gga_step.argtypes = [C.POINTER(SqGgaArgs), C.c_void_p]
+        for name in ('sq_gga_store', 'sq_gga_load'):
+            f = getattr(L, name)
+            f.restype = C.c_int
+            f.argtypes = [C.POINTER(SqGgaSlots), C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
+        L.sq_gga_supported.restype = C.c_int
+        L.sq_gga_supported.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         if L.sq_abi_version() != ABI_VERSION:
             raise RuntimeError(f'{LIB_PATH}: ABI version {L.sq_abi_version()}, this package expects {ABI_VERSION}')
         _lib = L

@@ -1,0 +1,235 @@
+"""The packed GGA / STEP slot with the FP8 window on the GPU (``statequant_amd.kernels.gga.GGAPacked`` -> sq_gga_step /
+sq_gga_store / sq_gga_load) against the CPU oracle (oracle/gga.py), the way the reference checks its own kernels
+against its fp32 emulation (tests/test_gga_packed.py there): pack / unpack of every width, every decode step from
+the same stored state and window (outputs, stored state, window, counters), padding rows, graph replay.
+
+Tolerances (the reference's own, test_gga_packed.py:47-76 and test_stepquant_kernel.py:28-33 there): only the order
+of the fit's reductions differs from the oracle, which can move a row / column factor or a code across a rounding
+threshold: outputs 1e-5 relative; < 2e-3 of the stored values off by more than 1e-3 of the largest; < 1e-3 of the
+window's left factors off; right factors, counters and fp16 pivots exact.  (The reference's bound on values that
+differ at all after a fit, 1e-3, is quoted on 512 heads; on the 24 small heads here one moved row factor is more than
+that, so the fit test counts heads instead.)
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gga as G
+from statequant_amd.kernels.gga import GGAPacked, GGAPlan
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+WIDTHS = [[2, 4, 6, 8, 16, 2, 4, 6], [8, 6, 4, 2, 2, 16, 8, 4]]
+
+
+def plan(hv, d, layers=2, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return GGAPlan({i: (torch.tensor((WIDTHS[i] * 4)[:hv]), torch.rand(hv, d, generator=g) + 0.5) for i in range(layers)})
+
+
+def tokens(n, B, HV, HK, D, seed=1, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)      # noqa: E731
+    return [(r(B, HK, D).to(dtype), r(B, HK, D).to(dtype), r(B, HV, D).to(dtype), r(B, HV) * 0.5 - 2, r(B, HV))
+            for _ in range(n)]
+
+
+def dev(*ts):
+    return [t.to(DEV) for t in ts]
+
+
+@pytest.mark.parametrize('D', [128, 64])
+@pytest.mark.parametrize('layer', [0, 1])
+def test_pack_unpack_equals_fit(D, layer):
+    B, HV, HK = 3, 8, 4
+    q = plan(HV, D)
+    pk = GGAPacked(q, HV, HK, D, D, pw=True)
+    assert pk.supported()
+    Vp = pk.views(pk.alloc(6, DEV))
+    idx = torch.tensor([4, 2, 5], dtype=torch.int32)
+    g = torch.Generator().manual_seed(7)
+    S = torch.randn(B, HV, D, D, generator=g) * torch.logspace(-3, 0, D)          # canonical [B, HV, d_k, d_v]
+    S[0, 1, 5, :] = 0                                                             # a zero row, a zero column
+    S[1, 3, :, 7] = 0
+    pk.write(Vp, idx.to(DEV), S.transpose(-1, -2).to(DEV), layer=layer)
+    got = pk.stored(Vp, idx.to(DEV), layer).cpu()
+    bits, w = q.plan[layer]
+    want = G.step_fit(S, bits, w)
+    # A row factor on an fp16 rounding threshold re-codes its whole row (d of 24 d^2 values here; the same sums taken
+    # in float64 on the CPU move the same few factors), so: few heads differ at all, and those by a rounding step.
+    heads_off = sum(not torch.equal(got[bi, h], want[bi, h]) for bi in range(B) for h in range(HV))
+    assert heads_off <= 3, heads_off
+    assert (got != want).float().mean().item() < 5e-3
+    assert ((got - want).norm() / want.norm()).item() < 1e-3
+    piv = bits == 16
+    assert torch.equal(got[:, piv], S[:, piv].half().float())
+    assert torch.equal(pk.read(Vp, idx.to(DEV), layer=layer).cpu(), got.transpose(-1, -2))     # empty window
+    # the bytes: every head whose fit agrees with the oracle's must be stored exactly as the layout says
+    rf, c, z, _ = G.fit_parts(S, bits, w)
+    blob = Vp['blob'].cpu().numpy()
+    offs = pk.tables[layer][0]
+    same = 0
+    for bi, slot in enumerate(idx.tolist()):
+        assert blob[slot, :8].view(np.int32).tolist() == [0, 0]
+        for h in range(HV):
+            b = int(bits[h])
+            if b == 16:
+                raw = G.pack_head(None, None, S[bi, h], 16)
+            else:
+                r = rf[bi, h, :, ::32] if b == 2 else rf[bi, h, :, 0]
+                raw = G.pack_head(r, c[bi, h, 0], z[bi, h], b)
+            assert raw.size == G.head_bytes(b, D, D)
+            have = blob[slot, offs[h]:offs[h] + raw.size]
+            if torch.equal(got[bi, h], want[bi, h]):
+                assert np.array_equal(have, raw), (slot, h, b)
+                same += 1
+    assert same >= 0.8 * B * HV, same
+    assert not blob[[0, 1, 3]].any()                                             # other slots untouched
+
+
+@pytest.mark.parametrize('D', [128, 64])
+@pytest.mark.parametrize('pw', [False, True])
+def test_step_matches_oracle(pw, D):
+    """Every step from the same stored state and window (the packed slot's, copied into the oracle)."""
+    B, HV, HK, layer = 3, 8, 4, 0
+    q = plan(HV, D)
+    bits, w = q.plan[layer]
+    pk = GGAPacked(q, HV, HK, D, D, pw=pw)
+    Vp = pk.views(pk.alloc(6, DEV))
+    idx = torch.tensor([4, 0, 5], dtype=torch.int32)                              # row 1 is padding
+    ok = idx > 0
+    live = idx[ok].to(DEV)
+    g = torch.Generator().manual_seed(3)
+    S0 = torch.randn(B, HV, D, D, generator=g) * 0.3
+    pk.write(Vp, live, S0[ok].transpose(-1, -2).to(DEV), layer=layer)
+    A_log, dtb = torch.randn(HV, generator=g) * 0.3, torch.randn(HV, generator=g) * 0.3
+    ora = G.GGAState(bits, w, 6, HV, HK, D, D, pw=pw, m=8)
+    piv = bits == 16
+    nonp = (~piv)[None, None, :, None]
+    untouched = Vp['blob'][[0, 1, 2, 3]].clone()
+    for t, (qq, kk, vv, a, b) in enumerate(tokens(21, B, HV, HK, D)):
+        ora.O[idx[ok].long()] = pk.stored(Vp, live, layer).cpu()
+        if pw:
+            P, V, n = pk.window(Vp, live)
+            ora.P[idx[ok].long()], ora.V[idx[ok].long()], ora.n[idx[ok].long()] = P.cpu(), V.cpu(), n.cpu().long()
+        op = torch.full((B, HV, D), 7.0, device=DEV)
+        pk.step(Vp, idx.to(DEV), *dev(qq, kk, vv), op, D ** -0.5, gate=tuple(dev(a, b, A_log, dtb)), layer=layer)
+        gl, beta = ora.gate(a, b, A_log, dtb)
+        oe = ora.step(idx, qq, kk, vv, D ** -0.5, gl, beta)
+        op = op.cpu()
+        assert float(op[1].abs().max()) == 0.
+        assert ((op - oe).norm() / oe.norm()).item() < 1e-5, t
+        Sp, Se = pk.stored(Vp, live, layer).cpu(), ora.O[idx[ok].long()]
+        flips = ((Sp - Se).abs() > 1e-3 * Se.abs().amax()).float().mean().item()
+        assert flips < 2e-3, (t, flips)
+        if pw:
+            P, V, n = pk.window(Vp, live)
+            P, V, n = P.cpu(), V.cpu(), n.cpu()
+            assert torch.equal(n.long(), ora.n[idx[ok].long()]), t
+            Pe, Ve = ora.P[idx[ok].long()], ora.V[idx[ok].long()]
+            assert ((P * nonp - Pe).abs() > 1e-6 * P.abs().amax()).float().mean().item() < 1e-3, t
+            assert torch.equal(V * nonp, Ve * nonp), t
+    assert torch.equal(Vp['blob'][[0, 1, 2, 3]], untouched)                     # slot 0 (padding) and the idle slots
+
+
+def test_g_beta_inputs_and_bf16_tokens():
+    """``g=`` / ``beta=`` instead of the gate gives the same step; bf16 q / k / v and a bf16 output are taken as is."""
+    B, HV, HK, D, layer = 2, 8, 4, 128, 1
+    q = plan(HV, D)
+    pk = GGAPacked(q, HV, HK, D, D, pw=True)
+    g = torch.Generator().manual_seed(9)
+    S0 = (torch.randn(B, HV, D, D, generator=g) * 0.3).to(DEV)
+    idx = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    Va, Vb = pk.views(pk.alloc(3, DEV)), pk.views(pk.alloc(3, DEV))
+    pk.write(Va, idx, S0, layer=layer)
+    pk.write(Vb, idx, S0, layer=layer)
+    A_log, dtb = torch.randn(HV, generator=g) * 0.3, torch.randn(HV, generator=g) * 0.3
+    for qq, kk, vv, a, b in tokens(10, B, HV, HK, D, seed=4, dtype=torch.bfloat16):
+        Vb['blob'].copy_(Va['blob'])                       # every step from the same slot bytes
+        oa = torch.empty(B, HV, D, device=DEV, dtype=torch.bfloat16)
+        ob = torch.empty(B, HV, D, device=DEV, dtype=torch.bfloat16)
+        pk.step(Va, idx, *dev(qq, kk, vv), oa, D ** -0.5, gate=tuple(dev(a, b, A_log, dtb)), layer=layer)
+        gl, beta = G.GGAState.gate(a, b, A_log, dtb)
+        pk.step(Vb, idx, *dev(qq, kk, vv), ob, D ** -0.5, g=gl.to(DEV), beta=beta.to(DEV), layer=layer)
+        # exp / softplus / sigmoid on the host and in the kernel differ in the last bit: compare to float rounding
+        assert ((oa.float() - ob.float()).norm() / ob.float().norm()).item() < 1e-2
+        Sa, Sb = pk.stored(Va, idx, layer), pk.stored(Vb, idx, layer)
+        assert ((Sa - Sb).abs() > 1e-3 * Sb.abs().amax()).float().mean().item() < 2e-3
+
+
+def test_logical_state_follows_the_delta_rule():
+    """``read`` (stored + window) after every token against the textbook gated delta rule from the same logical
+    state: the step's algebra at d = 128 with all widths, within what 8-bit heads and FP8 pairs allow."""
+    B, HV, HK, D, layer = 2, 4, 2, 128, 0
+    g = torch.Generator().manual_seed(12)
+    q = GGAPlan({0: (torch.tensor([8, 8, 16, 8]), torch.ones(HV, D))})
+    pk = GGAPacked(q, HV, HK, D, D, pw=True, m=4)
+    Vp = pk.views(pk.alloc(3, DEV))
+    idx = torch.tensor([2, 1], dtype=torch.int32, device=DEV)
+    pk.write(Vp, idx, (torch.randn(B, HV, D, D, generator=g) * 0.3).to(DEV), layer=layer)
+    for t in range(9):
+        S = pk.read(Vp, idx, layer=layer).transpose(-1, -2).cpu()
+        qq, kk, vv = torch.randn(B, HK, D, generator=g), torch.randn(B, HK, D, generator=g), torch.randn(B, HV, D, generator=g)
+        gl, beta = -torch.rand(B, HV, generator=g), torch.rand(B, HV, generator=g)
+        out = torch.empty(B, HV, D, device=DEV)
+        pk.step(Vp, idx, *dev(qq, kk, vv), out, D ** -0.5, g=gl.to(DEV), beta=beta.to(DEV), layer=layer)
+        o_ref, S_ref = G.textbook_step(S, qq, kk, vv, gl, beta, D ** -0.5, HV // HK)
+        assert ((out.cpu() - o_ref).norm() / o_ref.norm()).item() < 2e-2, t           # FP8 re-encoding of the factors
+        S_new = pk.read(Vp, idx, layer=layer).transpose(-1, -2).cpu()
+        assert ((S_new - S_ref).norm() / S_ref.norm()).item() < 3e-2, t
+        assert Vp['blob'][1, :8].view(torch.int32).tolist() == [min(t + 1, 4), max(0, t + 1 - 4) % 4]
+
+
+def test_graph_replay():
+    """A captured step replayed with fresh inputs, eager work and synchronisation between the replays, leaves the
+    bytes and outputs of an eagerly stepped twin."""
+    B, HV, HK, D, layer = 3, 8, 4, 128, 0
+    q = plan(HV, D)
+    pk = GGAPacked(q, HV, HK, D, D, pw=True).prepare(DEV)
+    Vp = pk.views(pk.alloc(6, DEV))
+    idx = torch.tensor([4, 0, 5], dtype=torch.int32, device=DEV)
+    g = torch.Generator().manual_seed(2)
+    pk.write(Vp, idx[[0, 2]], (torch.randn(2, HV, D, D, generator=g) * 0.3).to(DEV), layer=layer)
+    snap = Vp['blob'].clone()
+    toks = tokens(11, B, HV, HK, D, seed=5)
+    A_log, dtb = torch.zeros(HV, device=DEV), torch.zeros(HV, device=DEV)
+    args = dev(*toks[0])
+    out = torch.empty(B, HV, D, device=DEV)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        pk.step(Vp, idx, *args[:3], out, D ** -0.5, gate=(args[3], args[4], A_log, dtb), layer=layer)
+    torch.cuda.current_stream().wait_stream(s)
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        pk.step(Vp, idx, *args[:3], out, D ** -0.5, gate=(args[3], args[4], A_log, dtb), layer=layer)
+    Vp['blob'].copy_(snap)
+    ev = pk.views(snap.clone())
+    oe = torch.empty_like(out)
+    for tk in toks:
+        for a_, b_ in zip(args, dev(*tk)):
+            a_.copy_(b_)
+        gr.replay()
+        tk = dev(*tk)
+        pk.step(ev, idx, *tk[:3], oe, D ** -0.5, gate=(tk[3], tk[4], A_log, dtb), layer=layer)
+        torch.cuda.synchronize()
+        assert torch.equal(out, oe)
+    assert torch.equal(Vp['blob'], ev['blob'])
+
+
+def test_arguments_are_checked():
+    q = plan(8, 128)
+    pk = GGAPacked(q, 8, 4, 128, 128, pw=True)
+    Vp = pk.views(pk.alloc(2, DEV))
+    idx = torch.tensor([1], dtype=torch.int32, device=DEV)
+    z = lambda *s: torch.zeros(*s, device=DEV)      # noqa: E731
+    with pytest.raises(AssertionError):
+        pk.step(Vp, idx, z(1, 4, 128), z(1, 4, 128), z(1, 8, 128), z(1, 8, 128), 1.0, layer=0)     # no gate, no g / beta
+    with pytest.raises(RuntimeError):
+        GGAPacked(q, 8, 4, 128, 128, pw=True).step({'blob': torch.zeros(2, pk.nbytes, dtype=torch.uint8)}, idx.cpu(),
+                                                     z(1, 4, 128).cpu(), z(1, 4, 128).cpu(), z(1, 8, 128).cpu(),
+                                                     z(1, 8, 128).cpu(), 1.0, g=z(1, 8).cpu(), beta=z(1, 8).cpu(), layer=0)
+    q32 = GGAPlan({0: (torch.tensor([4] * 8), torch.ones(8, 32))})
+    assert not GGAPacked(q32, 8, 4, 32, 32).supported()                                   # no kernel for d = 32
+    out = pk.step(Vp, idx[:0], z(0, 4, 128), z(0, 4, 128), z(0, 8, 128), z(0, 8, 128), 1.0, g=z(0, 8), beta=z(0, 8), layer=0)
+    assert out.shape[0] == 0

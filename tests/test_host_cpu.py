@@ -148,7 +148,7 @@ def test_library_exports_every_declared_symbol():
     L = _hip.lib()
     for name in declared:
         assert hasattr(L, name), name
-    assert L.sq_abi_version() == _hip.ABI_VERSION == 3
+    assert L.sq_abi_version() == _hip.ABI_VERSION == 4
     assert L.sq_strerror(0) == b'ok'
     lay = _hip.SqLayout(bits=8, axis_k=1, group=128, buffer_bits=8, m=8, hv=32, hk=16, dk=128, dv=128)
     assert L.sq_supported(0, ctypes.byref(lay)) == 1
