@@ -50,6 +50,8 @@ WORKLOADS = {
     'gdn-bf16': ('gdn', 16, 128, 32, 16, 128, 128, 256, 24),
     'mamba2-int8-g128': ('mamba2', 8, 128, 128, 8, 128, 64, 128, 24),
     'kda-int4-g32': ('kda', 4, 32, 32, 32, 128, 128, 256, 24),
+    # the mixed-width GGA / STEP slot: bits = the plan's mean width, group = the FP8 window length
+    'gga4-pw8': ('gga', 4, 8, 32, 16, 128, 128, 256, 24),
 }
 
 
@@ -171,6 +173,126 @@ def cpu_baseline(workload, m, budget_s=20.0):
                       f'torch CPU oracle, {cores} threads'}
 
 
+def gga_plan(hv, dk, layers, seed=0):
+    """A synthetic plan at a mean of 4 bits with one fp16 pivot per layer (charged 8 bits, as the method's allocator
+    does): 12 x 2, 11 x 4, 6 x 6, 2 x 8 bits and the pivot over the 32 heads, shuffled per layer."""
+    from statequant_amd.kernels.gga import GGAPlan
+    gen = torch.Generator().manual_seed(seed)
+    base = [2] * 12 + [4] * 11 + [6] * 6 + [8] * 2 + [16]
+    base = (base * (-(-hv // len(base))))[:hv]
+    return GGAPlan({L: (torch.tensor(base)[torch.randperm(hv, generator=gen)], torch.rand(hv, dk, generator=gen) + 0.5)
+                    for L in range(layers)})
+
+
+def gga_bytes_per_slot_step(pk, layer):
+    """Algorithmic bytes of one token on one slot of one layer: every head read and re-written at its width; per
+    non-pivot head the full window read, its left factors re-written, one new pair written."""
+    from statequant_amd.kernels.gga import head_bytes
+    widths = pk.tables[layer][1]
+    st = 2 * sum(head_bytes(b, pk.DK, pk.DV) for b in widths)
+    nonp = sum(b != 16 for b in widths)
+    win = nonp * (pk.m * (pk.DK + pk.DV + 8) + pk.m * (pk.DK + 4) + pk.DK + pk.DV + 8) if pk.pw else 0
+    return st + win
+
+
+def bench_gga(a, dev):
+    """The GGA / STEP slot step (GGAPacked.step -> sq_gga_step) at the Qwen3.5-4B GDN shape: every token re-fits and
+    re-packs every head, so the state is read and written on every step."""
+    from statequant_amd.kernels.gga import GGAPacked
+    fam, bits, m, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
+    pk = GGAPacked(gga_plan(hv, dk, layers), hv, hk, dk, dv, pw=True, m=m).prepare(dev)
+    views = [pk.views(pk.alloc(slots + 1, dev)) for _ in range(layers)]
+    gen = torch.Generator(device=dev).manual_seed(1)
+    r = lambda *s: torch.randn(*s, device=dev, generator=gen)          # noqa: E731
+    idx = (torch.randperm(slots, generator=torch.Generator().manual_seed(0)) + 1).to(torch.int32).to(dev)
+    for L in range(layers):
+        pk.write(views[L], idx, r(slots, hv, dv, dk) * 0.3, layer=L)
+    A_log, dtb = r(hv) * 0.3, r(hv) * 0.3
+    period_len = 8
+    inputs = [dict(q=r(slots, hk, dk).bfloat16(), k=r(slots, hk, dk).bfloat16(), v=r(slots, hv, dv).bfloat16(),
+                   a=r(slots, hv) * 0.5 - 2, b=r(slots, hv)) for _ in range(period_len * layers)]
+    out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
+
+    def period():
+        for s in range(period_len):
+            for L in range(layers):
+                i = inputs[s * layers + L]
+                pk.step(views[L], idx, i['q'], i['k'], i['v'], out, dk ** -0.5, gate=(i['a'], i['b'], A_log, dtb), layer=L)
+
+    use_graph = not a.no_graph and a.steps % period_len == 0 and a.warmup % period_len == 0 and a.steps > 0
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        period()
+        stream.synchronize()
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                period()
+            run = lambda n: [graph.replay() for _ in range(n // period_len)]          # noqa: E731
+        else:
+            run = lambda n: [period() for _ in range(-(-n // period_len))]            # noqa: E731
+        run(max(a.warmup - period_len, 0))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        run(a.steps)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    steps = a.steps if use_graph else -(-a.steps // period_len) * period_len
+    assert torch.isfinite(out.float()).all(), 'non-finite output'
+    n_launch = steps * layers
+    us_wall, us_kernel = wall * 1e6 / n_launch, e0.elapsed_time(e1) * 1e3 / n_launch
+    alg = sum(gga_bytes_per_slot_step(pk, L) for L in range(layers)) / layers * slots
+    achieved = alg / (us_kernel * 1e-6) / 1e9
+    res = {
+        'metric': 'us_per_layer_decode_step', 'value': round(us_wall, 3), 'unit': 'us',
+        'n_gpus': 1, 'steps': steps, 'warmup': a.warmup, 'ms_per_step': round(wall * 1e3 / steps, 5),
+        'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': a.workload, 'family': 'gdn (GGA / STEP slot)', 'slots': slots, 'layers': layers,
+                   'value_heads': hv, 'key_heads': hk, 'd_k': dk, 'd_v': dv,
+                   'state': f'per-head widths 2/4/6/8 bit + one fp16 pivot per layer, {pk.bits_per_value():.3f} bits '
+                            f'per value with the window', 'window': f'FP8 pairs, m={m}', 'inputs': 'bf16',
+                   'launch': 'hip-graph' if use_graph else 'eager', 'bytes_per_slot': pk.nbytes,
+                   'algorithmic_bytes_per_slot_step': round(alg / slots)},
+        'hbm_gbs': round(achieved, 1),
+        'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(a.workload),
+                     'kernel_us': round(us_kernel, 3), 'algorithmic_bytes_per_launch': round(alg)},
+    }
+    if not a.no_cpu_baseline:
+        res['cpu_baseline'] = cpu_baseline_gga(a.workload, a.cpu_budget)
+    print(json.dumps(res))
+
+
+def cpu_baseline_gga(workload, budget_s=20.0):
+    """The CPU oracle of the GGA slot step on a bounded sample: one layer, 32 slots."""
+    from oracle import gga as G
+    fam, bits, m, hv, hk, dk, dv, slots, layers = WORKLOADS[workload]
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    n = min(slots, 32)
+    plan = gga_plan(hv, dk, 1)
+    b, w = plan.plan[0]
+    gen = torch.Generator().manual_seed(0)
+    r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
+    st = G.GGAState(b, w, n + 1, hv, hk, dk, dv, pw=True, m=m)
+    idx = torch.arange(1, n + 1, dtype=torch.int32)
+    st.write(idx, r(n, hv, dk, dv) * 0.3)
+    steps, t_total = 0, 0.0
+    while t_total < budget_s and steps < 16:
+        args = (r(n, hk, dk).bfloat16(), r(n, hk, dk).bfloat16(), r(n, hv, dv).bfloat16(), dk ** -0.5,
+                -torch.nn.functional.softplus(r(n, hv)), torch.sigmoid(r(n, hv)))
+        t0 = time.perf_counter()
+        st.step(idx, *args)
+        t_total += time.perf_counter() - t0
+        steps += 1
+    return {'value': round(t_total / steps * 1e6 * slots / n, 1), 'unit': 'us per layer-step', 'cores': cores,
+            'kind': 'port', 'sample': f'{workload}: 1 layer x {n} of {slots} slots (time scaled by {slots // n}), '
+                                      f'{steps} steps, torch CPU oracle, {cores} threads'}
+
+
 def calibrate_copy(dev, nbytes=1 << 30, reps=20):
     """`reps` plain copies of `nbytes` (reads nbytes, writes nbytes each): the reference point for the HBM counters."""
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -272,6 +394,8 @@ def main():
         w = WORKLOADS[a.workload]
         WORKLOADS[a.workload] = w[:7] + (a.slots,) + w[8:]
     fam, bits, group, hv, hk, dk, dv, slots, layers = WORKLOADS[a.workload]
+    if fam == 'gga':
+        return bench_gga(a, dev)
     fam, lay, views, idx = build(a.workload, m, dev)
     if a.op != 'step':
         return bench_convert(a, lay, views, idx, dev)

@@ -58,6 +58,24 @@ __host__ __device__ constexpr int gga_code_bytes(int b, int dk, int dv) { return
 // fp16 with the fit's clamp: [2^-24, 65504], round to nearest even.
 __device__ __forceinline__ float gga_half(float x) { return float(_Float16(fminf(fmaxf(x, FP16_TINY), 65504.0f))); }
 
+// x / d with the divisor's reciprocal rc = RN(1 / d) computed once per row or column: q = RN(x rc), the exact
+// remainder r = x - q d (one fma), q + r rc rounded once.  With a correctly rounded reciprocal this is the correctly
+// rounded quotient (Markstein's division; the exception, a divisor whose significand is all ones, cannot occur: the
+// divisors here are fp16 values or 3, 7, 31, 127), so the codes are those of an IEEE division at a third of its
+// instructions.
+__device__ __forceinline__ float gga_div(float x, float d, float rc) {
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, d, x);
+    return __builtin_fmaf(r, rc, q);
+}
+// RN(1 / d) for a divisor that is an fp16 value: the hardware estimate (1 ulp) and one Newton step with the exact
+// residual.  The step leaves a relative error of 2^-46 before its single rounding, and the reciprocal of an 11-bit
+// significand is never closer than 2^-12 ulp to a rounding boundary, so the result is the correctly rounded one.
+__device__ __forceinline__ float gga_rcp_f16(float d) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // sums / maxima along d_k: every thread ends with the totals of its CT columns (the same value in all row groups)
 // ---------------------------------------------------------------------------------------------------------------
@@ -229,18 +247,21 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
             for (int e = 0; e < CT; ++e) a = a + fabsf(x[s][e]);
             a = block_sum<RN>(a) * (1.0f / float(RN * CT));
             rf[s] = gga_half(sqrtf(fmaxf(a, 1e-20f) / wrow[s]));
+            const float rrc = gga_rcp_f16(rf[s]);
 #pragma unroll
             for (int e = 0; e < CT; ++e) {
-                y0[s][e] = x[s][e] / rf[s];
+                y0[s][e] = gga_div(x[s][e], rf[s], rrc);
                 cmax[0][e] = fmaxf(cmax[0][e], fabsf(y0[s][e]));
             }
         }
         gga_col_allreduce<T, 1, true>(cmax, red, t);
-        float c[CT];
+        float c[CT], crc[CT];
         float nd[2][CT];
 #pragma unroll
         for (int e = 0; e < CT; ++e) {
-            c[e] = gga_half(cmax[0][e] / QMAX);           // max_i (|y| / qmax) = (max_i |y|) / qmax: division is monotonic
+            // max_i (|y| / qmax) = (max_i |y|) / qmax: division is monotonic
+            c[e] = gga_half(gga_div(cmax[0][e], QMAX, 1.0f / QMAX));
+            crc[e] = gga_rcp_f16(c[e]);
             nd[0][e] = nd[1][e] = 0.0f;
         }
 #pragma unroll
@@ -248,22 +269,24 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
             const float ww = wrow[s] * wrow[s];
 #pragma unroll
             for (int e = 0; e < CT; ++e) {
-                const float vv = rf[s] * gga_encode<B>(y0[s][e] / c[e]);
-                nd[0][e] = nd[0][e] + (ww * vv) * x[s][e];
-                nd[1][e] = nd[1][e] + ww * (vv * vv);
+                const float vv = rf[s] * gga_encode<B>(gga_div(y0[s][e], c[e], crc[e]));
+                nd[0][e] = __builtin_fmaf(ww * vv, x[s][e], nd[0][e]);
+                nd[1][e] = __builtin_fmaf(ww, vv * vv, nd[1][e]);
             }
         }
         gga_col_allreduce<T, 2, false>(nd, red, t);
 #pragma unroll
-        for (int e = 0; e < CT; ++e)
+        for (int e = 0; e < CT; ++e) {
             c[e] = gga_half(nd[1][e] > 0.0f ? nd[0][e] / fmaxf(nd[1][e], 1e-30f) : c[e]);
+            crc[e] = gga_rcp_f16(c[e]);
+        }
 #pragma unroll
         for (int s = 0; s < RPT; ++s) {
             const int i = s * 16 + t.tr;
             uint64_t bits = 0;
 #pragma unroll
             for (int e = 0; e < CT; ++e) {
-                const float z = gga_encode<B>(y0[s][e] / c[e]);
+                const float z = gga_encode<B>(gga_div(y0[s][e], c[e], crc[e]));
                 const int u = B == 2 ? (int(z) + 3) >> 1 : int(z) + gga_qmax(B);
                 bits |= uint64_t(uint32_t(u)) << (e * B);
             }
@@ -504,7 +527,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
 #pragma unroll
     for (int s = 0; s < RPT; ++s)
 #pragma unroll
-        for (int e = 0; e < CT; ++e) acc[0][e] = acc[0][e] + krow[s] * x[s][e];
+        for (int e = 0; e < CT; ++e) acc[0][e] = __builtin_fmaf(krow[s], x[s][e], acc[0][e]);
     gga_col_allreduce<T, 1, false>(acc, L.red, t);
     float kO[CT];
 #pragma unroll
@@ -517,8 +540,8 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
         const float bk = beta * krow[s];
 #pragma unroll
         for (int e = 0; e < CT; ++e) {
-            x[s][e] = a * (x[s][e] - bk * kO[e]);
-            acc[0][e] = acc[0][e] + x[s][e] * qrow[s];
+            x[s][e] = a * __builtin_fmaf(-bk, kO[e], x[s][e]);
+            acc[0][e] = __builtin_fmaf(x[s][e], qrow[s], acc[0][e]);
         }
     }
     gga_col_allreduce<T, 1, false>(acc, L.red, t);
@@ -543,14 +566,14 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
             }
         }
         if (full) {
+            float v0[CT];
+#pragma unroll
+            for (int e = 0; e < CT; ++e) v0[e] = fp8_to_f32((vq[0][e / 4] >> (8 * (e % 4))) & 0xFFu) * vs[0];
 #pragma unroll
             for (int s = 0; s < RPT; ++s) {
                 const float r0 = L.r0[s * 16 + t.tr];
 #pragma unroll
-                for (int e = 0; e < CT; ++e) {
-                    const float v0 = fp8_to_f32((vq[0][e / 4] >> (8 * (e % 4))) & 0xFFu) * vs[0];
-                    x[s][e] = x[s][e] + r0 * v0;
-                }
+                for (int e = 0; e < CT; ++e) x[s][e] = __builtin_fmaf(r0, v0[e], x[s][e]);
             }
         }
     } else {
@@ -559,7 +582,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
         for (int s = 0; s < RPT; ++s) {
             const float bk = beta * krow[s];
 #pragma unroll
-            for (int e = 0; e < CT; ++e) x[s][e] = x[s][e] + bk * ve[e];
+            for (int e = 0; e < CT; ++e) x[s][e] = __builtin_fmaf(bk, ve[e], x[s][e]);
         }
     }
     if (t.tr == 0) {
