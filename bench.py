@@ -20,7 +20,8 @@ algorithmic bytes are (codes + scales) x (1 + 1/m) per slot (read every step, re
 ``cpu_baseline`` times the CPU oracle (a torch restatement of the reference's own CPU path) on this box's host cores
 on a bounded sample of the same workload; it is a reported baseline, not a target.
 
-Secondary figures: ``--workload`` (the other formats and families), ``--slots N`` (other batch sizes), ``--op write |
+Secondary figures: ``--workload`` (the other formats and families; ``gga4-pw8`` is the mixed-width GGA / STEP slot,
+which re-fits every head at every token), ``--slots N`` (other batch sizes), ``--op write |
 read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots)
 with or without ``--fold-first`` (the step calls' optional dispatch order, folding rows first), ``--calibrate-copy``
 (the known-size copy that the HBM counters are scaled by).
@@ -67,7 +68,7 @@ def describe_state(bits, group):
 
 # HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
 # over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
-MEASURED_TRAFFIC = {'gdn-int8-g128': 185331247}
+MEASURED_TRAFFIC = {'gdn-int8-g128': 185331247, 'gga4-pw8': 187902771}
 
 
 def stored_bytes_per_slot(bits, group, hv, dk, dv):

@@ -10,11 +10,14 @@ packed decode path (the classes its tests use as the yardstick for its Triton ke
                                                           (ReferenceMamba2State), kda.py:44-52, mamba2.py:45-70
     slots.py     per-slot byte layout, read, write    <- slots.py:76-95, 210-252; kda.py:311-323, 351-386;
                                                           mamba2.py:359-370
+    gga.py       mixed-width GGA / STEP slot, FP8     <- /root/reference/src/statequant/step_quant.py:35-96,
+                 window, its byte layout                 methods_ext/gga.py:225-233, integrations/vllm_gga.py:86-217,
+                                                          kernels/_gga_triton.py:3-13, 40-95
 
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import it, and only as
 the checker; nothing under ``statequant_amd/`` does.  It runs wherever torch runs (no GPU, no HIP library).
 
-How it is pinned (see tests/test_oracle_*.py):
+How it is pinned (see tests/test_oracle_*.py; gga.py states its own pins in its header):
   * bit-for-bit against golden vectors produced by the reference's own classes on seeded inputs
     (tests/golden/*.pt, written by tests/golden/make_golden.py) -- every function below is covered by them;
   * independently of those: pack/unpack against a per-group brute force in NumPy with np.float16 and against the

@@ -203,3 +203,37 @@ def test_bench_contract_off_the_gpu():
         fam, bits, group, hv, hk, dk, dv, slots, layers = bench.WORKLOADS[name]
         assert bench.state_bytes_per_slot(bits, group, hv, dk, dv, 8) == want, name
     assert bench.state_bytes_per_slot(8, 128, 32, 128, 128, 8) * 256 == 153354240
+
+
+def test_gga_packed_tables_match_the_reference(golden):
+    """``GGAPacked``: per-layer offset tables, window placement, slot size and bits per value as the reference's class
+    computes them for the plan of its own tests (recorded in tests/golden/gga.pt); no GPU, no library call."""
+    from statequant_amd.kernels.gga import GGAPacked, GGAPlan, head_bytes
+    t = golden('gga.pt')['tables']
+    hv, dk, dv, m = t['hv'], t['dk'], t['dv'], t['m']
+    plan = GGAPlan({i: (torch.tensor(wd), torch.ones(hv, dk)) for i, wd in enumerate(t['widths'])})
+    for pw in (False, True):
+        pk = GGAPacked(plan, hv, 4, dk, dv, pw=pw, m=m)
+        ref = t[pw]
+        assert [pk.tables[i][0] for i in range(2)] == ref['offs']
+        assert [pk.bytes_per_layer[i] for i in range(2)] == ref['bytes_per_layer']
+        assert (pk.QOFF, pk.QSZ, pk.nbytes) == (ref['QOFF'], ref['QSZ'], ref['nbytes'])
+        assert abs(pk.bits_per_value() - ref['bits_per_value']) < 1e-12
+        blob = torch.zeros(3, pk.nbytes + 16, dtype=torch.uint8)
+        assert pk.views(blob)['blob'] is blob
+    assert [head_bytes(b, 128, 128) for b in (2, 4, 6, 8, 16)] == [5376, 8704, 12800, 16896, 32768]
+    with pytest.raises(AssertionError):
+        GGAPacked(GGAPlan({0: (torch.tensor([3] * hv), torch.ones(hv, dk))}), hv, 4, dk, dv)     # no 3-bit heads
+    with pytest.raises(RuntimeError, match='GPU only'):
+        pk.stored(pk.views(blob), torch.tensor([1]), 0)                                          # CPU blob: loud
+
+
+def test_gga_bench_byte_model():
+    import sys
+    sys.path.insert(0, ROOT)
+    import bench
+    from statequant_amd.kernels.gga import GGAPacked
+    pk = GGAPacked(bench.gga_plan(32, 128, 2), 32, 16, 128, 128, pw=True, m=8)
+    state = 12 * 5376 + 11 * 8704 + 6 * 12800 + 2 * 16896 + 32768
+    window = 31 * (8 * (128 + 128 + 8) + 8 * (128 + 4) + 128 + 128 + 8)
+    assert bench.gga_bytes_per_slot_step(pk, 0) == 2 * state + window == 713624
