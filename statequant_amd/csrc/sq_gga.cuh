@@ -16,7 +16,7 @@
 //
 // A workgroup of four wavefronts holds the head's [d_k, d_v] tile in registers: thread (tr, tc) owns the columns
 // tc CT .. tc CT + CT - 1 (CT = d_v / 16) of the rows s 16 + tr.  The 16 threads of a row sit in one DPP row, so sums
-// along d_v are four DPP adds; sums along d_k go through two lane exchanges and one pass through LDS.
+// along d_v are four DPP adds; sums along d_k go through two lane swaps and one pass through LDS.
 #pragma once
 #include "sq_device.cuh"
 #include "sq_params.h"
@@ -79,19 +79,31 @@ __device__ __forceinline__ float gga_rcp_f16(float d) {
 // ---------------------------------------------------------------------------------------------------------------
 // sums / maxima along d_k: every thread ends with the totals of its CT columns (the same value in all row groups)
 // ---------------------------------------------------------------------------------------------------------------
-template <class T, int K, bool MAX>
+// The partner's value across 16 / 32 lanes and the lane's own, as one VALU swap each (v_permlane16_swap exchanges the
+// odd 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the
+// first with the lower half of the second; fed the same register twice they leave both values of a pair in both of
+// its lanes, in the same order, so the combined value is bit-identical across the pair).
+template <bool MAX>
+__device__ __forceinline__ float gga_pair16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(as_u32(v), as_u32(v), false, false);
+    return MAX ? fmaxf(as_f32(r[0]), as_f32(r[1])) : as_f32(r[0]) + as_f32(r[1]);
+}
+template <bool MAX>
+__device__ __forceinline__ float gga_pair32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(as_u32(v), as_u32(v), false, false);
+    return MAX ? fmaxf(as_f32(r[0]), as_f32(r[1])) : as_f32(r[0]) + as_f32(r[1]);
+}
+
+// `red` holds two buffers of 2 x GGA_WAVES x DV floats; consecutive reductions alternate between them (BUF), so one
+// barrier per reduction is enough: the barrier of reduction i + 1 separates the reads of reduction i from the writes
+// of reduction i + 2 into the same buffer.
+template <class T, int K, bool MAX, int BUF>
 __device__ __forceinline__ void gga_col_allreduce(float (&p)[K][T::CT], float* red, const GgaThread& t) {
+    red += BUF * (2 * GGA_WAVES * T::DV);
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
-        for (int e = 0; e < T::CT; ++e) {
-            float v = p[k][e];
-            float o = __shfl_xor(v, 16);
-            v = MAX ? fmaxf(v, o) : v + o;
-            o = __shfl_xor(v, 32);
-            p[k][e] = MAX ? fmaxf(v, o) : v + o;
-        }
-    __syncthreads();                                   // the previous reduction has been read
+        for (int e = 0; e < T::CT; ++e) p[k][e] = gga_pair32<MAX>(gga_pair16<MAX>(p[k][e]));
     if (t.lane < 16) {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -254,7 +266,7 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
                 cmax[0][e] = fmaxf(cmax[0][e], fabsf(y0[s][e]));
             }
         }
-        gga_col_allreduce<T, 1, true>(cmax, red, t);
+        gga_col_allreduce<T, 1, true, 0>(cmax, red, t);
         float c[CT], crc[CT];
         float nd[2][CT];
 #pragma unroll
@@ -274,7 +286,7 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
                 nd[1][e] = __builtin_fmaf(ww, vv * vv, nd[1][e]);
             }
         }
-        gga_col_allreduce<T, 2, false>(nd, red, t);
+        gga_col_allreduce<T, 2, false, 1>(nd, red, t);
 #pragma unroll
         for (int e = 0; e < CT; ++e) {
             c[e] = gga_half(nd[1][e] > 0.0f ? nd[0][e] / fmaxf(nd[1][e], 1e-30f) : c[e]);
@@ -368,7 +380,7 @@ template <class T>
 struct GgaLds {
     float kn[T::DK], qn[T::DK], r0[T::DK];
     float coef[GGA_MMAX];
-    float red[2 * GGA_WAVES * T::DV];
+    float red[2 * 2 * GGA_WAVES * T::DV];        // two buffers, see gga_col_allreduce
 };
 
 template <class T>
@@ -376,8 +388,10 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
     constexpr int CT = T::CT, RPT = T::RPT, DK = T::DK, DV = T::DV, NE = T::NE, NV = T::NV;
     __shared__ GgaLds<T> L;
     const GgaThread t = gga_thread();
-    const uint32_t bh = blockIdx.x;
-    const uint32_t b = bh / uint32_t(p.hv), h = bh - b * uint32_t(p.hv);
+    // head-major order: workgroups that run together work on the same head, hence on the same width, and share the
+    // instructions of one of the five width paths (each path is ~40 KB of straight-line code)
+    const uint32_t h = blockIdx.x / uint32_t(p.rows), b = blockIdx.x - h * uint32_t(p.rows);
+    const uint32_t bh = b * uint32_t(p.hv) + h;
     const uint32_t hk = h / uint32_t(p.gqa);
     void* const outp = advance(p.out, p.out_dt, uint64_t(bh) * DV);
     const int32_t seq = p.idx[b];
@@ -528,7 +542,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
     for (int s = 0; s < RPT; ++s)
 #pragma unroll
         for (int e = 0; e < CT; ++e) acc[0][e] = __builtin_fmaf(krow[s], x[s][e], acc[0][e]);
-    gga_col_allreduce<T, 1, false>(acc, L.red, t);
+    gga_col_allreduce<T, 1, false, 0>(acc, L.red, t);
     float kO[CT];
 #pragma unroll
     for (int e = 0; e < CT; ++e) {
@@ -544,7 +558,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
             acc[0][e] = __builtin_fmaf(x[s][e], qrow[s], acc[0][e]);
         }
     }
-    gga_col_allreduce<T, 1, false>(acc, L.red, t);
+    gga_col_allreduce<T, 1, false, 1>(acc, L.red, t);
     float ve[CT], o[CT];
 #pragma unroll
     for (int e = 0; e < CT; ++e) {
@@ -632,10 +646,12 @@ __global__ void gga_advance_kernel(uint8_t* blob, uint64_t slot_stride, const in
 template <class T>
 __global__ __launch_bounds__(GGA_THREADS, 2) void gga_store_kernel(const GgaParams p) {
     constexpr int CT = T::CT, RPT = T::RPT, DK = T::DK, DV = T::DV;
-    __shared__ float red[2 * GGA_WAVES * DV];
+    __shared__ float red[2 * 2 * GGA_WAVES * DV];
     const GgaThread t = gga_thread();
-    const uint32_t bh = blockIdx.x;
-    const uint32_t b = bh / uint32_t(p.hv), h = bh - b * uint32_t(p.hv);
+    // head-major order: workgroups that run together work on the same head, hence on the same width, and share the
+    // instructions of one of the five width paths (each path is ~40 KB of straight-line code)
+    const uint32_t h = blockIdx.x / uint32_t(p.rows), b = blockIdx.x - h * uint32_t(p.rows);
+    const uint32_t bh = b * uint32_t(p.hv) + h;
     const int32_t seq = p.idx[b];
     if (seq <= 0) return;
     uint8_t* const base = p.blob + uint64_t(seq) * p.slot_stride;
@@ -660,8 +676,10 @@ template <class T>
 __global__ __launch_bounds__(GGA_THREADS, 2) void gga_load_kernel(const GgaParams p) {
     constexpr int CT = T::CT, RPT = T::RPT, DK = T::DK, DV = T::DV;
     const GgaThread t = gga_thread();
-    const uint32_t bh = blockIdx.x;
-    const uint32_t b = bh / uint32_t(p.hv), h = bh - b * uint32_t(p.hv);
+    // head-major order: workgroups that run together work on the same head, hence on the same width, and share the
+    // instructions of one of the five width paths (each path is ~40 KB of straight-line code)
+    const uint32_t h = blockIdx.x / uint32_t(p.rows), b = blockIdx.x - h * uint32_t(p.rows);
+    const uint32_t bh = b * uint32_t(p.hv) + h;
     const int32_t seq = p.idx[b];
     float* Y = p.Y + uint64_t(bh) * (DK * DV);
     float x[RPT][CT];
