@@ -94,6 +94,13 @@ __device__ __forceinline__ float gga_pair32(float v) {
     return MAX ? fmaxf(as_f32(r[0]), as_f32(r[1])) : as_f32(r[0]) + as_f32(r[1]);
 }
 
+// Position of column tc CT + e of wavefront w's partial k: the 16 threads of a row access 16 consecutive groups of
+// four floats (one 128-bit access each, 256 contiguous bytes per instruction: no bank conflicts).
+template <class T>
+__device__ __forceinline__ int gga_red_pos(int k, int w, int tc, int e) {
+    return ((k * GGA_WAVES + w) * (T::CT / 4) + e / 4) * 64 + tc * 4 + e % 4;
+}
+
 // `red` holds two buffers of 2 x GGA_WAVES x DV floats; consecutive reductions alternate between them (BUF), so one
 // barrier per reduction is enough: the barrier of reduction i + 1 separates the reads of reduction i from the writes
 // of reduction i + 2 into the same buffer.
@@ -108,15 +115,15 @@ __device__ __forceinline__ void gga_col_allreduce(float (&p)[K][T::CT], float* r
 #pragma unroll
         for (int k = 0; k < K; ++k)
 #pragma unroll
-            for (int e = 0; e < T::CT; ++e) red[(k * GGA_WAVES + t.wave) * T::DV + t.tc * T::CT + e] = p[k][e];
+            for (int e = 0; e < T::CT; ++e) red[gga_red_pos<T>(k, t.wave, t.tc, e)] = p[k][e];
     }
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
         for (int e = 0; e < T::CT; ++e) {
-            const float* r = red + k * GGA_WAVES * T::DV + t.tc * T::CT + e;
-            const float a0 = r[0], a1 = r[T::DV], a2 = r[2 * T::DV], a3 = r[3 * T::DV];
+            const float a0 = red[gga_red_pos<T>(k, 0, t.tc, e)], a1 = red[gga_red_pos<T>(k, 1, t.tc, e)];
+            const float a2 = red[gga_red_pos<T>(k, 2, t.tc, e)], a3 = red[gga_red_pos<T>(k, 3, t.tc, e)];
             p[k][e] = MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (a0 + a1) + (a2 + a3);
         }
 }
