@@ -14,9 +14,11 @@
 //   the state is re-fitted at its width and re-packed in place; (R(beta k), R(v)) is queued.  Pivots (b = 16) and
 //   slots without a window take the new write into the state: O = Q(O_pre + beta k v^T).
 //
-// A workgroup of four wavefronts holds the head's [d_k, d_v] tile in registers: thread (tr, tc) owns the columns
-// tc CT .. tc CT + CT - 1 (CT = d_v / 16) of the rows s 16 + tr.  The 16 threads of a row sit in one DPP row, so sums
-// along d_v are four DPP adds; sums along d_k go through two lane swaps and one pass through LDS.
+// A workgroup of four wavefronts holds the head's [d_k, d_v] tile in registers.  Wavefront w owns a quarter of the
+// columns and all rows: lane (tr, q) = (lane / 4, lane % 4) owns the columns tc CT .. tc CT + CT - 1 (tc = 4 w + q,
+// CT = d_v / 16) of the rows s 16 + tr.  Sums along d_k -- the step and the fit take six of them per column -- stay
+// inside a wavefront (two DPP row rotations and two lane swaps, no LDS, no barrier); the one sum along d_v (the row
+// factors of the fit) is a quad reduction plus one exchange of per-wavefront partials through LDS.
 #pragma once
 #include "sq_device.cuh"
 #include "sq_params.h"
@@ -47,8 +49,8 @@ __device__ __forceinline__ GgaThread gga_thread() {
     t.tid = threadIdx.x;
     t.lane = t.tid & (WAVE - 1);
     t.wave = t.tid >> 6;
-    t.tc = t.tid & 15;
-    t.tr = t.tid >> 4;
+    t.tc = t.wave * 4 + (t.lane & 3);
+    t.tr = t.lane >> 2;
     return t;
 }
 
@@ -94,37 +96,20 @@ __device__ __forceinline__ float gga_pair32(float v) {
     return MAX ? fmaxf(as_f32(r[0]), as_f32(r[1])) : as_f32(r[0]) + as_f32(r[1]);
 }
 
-// Position of column tc CT + e of wavefront w's partial k: the 16 threads of a row access 16 consecutive groups of
-// four floats (one 128-bit access each, 256 contiguous bytes per instruction: no bank conflicts).
-template <class T>
-__device__ __forceinline__ int gga_red_pos(int k, int w, int tc, int e) {
-    return ((k * GGA_WAVES + w) * (T::CT / 4) + e / 4) * 64 + tc * 4 + e % 4;
-}
+constexpr int DPP_ROR4 = 0x124, DPP_ROR8 = 0x128;      // row_ror: lane i of a 16-lane row reads lane (i + n) % 16
 
-// `red` holds two buffers of 2 x GGA_WAVES x DV floats; consecutive reductions alternate between them (BUF), so one
-// barrier per reduction is enough: the barrier of reduction i + 1 separates the reads of reduction i from the writes
-// of reduction i + 2 into the same buffer.
-template <class T, int K, bool MAX, int BUF>
-__device__ __forceinline__ void gga_col_allreduce(float (&p)[K][T::CT], float* red, const GgaThread& t) {
-    red += BUF * (2 * GGA_WAVES * T::DV);
-#pragma unroll
-    for (int k = 0; k < K; ++k)
-#pragma unroll
-        for (int e = 0; e < T::CT; ++e) p[k][e] = gga_pair32<MAX>(gga_pair16<MAX>(p[k][e]));
-    if (t.lane < 16) {
-#pragma unroll
-        for (int k = 0; k < K; ++k)
-#pragma unroll
-            for (int e = 0; e < T::CT; ++e) red[gga_red_pos<T>(k, t.wave, t.tc, e)] = p[k][e];
-    }
-    __syncthreads();
+// Sum / maximum over the 16 row groups of a wavefront (lanes with the same lane % 4): every lane ends with the total
+// of its CT columns, bit-identical across the lanes of a column (each step combines a pair symmetrically).
+template <class T, int K, bool MAX>
+__device__ __forceinline__ void gga_col_allreduce(float (&p)[K][T::CT]) {
 #pragma unroll
     for (int k = 0; k < K; ++k)
 #pragma unroll
         for (int e = 0; e < T::CT; ++e) {
-            const float a0 = red[gga_red_pos<T>(k, 0, t.tc, e)], a1 = red[gga_red_pos<T>(k, 1, t.tc, e)];
-            const float a2 = red[gga_red_pos<T>(k, 2, t.tc, e)], a3 = red[gga_red_pos<T>(k, 3, t.tc, e)];
-            p[k][e] = MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (a0 + a1) + (a2 + a3);
+            float v = p[k][e];
+            v = MAX ? fmaxf(v, dpp<DPP_ROR8>(v)) : v + dpp<DPP_ROR8>(v);
+            v = MAX ? fmaxf(v, dpp<DPP_ROR4>(v)) : v + dpp<DPP_ROR4>(v);
+            p[k][e] = gga_pair32<MAX>(gga_pair16<MAX>(v));
         }
 }
 
@@ -254,7 +239,7 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
         constexpr int RN = B == 2 ? GGA_GROUP / CT : 16;                    // threads sharing one row factor
         uint16_t* R = reinterpret_cast<uint16_t*>(S + gga_code_bytes(B, DK, DV));
         uint16_t* C = R + (B == 2 ? DK * T::NG : DK);
-        float rf[RPT];
+        float rf[RPT], asum[RPT];
         float y0[RPT][CT];
         float cmax[1][CT];
 #pragma unroll
@@ -264,7 +249,25 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
             float a = 0.0f;
 #pragma unroll
             for (int e = 0; e < CT; ++e) a = a + fabsf(x[s][e]);
-            a = block_sum<RN>(a) * (1.0f / float(RN * CT));
+            asum[s] = block_sum<4>(a);                      // over the wavefront's 4 CT columns
+        }
+        constexpr bool OWN = B == 2 && 4 * CT >= GGA_GROUP;       // a two-bit group lies inside one wavefront's columns
+        if constexpr (!OWN) {
+            if ((t.lane & 3) == 0) {
+#pragma unroll
+                for (int s = 0; s < RPT; ++s) red[(s * 16 + t.tr) * GGA_WAVES + t.wave] = asum[s];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < RPT; ++s) {
+                const float4 w4 = *reinterpret_cast<const float4*>(red + (s * 16 + t.tr) * GGA_WAVES);
+                if constexpr (B == 2) asum[s] = t.wave < 2 ? w4.x + w4.y : w4.z + w4.w;     // d_v = 64: two wavefronts
+                else asum[s] = (w4.x + w4.y) + (w4.z + w4.w);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < RPT; ++s) {
+            const float a = asum[s] * (1.0f / float(RN * CT));
             rf[s] = gga_half(sqrtf(fmaxf(a, 1e-20f) / wrow[s]));
             const float rrc = gga_rcp_f16(rf[s]);
 #pragma unroll
@@ -273,7 +276,7 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
                 cmax[0][e] = fmaxf(cmax[0][e], fabsf(y0[s][e]));
             }
         }
-        gga_col_allreduce<T, 1, true, 0>(cmax, red, t);
+        gga_col_allreduce<T, 1, true>(cmax);
         float c[CT], crc[CT];
         float nd[2][CT];
 #pragma unroll
@@ -293,7 +296,7 @@ __device__ __forceinline__ void gga_fit_store(uint8_t* S, float (&x)[T::RPT][T::
                 nd[1][e] = __builtin_fmaf(ww, vv * vv, nd[1][e]);
             }
         }
-        gga_col_allreduce<T, 2, false, 1>(nd, red, t);
+        gga_col_allreduce<T, 2, false>(nd);
 #pragma unroll
         for (int e = 0; e < CT; ++e) {
             c[e] = gga_half(nd[1][e] > 0.0f ? nd[0][e] / fmaxf(nd[1][e], 1e-30f) : c[e]);
@@ -387,13 +390,13 @@ template <class T>
 struct GgaLds {
     float kn[T::DK], qn[T::DK], r0[T::DK];
     float coef[GGA_MMAX];
-    float red[2 * 2 * GGA_WAVES * T::DV];        // two buffers, see gga_col_allreduce
+    float red[GGA_WAVES * T::DK];                 // the fit's row sums: one partial per wavefront and row
 };
 
 template <class T>
 __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParams p) {
     constexpr int CT = T::CT, RPT = T::RPT, DK = T::DK, DV = T::DV, NE = T::NE, NV = T::NV;
-    __shared__ GgaLds<T> L;
+    __shared__ __attribute__((aligned(16))) GgaLds<T> L;
     const GgaThread t = gga_thread();
     // head-major order: workgroups that run together work on the same head, hence on the same width, and share the
     // instructions of one of the five width paths (each path is ~40 KB of straight-line code)
@@ -549,7 +552,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
     for (int s = 0; s < RPT; ++s)
 #pragma unroll
         for (int e = 0; e < CT; ++e) acc[0][e] = __builtin_fmaf(krow[s], x[s][e], acc[0][e]);
-    gga_col_allreduce<T, 1, false, 0>(acc, L.red, t);
+    gga_col_allreduce<T, 1, false>(acc);
     float kO[CT];
 #pragma unroll
     for (int e = 0; e < CT; ++e) {
@@ -565,7 +568,7 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
             acc[0][e] = __builtin_fmaf(x[s][e], qrow[s], acc[0][e]);
         }
     }
-    gga_col_allreduce<T, 1, false, 1>(acc, L.red, t);
+    gga_col_allreduce<T, 1, false>(acc);
     float ve[CT], o[CT];
 #pragma unroll
     for (int e = 0; e < CT; ++e) {
@@ -653,7 +656,7 @@ __global__ void gga_advance_kernel(uint8_t* blob, uint64_t slot_stride, const in
 template <class T>
 __global__ __launch_bounds__(GGA_THREADS, 2) void gga_store_kernel(const GgaParams p) {
     constexpr int CT = T::CT, RPT = T::RPT, DK = T::DK, DV = T::DV;
-    __shared__ float red[2 * 2 * GGA_WAVES * DV];
+    __shared__ __attribute__((aligned(16))) float red[GGA_WAVES * DK];
     const GgaThread t = gga_thread();
     // head-major order: workgroups that run together work on the same head, hence on the same width, and share the
     // instructions of one of the five width paths (each path is ~40 KB of straight-line code)
