@@ -233,3 +233,43 @@ def test_arguments_are_checked():
     assert not GGAPacked(q32, 8, 4, 32, 32).supported()                                   # no kernel for d = 32
     out = pk.step(Vp, idx[:0], z(0, 4, 128), z(0, 4, 128), z(0, 8, 128), z(0, 8, 128), 1.0, g=z(0, 8), beta=z(0, 8), layer=0)
     assert out.shape[0] == 0
+
+
+def test_many_slots_twin_rows_and_subset():
+    """64 batch rows x 32 heads (2 048 tiles, several per compute unit): rows r and r + 32 get the same state and the
+    same tokens, so their slots must stay byte-identical and their outputs equal wherever their tiles ran; two rows
+    are checked against the oracle step by step."""
+    B, HV, HK, D, layer = 64, 32, 16, 128, 0
+    g = torch.Generator().manual_seed(21)
+    q = GGAPlan({0: (torch.tensor((WIDTHS[0] * 4)[:HV])[torch.randperm(HV, generator=g)], torch.rand(HV, D, generator=g) + 0.5)})
+    bits, w = q.plan[layer]
+    pk = GGAPacked(q, HV, HK, D, D, pw=True)
+    Vp = pk.views(pk.alloc(B + 1, DEV))
+    idx = (torch.randperm(B, generator=g) + 1).to(torch.int32)
+    half = B // 2
+    S0 = torch.randn(half, HV, D, D, generator=g) * 0.3
+    pk.write(Vp, idx[:half].to(DEV), S0.transpose(-1, -2).to(DEV), layer=layer)
+    pk.write(Vp, idx[half:].to(DEV), S0.transpose(-1, -2).to(DEV), layer=layer)
+    A_log, dtb = torch.randn(HV, generator=g) * 0.3, torch.randn(HV, generator=g) * 0.3
+    rows = [3, 17]
+    sl = idx[rows]
+    ora = G.GGAState(bits, w, B + 1, HV, HK, D, D, pw=True, m=8)
+    two = lambda x: torch.cat([x, x]).to(DEV)                          # noqa: E731
+    for t, (qq, kk, vv, a, b) in enumerate(tokens(10, half, HV, HK, D, seed=8)):
+        ora.O[sl.long()] = pk.stored(Vp, sl.to(DEV), layer).cpu()
+        P, V, n = pk.window(Vp, sl.to(DEV))
+        ora.P[sl.long()], ora.V[sl.long()], ora.n[sl.long()] = P.cpu(), V.cpu(), n.cpu().long()
+        out = torch.full((B, HV, D), 7.0, device=DEV)
+        pk.step(Vp, idx.to(DEV), two(qq), two(kk), two(vv), out, D ** -0.5, gate=(two(a), two(b), A_log.to(DEV), dtb.to(DEV)),
+                layer=layer)
+        got = out.cpu()
+        assert torch.equal(got[:half], got[half:]), t
+        gl, beta = ora.gate(a[rows], b[rows], A_log, dtb)
+        want = ora.step(sl, qq[rows], kk[rows], vv[rows], D ** -0.5, gl, beta)
+        assert ((got[rows] - want).norm() / want.norm()).item() < 1e-5, t
+        Sp, Se = pk.stored(Vp, sl.to(DEV), layer).cpu(), ora.O[sl.long()]
+        assert ((Sp - Se).abs() > 1e-3 * Se.abs().amax()).float().mean().item() < 2e-3, t
+    blob = Vp['blob'].cpu()
+    assert torch.equal(blob[idx[:half].long()], blob[idx[half:].long()])
+    assert blob[idx.long(), :8].view(torch.int32).tolist() == [[8, 2]] * B          # 10 tokens: full, head moved twice
+    assert not blob[0].any()
