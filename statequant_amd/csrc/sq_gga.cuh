@@ -617,8 +617,11 @@ __global__ __launch_bounds__(GGA_THREADS, 2) void gga_step_kernel(const GgaParam
     // ---- re-fit and re-pack in place ----
     gga_store_any<T>(S, bits, x, wrow, L.red, t);
 
-    // ---- queue (R(beta k), R(v)): behind the barriers of the fit, so every read of the slot it may replace is done
+    // ---- queue (R(beta k), R(v)).  A full window's new pair replaces the oldest one, whose right factor every
+    // wavefront has read for the merge: the barrier puts the store behind all of those reads (each wavefront used its
+    // copy before it got here).
     if (window) {
+        __syncthreads();
         const int jn = n < m ? (hd + n) % m : hd;
         if (t.wave == 0) {
             uint32_t code[NE];
