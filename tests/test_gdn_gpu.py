@@ -384,3 +384,52 @@ def test_empty_batch_and_errors():
     SlotLayout(quantizer((4, 'v', 32)), HV, HK, D, D)._layout_struct()
     with pytest.raises(RuntimeError):                            # CPU tensors never reach a kernel
         PackedGDNState(torch.zeros(8, D, D), quantizer((4, 'k', 64)), hv=HV, hk=HK)
+
+
+@pytest.mark.parametrize('fmt', [(4, 'k', 64), (4, 'k', 32), (8, 'k', 32), (8, 'k', 64), (4, 'v', 32), 'bf16'])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+def test_padding_is_exact(fmt, m, bb):
+    """The 96 x 192 kernels == the 128 x 256 kernels on the zero-padded problem (the reference's
+    tests/test_kernels_nonpow2.py:94-136): stored state, buffers, decays and counters bit for bit, outputs to 1e-6
+    (the read's last fp32 operations may associate differently for the two tile shapes).  The padded twin is re-synced
+    to the other after every step, so a rounding flip is counted once."""
+    B, HV, HK, DK, DV, T = 2, 4, 2, 96, 192, 33
+    BH = B * HV
+    pad = lambda x, n: torch.nn.functional.pad(x, (0, n - x.shape[-1])).contiguous()          # noqa: E731
+    gen = torch.Generator().manual_seed(1)
+    S0 = (torch.randn(BH, DK, DV, generator=gen) * 0.5).to(DEV)
+    kw = dict(m=m, hv=HV, hk=HK, buffer_bits=bb, out_dtype=torch.float32)
+    a = PackedGDNState(S0, quantizer(fmt), **kw)
+    p = PackedGDNState(torch.nn.functional.pad(S0, (0, 256 - DV, 0, 128 - DK)), quantizer(fmt), **kw)
+    assert torch.equal(a.dequantize(), p.dequantize()[:, :DK, :DV])
+    diff = {'o': 0, 'S': 0, 'KB': 0, 'UB': 0, 'UBS': 0}
+    worst = 0.0
+    for t in range(T):
+        q, k = torch.randn(B * HK, DK, generator=gen).to(DEV), torch.randn(B * HK, DK, generator=gen).to(DEV)
+        v = torch.randn(BH, DV, generator=gen).to(DEV)
+        g = (-torch.rand(BH, generator=gen) * 0.08).to(DEV)
+        beta = (torch.rand(BH, generator=gen).sigmoid() * 2).to(DEV)                         # OLMo: beta in (0, 2)
+        oa = a.step(q, k, v, g, beta, DK ** -0.5).clone()
+        op = p.step(pad(q, 128), pad(k, 128), pad(v, 256), g, beta, DK ** -0.5).clone()
+        diff['o'] += (oa != op[:, :DV]).sum().item()
+        worst = max(worst, ((oa - op[:, :DV]).abs().max() / op.abs().max()).item())
+        assert torch.equal(op[:, DV:], torch.zeros_like(op[:, DV:]))
+        diff['S'] += (a.dequantize() != p.dequantize()[:, :DK, :DV]).sum().item()
+        diff['KB'] += (a.KB.float() != p.KB.float()[..., :DK]).sum().item()
+        diff['UB'] += (a.UB.float() != p.UB.float()[..., :DV]).sum().item()
+        diff['UBS'] += (a.UBS != p.UBS).sum().item() if bb == 8 else 0
+        assert torch.equal(a.GB, p.GB) and torch.equal(a.GCUR, p.GCUR)
+        assert a.n == p.n == (t + 1) % m
+        c = a.codes                                                                          # re-sync p to a
+        p.codes[:, :c.shape[1], :c.shape[2]] = c
+        if a.fmt is not None:
+            p.scales[:, :a.scales.shape[1], :a.scales.shape[2]] = a.scales
+        p.KB[..., :DK] = a.KB
+        p.UB[..., :DV] = a.UB
+        if bb == 8:
+            p.KBS.copy_(a.KBS)
+            p.UBS.copy_(a.UBS)
+    print(f'\n[pad {fmt} m={m} buf{bb}] differing entries vs the padded power-of-two run: {diff}, max rel o {worst:.1e}')
+    assert worst < 1e-6, (diff, worst)
+    assert all(n == 0 for k_, n in diff.items() if k_ != 'o'), diff
+    assert diff['o'] <= 1e-2 * T * BH * DV, diff
