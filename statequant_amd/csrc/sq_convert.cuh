@@ -68,11 +68,10 @@ __global__ __launch_bounds__(WAVE) void pack_kernel(const PackParams p) {
     reset_counters(p, seq, h, l.lane);
 }
 
-// Value-axis groups of 32 rows (fold.py:139-146): scales [dv / 32][DK].  A lane owns columns 2 lane, 2 lane + 1 and
-// walks the 32 rows of a block twice (absmax, then codes) with the block's 64 values in registers.
-template <int BITS, int DK>
+// Value-axis groups of G rows (fold.py:139-146): scales [dv / G][DK].  A lane owns columns 2 lane, 2 lane + 1 and
+// walks the G rows of a group twice (absmax, then codes) with the group's 2 G values in registers.
+template <int BITS, int DK, int G>
 __global__ __launch_bounds__(WAVE) void pack_v_kernel(const PackParams p) {
-    constexpr int G = 32;
     constexpr float QMAX = float((1 << (BITS - 1)) - 1);
     constexpr int ROW_BYTES = DK * BITS / 8;
     static_assert(DK % 2 == 0 && DK <= 2 * WAVE, "two columns per lane");
@@ -135,11 +134,11 @@ __global__ __launch_bounds__(WAVE) void pack_f_kernel(const PackParams p) {
     reset_counters(p, seq, h, lane);
 }
 
-// AXV: value-axis groups (GROUP = 32); BITS 16 / 32: the unquantized state (GROUP = DK).
+// AXV: value-axis groups of GROUP rows; BITS 16 / 32: the unquantized state (GROUP = DK).
 template <int BITS, int DK, int GROUP, bool AXV>
 int launch_pack(const PackParams& p, hipStream_t stream) {
     if constexpr (BITS >= 16) hipLaunchKernelGGL((pack_f_kernel<BITS, DK>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
-    else if constexpr (AXV) hipLaunchKernelGGL((pack_v_kernel<BITS, DK>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    else if constexpr (AXV) hipLaunchKernelGGL((pack_v_kernel<BITS, DK, GROUP>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     else hipLaunchKernelGGL((pack_kernel<BITS, DK, GROUP>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     return int(hipGetLastError());
 }
@@ -226,7 +225,7 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
                 if constexpr (T::FLT) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) s4[c] = 1.0f;
-                } else if constexpr (AXV) {                       // one scale per (32-row block, column)
+                } else if constexpr (AXV) {                       // one scale per (group of rows, column)
                     const uint2 w = *reinterpret_cast<const uint2*>(SCh + (rc[k] / GROUP) * DK + col);
                     s4[0] = f16_to_f32(uint16_t(w.x)); s4[1] = f16_to_f32(uint16_t(w.x >> 16));
                     s4[2] = f16_to_f32(uint16_t(w.y)); s4[3] = f16_to_f32(uint16_t(w.y >> 16));

@@ -67,7 +67,9 @@ struct Tile {
     // matrix-core pass: blocks of MR rows x MK columns (one lane: one row, 16 columns; lanes 32.. the next 16)
     static constexpr int MR = 32, MK = 32;
     static_assert(DV % MR == 0 && DK % MK == 0 && GROUP % MK == 0, "tile / group must be multiples of 32");
-    static_assert(!AXV || GROUP == MR, "value-axis groups are one row block (32 rows)");
+    static_assert(!AXV || ((GROUP == MR || GROUP == 2 * MR) && DV % GROUP == 0),
+                  "value-axis groups are one or two row blocks (32 or 64 rows)");
+    static constexpr int VB = AXV ? GROUP / MR : 1;       // row blocks per value-axis scale group
     static constexpr int NRB = DV / MR;                   // row blocks
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
@@ -438,12 +440,12 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 
 #pragma unroll
     for (int rb = 0; rb < T::NRB; ++rb) {
-        if constexpr (T::AXV) {
+        if (T::AXV && rb % T::VB == 0) {                     // a new scale group: its planes serve VB row blocks
             float xr[NV][T::NE];
 #pragma unroll
             for (int t = 0; t < T::NE; ++t) {
                 const int e = l.lane + WAVE * t;
-                const float s = e < T::DK ? f16_to_f32(lds_sc[rb * T::DK + (e < T::DK ? e : 0)]) : 0.0f;
+                const float s = e < T::DK ? f16_to_f32(lds_sc[(rb / T::VB) * T::DK + (e < T::DK ? e : 0)]) : 0.0f;
 #pragma unroll
                 for (int v = 0; v < NV; ++v) xr[v][t] = xe[v][t] * s;
             }
@@ -930,7 +932,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
 }
 }
 
-// The fold for value-axis scale groups: one scale per (32-row block, key column), so the block is held "columns
+// The fold for value-axis scale groups: one scale per (group of 32 or 64 rows, key column); a 32-row block is held "columns
 // across lanes" -- lane (j = lane % 32, kb = lane / 32) owns column j of a 32-column step and, in accumulator element
 // 4a + b, row 8a + 4 kb + b -- and a column's absmax is again a per-lane maximum plus one lane exchange.  The rank-1
 // updates run as above with the operands' roles swapped (values feed the rows, keys the columns).  The codes arrive in
@@ -979,8 +981,16 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
 #pragma unroll
     for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[32 * cs + j];
 
+    // A scale group of two row blocks (VB = 2) is visited twice: first for the column maxima over its 64 rows, then
+    // -- the folded values computed again from the still untouched codes -- for the codes.  Visit v: group
+    // v / (VB PH), phase (v / VB) % PH, block v % VB of the group.
+    constexpr int VB = T::VB, PH = VB > 1 ? 2 : 1, VISITS = T::NRB * PH;
+    auto block_of = [](int v) { return (v / (VB * PH)) * VB + v % VB; };
+    float gmx[NCS];
 #pragma unroll 1
-    for (int rb = 0; rb < T::NRB; ++rb) {
+    for (int v = 0; v < VISITS; ++v) {
+        const int rb = block_of(v), grp = rb / VB;
+        const bool last_phase = (v / VB) % PH == PH - 1;
         uint16_t scr[NCS];
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) scr[cs] = scn[cs];
@@ -989,12 +999,13 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
             for (int t = 0; t < NL; ++t)
                 store_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES, nxt[t]);
         }
-        if (rb + 1 < T::NRB) {
+        if (v + 1 < VISITS) {
+            const int rn = block_of(v + 1);
 #pragma unroll
             for (int t = 0; t < NL; ++t)
-                nxt[t] = load_row<T::BITS>(lane_base + ((rb + 1) * T::MR + t * T::RG) * T::ROW_BYTES);
+                nxt[t] = load_row<T::BITS>(lane_base + (rn * T::MR + t * T::RG) * T::ROW_BYTES);
 #pragma unroll
-            for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[(rb + 1) * T::DK + 32 * cs + j];
+            for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[(rn / VB) * T::DK + 32 * cs + j];
         }
         float dop[MT];
 #pragma unroll
@@ -1023,11 +1034,18 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
             float mx = 0.0f;
 #pragma unroll
             for (int e = 0; e < CPL; ++e) mx = fmaxf(mx, fabsf(acc[cs][e]));
-            const float sc = fp16_scale(fmaxf(mx, __shfl_xor(mx, 32)), T::QMAX);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            if constexpr (VB > 1) {
+                if (!last_phase) gmx[cs] = v % VB == 0 ? mx : fmaxf(gmx[cs], mx);
+                mx = gmx[cs];
+            }
+            const float sc = fp16_scale(mx, T::QMAX);
             rs[cs] = 1.0f / sc;
-            if (kb == 0) sc_head[rb * T::DK + 32 * cs + j] = f32_to_f16(sc);
+            // the group's last block writes the scale: the earlier ones' codes were decoded with the old one by then
+            if (kb == 0 && last_phase && v % VB == VB - 1) sc_head[grp * T::DK + 32 * cs + j] = f32_to_f16(sc);
         }
         __syncthreads();                                     // every lane has its codes: the block takes the new ones
+        if (!last_phase) continue;
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) {
 #pragma unroll

@@ -18,11 +18,14 @@ pytestmark = pytest.mark.gpu
 DEV = 'cuda'
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32), (8, 'v', 32), (4, 'v', 32)])
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (8, 'k', 32), (4, 'k', 64), (4, 'k', 32), (8, 'v', 32), (4, 'v', 32), (8, 'v', 64),
+                                 (4, 'v', 64)])
 @pytest.mark.parametrize('dv,dk', [(128, 128), (64, 64), (192, 96), (96, 96)])
 def test_pack_matches_oracle(fmt, dv, dk):
     if fmt[1] == 'k' and fmt[2] > (1 << (dk - 1).bit_length()):
         pytest.skip('group longer than the padded row')
+    if fmt[1] == 'v' and dv % fmt[2]:
+        pytest.skip('value-axis group does not divide d_v')
     gen = torch.Generator().manual_seed(dv + dk + fmt[0] + fmt[2])
     x = torch.randn(37, dv, dk, generator=gen)
     x[0] = 0.0                                             # all-zero heads: scale floor, codes 0
@@ -47,7 +50,7 @@ def _blob_pair(lay, table_args, n_slots, seed):
     return gen, table, raw, dev
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 64), (4, 'k', 32), (4, 'v', 32), (8, 'v', 32), 'bf16', 'fp32'])
+@pytest.mark.parametrize('fmt', [(8, 'k', 64), (4, 'k', 32), (4, 'v', 32), (8, 'v', 32), (8, 'v', 64), 'bf16', 'fp32'])
 def test_write_matches_oracle_whole_blob(fmt):
     HV, HK, D, m = 4, 2, 128, 8
     lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=8)
@@ -66,7 +69,7 @@ def _advance(lay, views, step_fn, schedule):
         step_fn(torch.tensor(live, dtype=torch.int32, device=DEV))
 
 
-@pytest.mark.parametrize('fmt,bb', [((8, 'k', 128), 8), ((4, 'k', 32), 16), ((4, 'v', 32), 8), ((8, 'v', 32), 16),
+@pytest.mark.parametrize('fmt,bb', [((8, 'k', 128), 8), ((4, 'k', 32), 16), ((4, 'v', 32), 8), ((8, 'v', 32), 16), ((4, 'v', 64), 8),
                                     ('bf16', 8), ('fp32', 16)])
 def test_gdn_read_matches_oracle(fmt, bb):
     HV, HK, D, m = 4, 2, 128, 8

@@ -77,12 +77,13 @@ def test_decode_vs_oracle(name, m, bb):
     check(run_decode(FORMATS[name], m, bb), f'{name} m={m} buf{bb}', 40, m)
 
 
-@pytest.mark.parametrize('fmt', [(4, 'v', 32), (8, 'v', 32)])
+@pytest.mark.parametrize('fmt', [(4, 'v', 32), (8, 'v', 32), (8, 'v', 64), (4, 'v', 64)])
 @pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
 @pytest.mark.parametrize('D,DV', [(128, 128), (64, 64), (96, 192)])
 def test_value_axis_groups(fmt, m, bb, D, DV):
-    """Scale groups of 32 value rows per key column (the serving presets int4v / int8v): the scales ride on the
-    read-out vectors in the state pass and the fold holds a block columns-across-lanes."""
+    """Scale groups of 32 value rows per key column (the serving presets int4v / int8v) and of 64 (the int8-v-g64 of
+    the reference's tests): the scales ride on the read-out vectors in the state pass and the fold holds a block
+    columns-across-lanes, visiting a 64-row group twice (column maxima, then codes)."""
     T = 3 * m + 2 if m > 1 else 4
     check(run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=D, DV=DV, T=T), f'{fmt} {D}x{DV} m{m} bb{bb}', T, m)
 
@@ -379,14 +380,14 @@ def test_empty_batch_and_errors():
     e = torch.zeros(0, HK, D, device=DEV)
     assert lay.step(lay.views(blob), torch.zeros(0, dtype=torch.int32, device=DEV), e, e, out, out, 1.0,
                     g=out, beta=out) is out
-    with pytest.raises(NotImplementedError):                     # value-axis groups of 64: layout yes, no kernel built
-        SlotLayout(quantizer((4, 'v', 64)), HV, HK, D, D)._layout_struct()
+    with pytest.raises(NotImplementedError):                     # value-axis groups of 16: layout yes, no kernel built
+        SlotLayout(quantizer((4, 'v', 16)), HV, HK, D, D)._layout_struct()
     SlotLayout(quantizer((4, 'v', 32)), HV, HK, D, D)._layout_struct()
     with pytest.raises(RuntimeError):                            # CPU tensors never reach a kernel
         PackedGDNState(torch.zeros(8, D, D), quantizer((4, 'k', 64)), hv=HV, hk=HK)
 
 
-@pytest.mark.parametrize('fmt', [(4, 'k', 64), (4, 'k', 32), (8, 'k', 32), (8, 'k', 64), (4, 'v', 32), 'bf16'])
+@pytest.mark.parametrize('fmt', [(4, 'k', 64), (4, 'k', 32), (8, 'k', 32), (8, 'k', 64), (4, 'v', 32), (8, 'v', 64), 'bf16'])
 @pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
 def test_padding_is_exact(fmt, m, bb):
     """The 96 x 192 kernels == the 128 x 256 kernels on the zero-padded problem (the reference's

@@ -65,7 +65,8 @@ def check(tal, tag, T, m):
     assert tal.worst_raw < 0.2
 
 
-@pytest.mark.parametrize('fmt,m,bb', [((4, 'v', 32), 8, 8), ((8, 'v', 32), 4, 16), ((4, 'v', 32), 1, 8)])
+@pytest.mark.parametrize('fmt,m,bb', [((4, 'v', 32), 8, 8), ((8, 'v', 32), 4, 16), ((4, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
+                                      ((4, 'v', 64), 4, 16)])
 def test_value_axis_groups(fmt, m, bb):
     """Scale groups of 32 value rows per key column, with KDA's per-channel decay on the stored state."""
     T = 24 if m > 1 else 4

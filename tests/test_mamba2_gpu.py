@@ -73,7 +73,8 @@ def check(tal, tag, T, m):
     assert tal.worst_raw < 0.2
 
 
-@pytest.mark.parametrize('fmt,m,bb', [((8, 'v', 32), 8, 8), ((4, 'v', 32), 4, 16), ((8, 'v', 32), 1, 8)])
+@pytest.mark.parametrize('fmt,m,bb', [((8, 'v', 32), 8, 8), ((4, 'v', 32), 4, 16), ((8, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
+                                      ((4, 'v', 64), 4, 16)])
 def test_value_axis_groups(fmt, m, bb):
     T = 24 if m > 1 else 4
     check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
