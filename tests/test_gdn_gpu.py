@@ -106,6 +106,7 @@ def test_other_head_shapes(D, DV, HV, HK, fmt):
     counts and GQA factors that are not powers of two (6 / 2, 12 / 12: the tile split divides instead of shifting)."""
     T, m = 20, 4
     check(run_decode(fmt, m, 8, B=3, HV=HV, HK=HK, D=D, DV=DV, T=T), f'{D}x{DV} {fmt}', T, m)
+    check(run_decode(fmt, 16, 16, B=2, HV=HV, HK=HK, D=D, DV=DV, T=34), f'{D}x{DV} {fmt} m=16', 34, 16)
 
 
 def test_bf16_inputs_and_output():
@@ -388,13 +389,15 @@ def test_empty_batch_and_errors():
 
 
 @pytest.mark.parametrize('fmt', [(4, 'k', 64), (4, 'k', 32), (8, 'k', 32), (8, 'k', 64), (4, 'v', 32), (8, 'v', 64), 'bf16'])
-@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (16, 16), (4, 16), (1, 8)])
 def test_padding_is_exact(fmt, m, bb):
     """The 96 x 192 kernels == the 128 x 256 kernels on the zero-padded problem (the reference's
     tests/test_kernels_nonpow2.py:94-136): stored state, buffers, decays and counters bit for bit, outputs to 1e-6
     (the read's last fp32 operations may associate differently for the two tile shapes).  The padded twin is re-synced
     to the other after every step, so a rounding flip is counted once."""
     B, HV, HK, DK, DV, T = 2, 4, 2, 96, 192, 33
+    if m == 16 and (fmt == 'bf16' or fmt[1] == 'v'):
+        pytest.skip('value-axis groups and the unquantized control are built for m <= 8')
     BH = B * HV
     pad = lambda x, n: torch.nn.functional.pad(x, (0, n - x.shape[-1])).contiguous()          # noqa: E731
     gen = torch.Generator().manual_seed(1)

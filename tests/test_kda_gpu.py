@@ -92,13 +92,14 @@ def test_decode_vs_oracle(fmt, m, bb):
 @pytest.mark.parametrize('D,fmt', [(96, (4, 'k', 32)), (96, (8, 'k', 32)), (64, (4, 'k', 32)), (64, (8, 'k', 64))])
 def test_non_pow2_and_small_heads(D, fmt):
     check(run_decode(fmt, 4, 8, B=2, H=5, DK=D, DV=D, T=12), f'kda d={D} {fmt}', 12, 4)
+    check(run_decode(fmt, 16, 16, B=1, H=3, DK=D, DV=D, T=33), f'kda d={D} {fmt} m=16', 33, 16)
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((4, 'k', 32), 8, 8), ((8, 'k', 32), 4, 16), ((4, 'k', 64), 1, 8), ((4, 'v', 32), 8, 8),
-                                      ('bf16', 4, 8)])
+                                      ('bf16', 4, 8), ((8, 'k', 64), 16, 16)])
 def test_wide_value_heads(fmt, m, bb):
     """d_k 128, d_v 256: the 'wide' head of the reference's KDA tests (tests/test_kda_kernels.py:21 there)."""
-    T = 20 if m > 1 else 4
+    T = 4 if m == 1 else 34 if m == 16 else 20
     check(run_decode(fmt, m, bb, B=2, H=2, DK=128, DV=256, T=T), f'kda 128x256 {fmt} m={m} buf{bb}', T, m)
 
 

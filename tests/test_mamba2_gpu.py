@@ -99,6 +99,7 @@ def test_decode_vs_oracle(fmt, m, bb):
 @pytest.mark.parametrize('DK,DV,H,G', [(128, 128, 4, 1), (64, 64, 4, 4), (128, 64, 14, 2)])
 def test_other_head_shapes(DK, DV, H, G):
     check(run_decode((8, 'k', 64), 4, 8, B=3, H=H, G=G, DK=DK, DV=DV, T=12), f'mamba2 {DK}x{DV}', 12, 4)
+    check(run_decode((4, 'k', 32), 16, 16, B=2, H=H, G=G, DK=DK, DV=DV, T=33), f'mamba2 {DK}x{DV} m=16', 33, 16)
 
 
 def test_dt_options_and_bf16_inputs():
