@@ -78,7 +78,7 @@ def test_decode_vs_oracle(name, m, bb):
 
 
 @pytest.mark.parametrize('fmt', [(4, 'v', 32), (8, 'v', 32), (8, 'v', 64), (4, 'v', 64)])
-@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 16)])
 @pytest.mark.parametrize('D,DV', [(128, 128), (64, 64), (96, 192)])
 def test_value_axis_groups(fmt, m, bb, D, DV):
     """Scale groups of 32 value rows per key column (the serving presets int4v / int8v) and of 64 (the int8-v-g64 of
@@ -88,7 +88,7 @@ def test_value_axis_groups(fmt, m, bb, D, DV):
     check(run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=D, DV=DV, T=T), f'{fmt} {D}x{DV} m{m} bb{bb}', T, m)
 
 
-@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 8)])
 @pytest.mark.parametrize('D,DV', [(128, 128), (64, 64), (96, 192), (96, 96)])
 def test_unquantized_state_control(m, bb, D, DV):
     """The bf16 state (the reference's control for the packed formats, fold.py:97,128): same step, the state read as
@@ -396,8 +396,6 @@ def test_padding_is_exact(fmt, m, bb):
     (the read's last fp32 operations may associate differently for the two tile shapes).  The padded twin is re-synced
     to the other after every step, so a rounding flip is counted once."""
     B, HV, HK, DK, DV, T = 2, 4, 2, 96, 192, 33
-    if m == 16 and (fmt == 'bf16' or fmt[1] == 'v'):
-        pytest.skip('value-axis groups and the unquantized control are built for m <= 8')
     BH = B * HV
     pad = lambda x, n: torch.nn.functional.pad(x, (0, n - x.shape[-1])).contiguous()          # noqa: E731
     gen = torch.Generator().manual_seed(1)

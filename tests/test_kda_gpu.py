@@ -66,14 +66,14 @@ def check(tal, tag, T, m):
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((4, 'v', 32), 8, 8), ((8, 'v', 32), 4, 16), ((4, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
-                                      ((4, 'v', 64), 4, 16)])
+                                      ((4, 'v', 64), 4, 16), ((8, 'v', 32), 16, 16)])
 def test_value_axis_groups(fmt, m, bb):
     """Scale groups of 32 value rows per key column, with KDA's per-channel decay on the stored state."""
-    T = 24 if m > 1 else 4
+    T = 4 if m == 1 else 34 if m == 16 else 24
     check(run_decode(fmt, m, bb, T=T), f'kda {fmt} m={m} buf{bb}', T, m)
 
 
-@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 16)])
 @pytest.mark.parametrize('D', [128, 96, 64])
 def test_unquantized_state_control(m, bb, D):
     """The bf16 state (kda.py:304: the control for the packed formats) through the same step; the fold multiplies the

@@ -74,13 +74,13 @@ def check(tal, tag, T, m):
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((8, 'v', 32), 8, 8), ((4, 'v', 32), 4, 16), ((8, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
-                                      ((4, 'v', 64), 4, 16)])
+                                      ((4, 'v', 64), 4, 16), ((4, 'v', 32), 16, 8)])
 def test_value_axis_groups(fmt, m, bb):
-    T = 24 if m > 1 else 4
+    T = 4 if m == 1 else 34 if m == 16 else 24
     check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
 
 
-@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8)])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 16)])
 @pytest.mark.parametrize('DK,DV', [(128, 64), (128, 128), (64, 64)])
 def test_unquantized_state_control(m, bb, DK, DV):
     """The bf16 state (mamba2.py:352: the control for the packed formats) through the same step."""
