@@ -68,7 +68,7 @@ typedef struct sq_state {
 typedef struct sq_layout {
     int32_t bits;         /* 4 or 8: codes; 16 / 32: the state kept as bf16 / fp32, no scales (axis_k, group ignored) */
     int32_t axis_k;       /* 1: scale groups along d_k; 0: along d_v (group rows of one key column share a scale) */
-    int32_t group;        /* scale group length, a power of two (value-axis: must divide d_v; built for 32 and 64) */
+    int32_t group;        /* scale group length, a power of two (value-axis: must divide d_v; built for 16, 32, 64) */
     int32_t buffer_bits;  /* 8 (int8 + fp16 scale per vector) or 16 (bf16) */
     int32_t m;            /* buffer length, a power of two */
     int32_t hv, hk;       /* value heads, key heads (groups); hv % hk == 0 */

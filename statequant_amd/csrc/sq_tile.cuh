@@ -66,15 +66,17 @@ struct Tile {
     static constexpr int UROW = NOWN * WAVE;              // floats per d_v vector in LDS
     // matrix-core pass: blocks of MR rows x MK columns (one lane: one row, 16 columns; lanes 32.. the next 16)
     static constexpr int MR = 32, MK = 32;
-    static_assert(DV % MR == 0 && DK % MK == 0 && GROUP % MK == 0, "tile / group must be multiples of 32");
-    static_assert(!AXV || ((GROUP == MR || GROUP == 2 * MR) && DV % GROUP == 0),
-                  "value-axis groups are one or two row blocks (32 or 64 rows)");
-    static constexpr int VB = AXV ? GROUP / MR : 1;       // row blocks per value-axis scale group
+    static_assert(DV % MR == 0 && DK % MK == 0 && (AXV || GROUP % MK == 0), "tile / key-axis group must be multiples of 32");
+    static_assert(!AXV || ((2 * GROUP == MR || GROUP == MR || GROUP == 2 * MR) && DV % GROUP == 0),
+                  "value-axis groups are half a row block, one or two (16, 32 or 64 rows)");
+    static constexpr int VB = AXV && GROUP > MR ? GROUP / MR : 1;    // row blocks per value-axis scale group
+    static constexpr int VH = AXV && GROUP < MR ? MR / GROUP : 1;    // value-axis scale groups per row block
+    static constexpr int PSLOTS = VH > 1 ? 16 : 8;        // digit-plane slots per 16-column piece
     static constexpr int NRB = DV / MR;                   // row blocks
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
     // digit planes: [16-column piece][8 planes][16]; float state: the read-out vectors themselves (at most two)
-    static constexpr int B_BYTES = FLT ? 2 * KROW * 4 : (DK / CPL) * 8 * CPL;
+    static constexpr int B_BYTES = FLT ? 2 * KROW * 4 : (DK / CPL) * PSLOTS * CPL;
     static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
     static constexpr int A_BYTES = FLT ? 0 : MR * A_PITCH;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
@@ -94,10 +96,10 @@ struct LdsPlan {
     static constexpr int XS = SC + T::SC_BYTES;
     // one region, three tenants in turn: the digit planes (until the pass has them in registers), then per row block
     // the codes on their way to operand shape and, once the block's products are issued, its integer sums
-    static constexpr int B = XS + round_up(NV * T::NG * 4, 16);
+    static constexpr int B = XS + round_up(NV * T::VH * T::NG * 4, 16);
     static constexpr int A = B + (T::AXV ? T::B_BYTES : 0);    // value-axis: planes are rebuilt per row block
     static constexpr int C = A;
-    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::PLANES * NV * T::MR * 4;
+    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::VH * T::PLANES * NV * T::MR * 4;
     static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
                                                     : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
     static constexpr int OWN = A + BAC;
@@ -262,7 +264,7 @@ __device__ __forceinline__ void stage_planes(const float (&xe)[NV][T::NE], const
             const uint32_t d = (as_u32(f) + 0x408080u) ^ 0x808080u;
             const int e = l.lane + WAVE * t;
             if (e < T::DK) {
-                uint8_t* at = lds_b + ((e / CPL) * 8 + T::PLANES * v) * CPL + operand_pos<T::BITS>(e % CPL);
+                uint8_t* at = lds_b + ((e / CPL) * T::PSLOTS + T::PLANES * v) * CPL + operand_pos<T::BITS>(e % CPL);
                 at[0] = uint8_t(d);
                 at[CPL] = uint8_t(d >> 8);
                 at[2 * CPL] = uint8_t(d >> 16);
@@ -414,7 +416,10 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
         return;
     } else {
     constexpr int NPL = T::PLANES * NV;
-    constexpr int NCOL = NPL * T::NG;                        // result columns in use: (scale group, vector, digit)
+    // result columns in use: (scale group, vector, digit); value-axis groups of half a row block take the group's
+    // place: columns [h NPL, (h + 1) NPL) carry the read-out against the scales of half h, and a row keeps its own half's
+    constexpr int NGC = T::NG * T::VH;
+    constexpr int NCOL = NPL * NGC;
     static_assert(NCOL <= T::MR && NV <= 2, "groups x digit planes must fit the instruction's 32 result columns");
     const int j = l.lane % T::MR, kb = l.lane / T::MR;
     // second operand, per column step: result column j = g NPL + p takes digit plane p, but only on the column steps
@@ -422,16 +427,18 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
     // its own columns
     const int colg = j / NPL, colp = j - colg * NPL;
     v4i bop[T::NKS];
-    float xs[T::NG];
+    float xs[NGC];
     auto fetch_planes = [&] {
 #pragma unroll
         for (int ks = 0; ks < T::NKS; ++ks) {
-            const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * 8 + (colp & 7)) * CPL);
-            const bool mine = colg == (ks * T::MK) / T::KGROUP;
+            const int slot = T::VH > 1 ? (colg < T::VH ? colg * NPL + colp : 0) : (colp & 7);
+            const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * T::PSLOTS + slot) * CPL);
+            const bool mine = T::VH > 1 ? true : colg == (ks * T::MK) / T::KGROUP;
             bop[ks] = mine ? d : v4i{0, 0, 0, 0};
         }
 #pragma unroll
-        for (int g = 0; g < T::NG; ++g) xs[g] = lds_xs[(kb < NV ? kb : 0) * T::NG + g];
+        for (int g = 0; g < NGC; ++g)
+            xs[g] = T::VH > 1 ? lds_xs[g * NV + (kb < NV ? kb : 0)] : lds_xs[(kb < NV ? kb : 0) * T::NG + g];
     };
     if constexpr (!T::AXV) {
         fetch_planes();
@@ -441,15 +448,19 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 #pragma unroll
     for (int rb = 0; rb < T::NRB; ++rb) {
         if (T::AXV && rb % T::VB == 0) {                     // a new scale group: its planes serve VB row blocks
-            float xr[NV][T::NE];
+            float xr[NV * T::VH][T::NE];                     // (half h, vector v) at h NV + v
 #pragma unroll
             for (int t = 0; t < T::NE; ++t) {
                 const int e = l.lane + WAVE * t;
-                const float s = e < T::DK ? f16_to_f32(lds_sc[(rb / T::VB) * T::DK + (e < T::DK ? e : 0)]) : 0.0f;
 #pragma unroll
-                for (int v = 0; v < NV; ++v) xr[v][t] = xe[v][t] * s;
+                for (int hf = 0; hf < T::VH; ++hf) {
+                    const int grp = T::VH > 1 ? rb * T::VH + hf : rb / T::VB;
+                    const float s = e < T::DK ? f16_to_f32(lds_sc[grp * T::DK + (e < T::DK ? e : 0)]) : 0.0f;
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) xr[hf * NV + v][t] = xe[v][t] * s;
+                }
             }
-            stage_planes<T, NV>(xr, l, lds_b, lds_xs);
+            stage_planes<T, NV * T::VH>(xr, l, lds_b, lds_xs);
             __syncthreads();
             fetch_planes();
         }
@@ -477,13 +488,21 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
         if (kb < NV) {
             const int row = rb * T::MR + j;
             float s = 0.0f;
-#pragma unroll
-            for (int g = 0; g < T::NG; ++g) {
+            if constexpr (T::VH > 1) {                       // the columns of the row's own half
+                const int g = j / T::GROUP;
                 const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
                 const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
                                                __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
-                const float term = T::AXV ? f * xs[g] : (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
-                s = g == 0 ? term : s + term;
+                s = f * (g == 0 ? xs[0] : xs[T::VH - 1]);
+            } else {
+#pragma unroll
+                for (int g = 0; g < T::NG; ++g) {
+                    const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
+                    const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
+                                                   __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
+                    const float term = T::AXV ? f * xs[g] : (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
+                    s = g == 0 ? term : s + term;
+                }
             }
             lds_own[kb * T::UROW + row] = s;
         }
@@ -974,12 +993,17 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
     uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
     uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
 
+    // groups of half a row block (VH = 2): accumulator elements 0..7 (rows 8a + 4 kb + b, a < 2) belong to the first
+    // 16 rows of the block, elements 8..15 to the second; each half has its own scale per column
+    constexpr int VH = T::VH;
     RawRow<T::BITS> nxt[NL];
-    uint16_t scn[NCS];
+    uint16_t scn[NCS][VH];
 #pragma unroll
     for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
 #pragma unroll
-    for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[32 * cs + j];
+    for (int cs = 0; cs < NCS; ++cs)
+#pragma unroll
+        for (int hf = 0; hf < VH; ++hf) scn[cs][hf] = sc_head[hf * T::DK + 32 * cs + j];
 
     // A scale group of two row blocks (VB = 2) is visited twice: first for the column maxima over its 64 rows, then
     // -- the folded values computed again from the still untouched codes -- for the codes.  Visit v: group
@@ -991,9 +1015,11 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
     for (int v = 0; v < VISITS; ++v) {
         const int rb = block_of(v), grp = rb / VB;
         const bool last_phase = (v / VB) % PH == PH - 1;
-        uint16_t scr[NCS];
+        uint16_t scr[NCS][VH];
 #pragma unroll
-        for (int cs = 0; cs < NCS; ++cs) scr[cs] = scn[cs];
+        for (int cs = 0; cs < NCS; ++cs)
+#pragma unroll
+            for (int hf = 0; hf < VH; ++hf) scr[cs][hf] = scn[cs][hf];
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
@@ -1005,7 +1031,9 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
             for (int t = 0; t < NL; ++t)
                 nxt[t] = load_row<T::BITS>(lane_base + (rn * T::MR + t * T::RG) * T::ROW_BYTES);
 #pragma unroll
-            for (int cs = 0; cs < NCS; ++cs) scn[cs] = sc_head[(rn / VB) * T::DK + 32 * cs + j];
+            for (int cs = 0; cs < NCS; ++cs)
+#pragma unroll
+                for (int hf = 0; hf < VH; ++hf) scn[cs][hf] = sc_head[((rn / VB) * VH + hf) * T::DK + 32 * cs + j];
         }
         float dop[MT];
 #pragma unroll
@@ -1021,28 +1049,38 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         for (int cs = 0; cs < NCS; ++cs) {
             const RawRow<T::BITS> r = load_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES);
             const v16i ci = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), ident, v16i{0}, 0, 0, 0);
-            const float s = f16_to_f32(scr[cs]) * DECODE_UNIT<T::BITS>;          // exact (int4 operands are 16 x code)
+            float s[VH];
 #pragma unroll
-            for (int e = 0; e < CPL; ++e) acc[cs][e] = COLVEC ? (float(ci[e]) * s) * cm[cs] : float(ci[e]) * (s * cm[cs]);
+            for (int hf = 0; hf < VH; ++hf)
+                s[hf] = f16_to_f32(scr[cs][hf]) * DECODE_UNIT<T::BITS>;          // exact (int4 operands are 16 x code)
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) {
+                const float se = s[VH > 1 ? e / 8 : 0];
+                acc[cs][e] = COLVEC ? (float(ci[e]) * se) * cm[cs] : float(ci[e]) * (se * cm[cs]);
+            }
 #pragma unroll
             for (int t = 0; t < MT; ++t)
                 acc[cs] = __builtin_amdgcn_mfma_f32_32x32x2f32(dop[t], kop[cs][t], acc[cs], 0, 0, 0);
         }
-        float rs[NCS];
+        float rs[NCS][VH];
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) {
-            float mx = 0.0f;
 #pragma unroll
-            for (int e = 0; e < CPL; ++e) mx = fmaxf(mx, fabsf(acc[cs][e]));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            if constexpr (VB > 1) {
-                if (!last_phase) gmx[cs] = v % VB == 0 ? mx : fmaxf(gmx[cs], mx);
-                mx = gmx[cs];
+            for (int hf = 0; hf < VH; ++hf) {
+                float mx = 0.0f;
+#pragma unroll
+                for (int e = hf * (CPL / VH); e < (hf + 1) * (CPL / VH); ++e) mx = fmaxf(mx, fabsf(acc[cs][e]));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                if constexpr (VB > 1) {
+                    if (!last_phase) gmx[cs] = v % VB == 0 ? mx : fmaxf(gmx[cs], mx);
+                    mx = gmx[cs];
+                }
+                const float sc = fp16_scale(mx, T::QMAX);
+                rs[cs][hf] = 1.0f / sc;
+                // the group's last block writes the scale: the earlier ones' codes were decoded with the old one by then
+                if (kb == 0 && last_phase && v % VB == VB - 1)
+                    sc_head[(grp * VH + hf) * T::DK + 32 * cs + j] = f32_to_f16(sc);
             }
-            const float sc = fp16_scale(mx, T::QMAX);
-            rs[cs] = 1.0f / sc;
-            // the group's last block writes the scale: the earlier ones' codes were decoded with the old one by then
-            if (kb == 0 && last_phase && v % VB == VB - 1) sc_head[grp * T::DK + 32 * cs + j] = f32_to_f16(sc);
         }
         __syncthreads();                                     // every lane has its codes: the block takes the new ones
         if (!last_phase) continue;
@@ -1050,7 +1088,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         for (int cs = 0; cs < NCS; ++cs) {
 #pragma unroll
             for (int e = 0; e < CPL; ++e) {
-                const float f = __builtin_fmaf(acc[cs][e], rs[cs], MAGIC);
+                const float f = __builtin_fmaf(acc[cs][e], rs[cs][VH > 1 ? e / 8 : 0], MAGIC);
                 const uint32_t u = as_u32(__builtin_amdgcn_fmed3f(f, MAGIC - T::QMAX, MAGIC + T::QMAX));
                 const int row = 8 * (e / 4) + 4 * kb + (e % 4);
                 if constexpr (T::BITS == 8) {

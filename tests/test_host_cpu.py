@@ -181,7 +181,7 @@ def test_no_fallback_off_the_gpu():
     """CPU tensors never reach a kernel, and nothing else computes the step instead."""
     with pytest.raises(RuntimeError, match='GPU only'):
         PackedGDNState(torch.zeros(8, 64, 64), sq.Quantizer(4, 'k', 32), hv=4, hk=2)
-    lay = SlotLayout(sq.Quantizer(4, 'v', 16), 4, 2, 128, 128)       # a layout with no kernel instance
+    lay = SlotLayout(sq.Quantizer(4, 'v', 8), 4, 2, 128, 128)        # a layout with no kernel instance
     with pytest.raises(NotImplementedError):
         lay._layout_struct()
     SlotLayout(sq.Quantizer(4, 'v', 32), 4, 2, 128, 128)._layout_struct()

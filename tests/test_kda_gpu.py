@@ -66,7 +66,8 @@ def check(tal, tag, T, m):
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((4, 'v', 32), 8, 8), ((8, 'v', 32), 4, 16), ((4, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
-                                      ((4, 'v', 64), 4, 16), ((8, 'v', 32), 16, 16)])
+                                      ((4, 'v', 64), 4, 16), ((8, 'v', 32), 16, 16), ((4, 'v', 16), 8, 8),
+                                      ((8, 'v', 16), 4, 16), ((4, 'v', 16), 1, 8), ((8, 'v', 16), 16, 8)])
 def test_value_axis_groups(fmt, m, bb):
     """Scale groups of 32 value rows per key column, with KDA's per-channel decay on the stored state."""
     T = 4 if m == 1 else 34 if m == 16 else 24
@@ -96,7 +97,7 @@ def test_non_pow2_and_small_heads(D, fmt):
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((4, 'k', 32), 8, 8), ((8, 'k', 32), 4, 16), ((4, 'k', 64), 1, 8), ((4, 'v', 32), 8, 8),
-                                      ('bf16', 4, 8), ((8, 'k', 64), 16, 16)])
+                                      ('bf16', 4, 8), ((8, 'k', 64), 16, 16), ((8, 'v', 16), 8, 8)])
 def test_wide_value_heads(fmt, m, bb):
     """d_k 128, d_v 256: the 'wide' head of the reference's KDA tests (tests/test_kda_kernels.py:21 there)."""
     T = 4 if m == 1 else 34 if m == 16 else 20

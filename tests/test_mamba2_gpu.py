@@ -74,7 +74,8 @@ def check(tal, tag, T, m):
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((8, 'v', 32), 8, 8), ((4, 'v', 32), 4, 16), ((8, 'v', 32), 1, 8), ((8, 'v', 64), 8, 8),
-                                      ((4, 'v', 64), 4, 16), ((4, 'v', 32), 16, 8)])
+                                      ((4, 'v', 64), 4, 16), ((4, 'v', 32), 16, 8), ((4, 'v', 16), 8, 8),
+                                      ((8, 'v', 16), 4, 16), ((8, 'v', 16), 1, 8), ((4, 'v', 16), 16, 16)])
 def test_value_axis_groups(fmt, m, bb):
     T = 4 if m == 1 else 34 if m == 16 else 24
     check(run_decode(fmt, m, bb, T=T), f'mamba2 {fmt} m={m} buf{bb}', T, m)
