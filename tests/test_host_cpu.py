@@ -237,3 +237,31 @@ def test_gga_bench_byte_model():
     state = 12 * 5376 + 11 * 8704 + 6 * 12800 + 2 * 16896 + 32768
     window = 31 * (8 * (128 + 128 + 8) + 8 * (128 + 4) + 128 + 128 + 8)
     assert bench.gga_bytes_per_slot_step(pk, 0) == 2 * state + window == 713624
+
+
+def test_ctypes_structs_match_the_c_header(tmp_path):
+    """Every argument struct of include/statequant_hip.h as gcc lays it out (size and the offset of each field)
+    against its ctypes mirror in statequant_amd/kernels/_hip.py: a field added, dropped or retyped on one side only
+    would shift everything behind it."""
+    import subprocess
+    pairs = {'sq_state': _hip.SqState, 'sq_layout': _hip.SqLayout, 'sq_gdn_args': _hip.SqGdnArgs,
+             'sq_kda_args': _hip.SqKdaArgs, 'sq_mamba2_args': _hip.SqMamba2Args, 'sq_pack_args': _hip.SqPackArgs,
+             'sq_read_args': _hip.SqReadArgs, 'sq_gga_slots': _hip.SqGgaSlots, 'sq_gga_args': _hip.SqGgaArgs}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{os.path.join(ROOT, "include", "statequant_hip.h")}"',
+             'int main(void) {']
+    for cname, T in pairs.items():
+        lines.append(f'  printf("{cname} %zu", sizeof({cname}));')
+        for fname, _ in T._fields_:
+            lines.append(f'  printf(" %zu", offsetof({cname}, {fname}));')
+        lines.append('  printf("\\n");')
+    lines += ['  return 0;', '}']
+    src, exe = tmp_path / 'abi.c', tmp_path / 'abi'
+    src.write_text('\n'.join(lines))
+    subprocess.run(['gcc', '-std=c11', '-o', str(exe), str(src)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.strip().split('\n')
+    assert len(out) == len(pairs)
+    for line in out:
+        name, size, *offs = line.split()
+        T = pairs[name]
+        assert int(size) == ctypes.sizeof(T), name
+        assert [int(o) for o in offs] == [getattr(T, f).offset for f, _ in T._fields_], name
