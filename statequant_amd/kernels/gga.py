@@ -115,7 +115,9 @@ class GGAPacked:
         return {'blob': blob}
 
     def alloc(self, num_slots, device='cuda'):
-        return torch.zeros(num_slots, self.nbytes, dtype=torch.uint8, device=device)
+        """A zeroed blob; its slot stride is ``nbytes`` rounded up to 16 (``nbytes`` itself is not a multiple of 16 when
+        the window length times the head count is odd)."""
+        return torch.zeros(num_slots, _al(self.nbytes), dtype=torch.uint8, device=device)
 
     def _slots(self, blob, layer):
         _hip.require_gpu(blob, 'GGAPacked')

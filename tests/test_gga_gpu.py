@@ -273,3 +273,57 @@ def test_many_slots_twin_rows_and_subset():
     assert torch.equal(blob[idx[:half].long()], blob[idx[half:].long()])
     assert blob[idx.long(), :8].view(torch.int32).tolist() == [[8, 2]] * B          # 10 tokens: full, head moved twice
     assert not blob[0].any()
+
+
+def _random_gga_configs(n, seed=77):
+    import random
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        HK = rng.choice([1, 2, 3])
+        HV = HK * rng.choice([1, 2, 4])
+        out.append(dict(D=rng.choice([128, 64]), HV=HV, HK=HK, pw=rng.random() < 0.75, m=rng.choice([1, 2, 3, 5, 8]),
+                        B=rng.choice([1, 2, 4]), widths=[rng.choice([2, 4, 6, 8, 16]) for _ in range(HV)],
+                        seed=rng.randrange(1000), bf16=rng.random() < 0.3, steps=rng.choice([6, 12, 19])))
+    return out
+
+
+@pytest.mark.parametrize('cfg', _random_gga_configs(16),
+                         ids=lambda c: f"d{c['D']}-hv{c['HV']}hk{c['HK']}-{'pw%d' % c['m'] if c['pw'] else 'nopw'}-b{c['B']}")
+def test_random_configurations(cfg):
+    """Seeded random plans (any mix of widths, also all pivots or none), head counts, window lengths (also not powers
+    of two), batch sizes with a padding row, fp32 or bf16 tokens: every step from the same stored state and window."""
+    D, HV, HK, B, m, pw = cfg['D'], cfg['HV'], cfg['HK'], cfg['B'], cfg['m'], cfg['pw']
+    g = torch.Generator().manual_seed(cfg['seed'])
+    bits, w = torch.tensor(cfg['widths']), torch.rand(HV, D, generator=g) + 0.5
+    pk = GGAPacked(GGAPlan({3: (bits, w)}), HV, HK, D, D, pw=pw, m=m)
+    Vp = pk.views(pk.alloc(B + 2, DEV))
+    slots = (torch.randperm(B + 1, generator=g)[:B] + 1).to(torch.int32)
+    idx = torch.cat([slots[:1], torch.zeros(1, dtype=torch.int32), slots[1:]])           # row 1 is padding
+    ok = idx > 0
+    live, li = idx[ok].to(DEV), idx[ok].long()
+    pk.write(Vp, live, (torch.randn(B, HV, D, D, generator=g) * 0.3).transpose(-1, -2).to(DEV), layer=3)
+    A_log, dtb = torch.randn(HV, generator=g) * 0.3, torch.randn(HV, generator=g) * 0.3
+    ora = G.GGAState(bits, w, B + 2, HV, HK, D, D, pw=pw, m=m)
+    nonp = (bits != 16)[None, None, :, None]
+    dt = torch.bfloat16 if cfg['bf16'] else torch.float32
+    for t, (qq, kk, vv, a, b) in enumerate(tokens(cfg['steps'], B + 1, HV, HK, D, seed=cfg['seed'] + 1, dtype=dt)):
+        ora.O[li] = pk.stored(Vp, live, 3).cpu()
+        if pw:
+            P, V, n = pk.window(Vp, live)
+            ora.P[li], ora.V[li], ora.n[li] = P.cpu(), V.cpu(), n.cpu().long()
+        op = torch.full((B + 1, HV, D), 7.0, device=DEV)
+        pk.step(Vp, idx.to(DEV), *dev(qq, kk, vv), op, D ** -0.5, gate=tuple(dev(a, b, A_log, dtb)), layer=3)
+        gl, beta = ora.gate(a, b, A_log, dtb)
+        oe = ora.step(idx, qq, kk, vv, D ** -0.5, gl, beta)
+        op = op.cpu()
+        assert float(op[1].abs().max()) == 0.
+        assert ((op - oe).norm() / oe.norm()).item() < 1e-5, t
+        Sp, Se = pk.stored(Vp, live, 3).cpu(), ora.O[li]
+        assert ((Sp - Se).abs() > 1e-3 * Se.abs().amax()).float().mean().item() < 3e-3, t
+        if pw:
+            P, V, n = pk.window(Vp, live)
+            assert torch.equal(n.cpu().long(), ora.n[li]), t
+            assert ((P.cpu() * nonp - ora.P[li]).abs() > 1e-6 * P.abs().amax().cpu()).float().mean().item() < 2e-3, t
+            assert torch.equal(V.cpu() * nonp, ora.V[li] * nonp), t
+    assert not Vp['blob'][0].any()
