@@ -246,3 +246,32 @@ def test_read_is_the_state_the_next_step_reads():
         lay.step(views, idx, q, k, v, g, beta, out)
     rel = ((out - o_pred).norm() / o_pred.norm()).item()
     assert rel < 1e-5, rel
+
+
+def _random_configs(n, seed=59):
+    import random
+    rng = random.Random(seed)
+    fmts = [(4, 'k', 32), (4, 'k', 64), (8, 'k', 32), (8, 'k', 128), (4, 'v', 32), (4, 'v', 16), (8, 'v', 64), 'bf16']
+    out = []
+    while len(out) < n:
+        fmt = rng.choice(fmts)
+        DK, DV = rng.choice([(128, 128), (96, 96), (64, 64), (128, 256)])
+        if fmt != 'bf16' and (DK if fmt[1] == 'k' else DV) % fmt[2]:      # KDA: a group divides its axis (kda.py:55-64)
+            continue
+        out.append(dict(fmt=fmt, DK=DK, DV=DV, m=rng.choice([1, 2, 4, 8, 16]), bb=rng.choice([8, 16]),
+                        H=rng.choice([1, 3, 4, 5]), B=rng.choice([1, 3]), seed=rng.randrange(1000),
+                        dtype=rng.choice([torch.float32, torch.bfloat16])))
+    return out
+
+
+@pytest.mark.parametrize('cfg', _random_configs(12), ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}")
+def test_random_configurations(cfg):
+    """Seeded random combinations of format, head shape, buffer, head count and input dtype; the task's bounds."""
+    T = max(2 * cfg['m'] + 1, 5)
+    tal = run_decode(cfg['fmt'], cfg['m'], cfg['bb'], B=cfg['B'], H=cfg['H'], DK=cfg['DK'], DV=cfg['DV'], T=T,
+                     seed=cfg['seed'], dtype=cfg['dtype'])
+    print('\n' + tal.report(str(cfg)))
+    assert tal.folds == T // cfg['m']
+    assert tal.worst_o < 1e-4, tal.worst_o
+    assert tal.buf_flips <= max(1, 1e-3 * tal.buf_entries), (tal.buf_flips, tal.buf_entries)
+    assert tal.code_mism <= max(1, 1e-3 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)

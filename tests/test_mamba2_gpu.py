@@ -46,10 +46,11 @@ def run_decode(fmt, m, bb, B=2, H=8, G=2, DK=128, DV=64, T=24, seed=1, dtype=tor
         kb, ub = buffer_entry(ker.T, slot, bb == 8)
         tal.entries(kb, ref.K[:, slot])
         tal.entries(ub, ref.U[:, slot])
-        # the decay goes through softplus (log, exp): the device's and the host's libm may differ in the last bit,
-        # so compare to a few ulps and let the oracle continue from the kernel's value
+        # the decay goes through softplus (log (1 + exp)): the device's and the host's libm may differ in the last bit of
+        # the exponential, which the logarithm of a sum near 1 magnifies -- compare to a few ulps of that and let the
+        # oracle continue from the kernel's value
         gk = ker.GB[:, slot].cpu()
-        assert torch.allclose(gk, ref.G[:, slot], rtol=1e-6, atol=1e-7), t
+        assert torch.allclose(gk, ref.G[:, slot], rtol=5e-6, atol=1e-7), t
         ref.G[:, slot] = gk
         ref.gcur = gk.clone()
         ref.K[:, slot], ref.U[:, slot] = kb, ub
@@ -248,3 +249,35 @@ def test_read_is_the_state_the_next_step_reads():
     from statequant_amd.kernels import pack_vk
     c, s = pack_vk(S.reshape(-1, DV, DK), quantizer((8, 'k', 32)))
     assert torch.equal(got, unpack_vk(c, s, quantizer((8, 'k', 32)), DK).view_as(S))
+
+
+def _random_configs(n, seed=31):
+    import random
+    rng = random.Random(seed)
+    fmts = [(4, 'k', 32), (4, 'k', 64), (8, 'k', 32), (8, 'k', 128), (4, 'v', 32), (8, 'v', 16), (8, 'v', 64), 'bf16']
+    out = []
+    while len(out) < n:
+        fmt = rng.choice(fmts)
+        DK, DV = rng.choice([(128, 64), (128, 128), (64, 64)])
+        if fmt != 'bf16' and ((fmt[1] == 'k' and fmt[2] > DK) or (fmt[1] == 'v' and DV % fmt[2])):
+            continue
+        G = rng.choice([1, 2, 3])
+        out.append(dict(fmt=fmt, DK=DK, DV=DV, m=rng.choice([1, 2, 4, 8, 16]), bb=rng.choice([8, 16]), G=G,
+                        H=G * rng.choice([1, 2, 7]), B=rng.choice([1, 3]), seed=rng.randrange(1000),
+                        dtype=rng.choice([torch.float32, torch.bfloat16]), use_D=rng.random() < 0.7,
+                        use_bias=rng.random() < 0.7))
+    return out
+
+
+@pytest.mark.parametrize('cfg', _random_configs(12), ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}g{c['G']}")
+def test_random_configurations(cfg):
+    """Seeded random combinations of format, head shape, buffer, head / group counts (also 7 heads per group), D /
+    dt_bias present or not and input dtype; the task's bounds (99.9 % of entries and codes identical, none off by more than a step)."""
+    T = max(2 * cfg['m'] + 1, 5)
+    tal = run_decode(cfg['fmt'], cfg['m'], cfg['bb'], B=cfg['B'], H=cfg['H'], G=cfg['G'], DK=cfg['DK'], DV=cfg['DV'], T=T,
+                     seed=cfg['seed'], dtype=cfg['dtype'], use_D=cfg['use_D'], use_bias=cfg['use_bias'])
+    print('\n' + tal.report(str(cfg)))
+    assert tal.folds == T // cfg['m']
+    assert tal.worst_o < 1e-4, tal.worst_o
+    assert tal.buf_flips <= max(1, 1e-3 * tal.buf_entries), (tal.buf_flips, tal.buf_entries)
+    assert tal.code_mism <= max(1, 1e-3 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)
