@@ -43,7 +43,7 @@ struct Tile {
     static constexpr int LPR = DK / CPL;                  // live lanes per row
     static constexpr int LPRP = pow2_ceil(LPR);           // lanes per row incl. idle ones
     static constexpr int RG = WAVE / LPRP;                // rows per wavefront load
-    static_assert(DV % (4 * RG) == 0, "d_v must be a multiple of 4 x the rows one wavefront load covers");
+    static_assert(DV % RG == 0 && DV >= 32, "d_v must be a multiple of the rows one wavefront load covers");
     static constexpr int RPL = DV / RG;                   // rows per lane (fold, buffer passes)
     static constexpr int NOWN = (DV + WAVE - 1) / WAVE;   // rows a lane owns after the state pass: lane + 64 t
     static constexpr int KGROUP = AXV ? pow2_ceil(DK) : GROUP;     // length of a scale group along a row
@@ -66,13 +66,16 @@ struct Tile {
     static constexpr int UROW = NOWN * WAVE;              // floats per d_v vector in LDS
     // matrix-core pass: blocks of MR rows x MK columns (one lane: one row, 16 columns; lanes 32.. the next 16)
     static constexpr int MR = 32, MK = 32;
-    static_assert(DV % MR == 0 && DK % MK == 0 && (AXV || GROUP % MK == 0), "tile / key-axis group must be multiples of 32");
+    static_assert(DK % MK == 0 && (AXV || GROUP % MK == 0), "d_k / key-axis group must be multiples of 32");
+    // d_v need not be a multiple of the block height (Nemotron-3-Nano: head_dim 80): the last row block is then
+    // partly empty -- its wavefront loads beyond d_v are skipped (zeros), its stores and scales masked
+    static constexpr bool RAGV = DV % MR != 0;
     static_assert(!AXV || ((2 * GROUP == MR || GROUP == MR || GROUP == 2 * MR) && DV % GROUP == 0),
                   "value-axis groups are half a row block, one or two (16, 32 or 64 rows)");
     static constexpr int VB = AXV && GROUP > MR ? GROUP / MR : 1;    // row blocks per value-axis scale group
     static constexpr int VH = AXV && GROUP < MR ? MR / GROUP : 1;    // value-axis scale groups per row block
     static constexpr int PSLOTS = VH > 1 ? 16 : 8;        // digit-plane slots per 16-column piece
-    static constexpr int NRB = DV / MR;                   // row blocks
+    static constexpr int NRB = (DV + MR - 1) / MR;        // row blocks (the last one may be partly empty)
     static constexpr int NKS = DK / MK;                   // column steps
     static constexpr int PLANES = 3;                      // fixed-point digits per read-out vector
     // digit planes: [16-column piece][8 planes][16]; float state: the read-out vectors themselves (at most two)
@@ -297,14 +300,26 @@ struct Window {
 // Float state: the next FW wavefront loads (SRG rows each), 32 registers as well.
 template <class T>
 struct Window<T, true> {
-    static constexpr int FW = T::NLD < 8 ? T::NLD : 8;
+    static constexpr int FW = T::NLD % 8 == 0 ? 8 : T::NLD % 5 == 0 ? 5 : T::NLD % 4 == 0 ? 4 : T::NLD % 3 == 0 ? 3 : 1;
     uint4 a[FW];
 };
+// One wavefront load of the row-shaped layout: the rows first .. first + RG - 1 (a lane's own: first + rg).  d_v is a
+// multiple of RG, so a load lies wholly inside the head or wholly behind it; behind it nothing is read or written.
+template <class T>
+__device__ __forceinline__ bool rows_inside(int first) { return !T::RAGV || first < T::DV; }
+template <class T>
+__device__ __forceinline__ RawRow<T::BITS> load_rows(const uint8_t* lane_base, int first) {
+    if (!rows_inside<T>(first)) return zero_row<T::BITS>();
+    return load_row<T::BITS>(lane_base + first * T::ROW_BYTES);
+}
+template <class T>
+__device__ __forceinline__ void store_rows(uint8_t* lane_base, int first, const RawRow<T::BITS>& r) {
+    if (rows_inside<T>(first)) store_row<T::BITS>(lane_base + first * T::ROW_BYTES, r);
+}
 template <class T>
 __device__ __forceinline__ void window_load(const uint8_t* lane_base, int rb, Window<T>& w) {
 #pragma unroll
-    for (int j = 0; j < Window<T>::NL; ++j)
-        w.a[rb & 1][j] = load_row<T::BITS>(lane_base + (rb * T::MR + j * T::RG) * T::ROW_BYTES);
+    for (int j = 0; j < Window<T>::NL; ++j) w.a[rb & 1][j] = load_rows<T>(lane_base, rb * T::MR + j * T::RG);
 }
 template <class T>
 __device__ __forceinline__ void window_init(const uint8_t* lane_base, Window<T>& w) {
@@ -857,7 +872,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
     RawRow<T::BITS> nxt[NL];                                 // the next row block and its scales, a block ahead
     uint16_t scn[T::NG];
 #pragma unroll
-    for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
+    for (int t = 0; t < NL; ++t) nxt[t] = load_rows<T>(lane_base, t * T::RG);
 #pragma unroll
     for (int g = 0; g < T::NG; ++g) scn[g] = sc_head[j * T::NG + g];
 
@@ -874,10 +889,10 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
         }
         if (rb + 1 < T::NRB) {
 #pragma unroll
-            for (int t = 0; t < NL; ++t)
-                nxt[t] = load_row<T::BITS>(lane_base + ((rb + 1) * T::MR + t * T::RG) * T::ROW_BYTES);
+            for (int t = 0; t < NL; ++t) nxt[t] = load_rows<T>(lane_base, (rb + 1) * T::MR + t * T::RG);
+            const int rown = !T::RAGV || row + T::MR < T::DV ? row + T::MR : T::DV - 1;     // rows behind d_v: unused
 #pragma unroll
-            for (int g = 0; g < T::NG; ++g) scn[g] = sc_head[(row + T::MR) * T::NG + g];
+            for (int g = 0; g < T::NG; ++g) scn[g] = sc_head[rown * T::NG + g];
         }
         float bop[MT];
 #pragma unroll
@@ -929,7 +944,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             const float other = __shfl_xor(gmax[g], 32);
             const float sc = fp16_scale(fmaxf(gmax[g], other), T::QMAX);
             rs[g] = 1.0f / sc;
-            if (kb == 0) sc_head[row * T::NG + g] = f32_to_f16(sc);
+            if (kb == 0 && (!T::RAGV || row < T::DV)) sc_head[row * T::NG + g] = f32_to_f16(sc);
         }
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) {
@@ -943,8 +958,8 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
-                store_row<T::BITS>(lane_base + (rb * T::MR + t * T::RG) * T::ROW_BYTES,
-                                   load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
+                store_rows<T>(lane_base, rb * T::MR + t * T::RG,
+                              load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
         }
         __syncthreads();
     }
@@ -999,11 +1014,12 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
     RawRow<T::BITS> nxt[NL];
     uint16_t scn[NCS][VH];
 #pragma unroll
-    for (int t = 0; t < NL; ++t) nxt[t] = load_row<T::BITS>(lane_base + (t * T::RG) * T::ROW_BYTES);
+    for (int t = 0; t < NL; ++t) nxt[t] = load_rows<T>(lane_base, t * T::RG);
 #pragma unroll
     for (int cs = 0; cs < NCS; ++cs)
 #pragma unroll
         for (int hf = 0; hf < VH; ++hf) scn[cs][hf] = sc_head[hf * T::DK + 32 * cs + j];
+    constexpr int NGRP = T::DV / T::GROUP;                   // scale groups of the head (a ragged last block has fewer)
 
     // A scale group of two row blocks (VB = 2) is visited twice: first for the column maxima over its 64 rows, then
     // -- the folded values computed again from the still untouched codes -- for the codes.  Visit v: group
@@ -1028,12 +1044,14 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         if (v + 1 < VISITS) {
             const int rn = block_of(v + 1);
 #pragma unroll
-            for (int t = 0; t < NL; ++t)
-                nxt[t] = load_row<T::BITS>(lane_base + (rn * T::MR + t * T::RG) * T::ROW_BYTES);
+            for (int t = 0; t < NL; ++t) nxt[t] = load_rows<T>(lane_base, rn * T::MR + t * T::RG);
 #pragma unroll
             for (int cs = 0; cs < NCS; ++cs)
 #pragma unroll
-                for (int hf = 0; hf < VH; ++hf) scn[cs][hf] = sc_head[((rn / VB) * VH + hf) * T::DK + 32 * cs + j];
+                for (int hf = 0; hf < VH; ++hf) {
+                    const int gi = (rn / VB) * VH + hf;
+                    scn[cs][hf] = sc_head[(gi < NGRP ? gi : NGRP - 1) * T::DK + 32 * cs + j];
+                }
         }
         float dop[MT];
 #pragma unroll
@@ -1078,7 +1096,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
                 const float sc = fp16_scale(mx, T::QMAX);
                 rs[cs][hf] = 1.0f / sc;
                 // the group's last block writes the scale: the earlier ones' codes were decoded with the old one by then
-                if (kb == 0 && last_phase && v % VB == VB - 1)
+                if (kb == 0 && last_phase && v % VB == VB - 1 && grp * VH + hf < NGRP)
                     sc_head[(grp * VH + hf) * T::DK + 32 * cs + j] = f32_to_f16(sc);
             }
         }
@@ -1104,8 +1122,8 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
-                store_row<T::BITS>(lane_base + (rb * T::MR + t * T::RG) * T::ROW_BYTES,
-                                   load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
+                store_rows<T>(lane_base, rb * T::MR + t * T::RG,
+                              load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
         }
         __syncthreads();
     }

@@ -104,6 +104,20 @@ def test_other_head_shapes(DK, DV, H, G):
     check(run_decode((4, 'k', 32), 16, 16, B=2, H=H, G=G, DK=DK, DV=DV, T=33), f'mamba2 {DK}x{DV} m=16', 33, 16)
 
 
+@pytest.mark.parametrize('DK,DV,H,G', [(128, 80, 6, 2), (96, 80, 6, 2)])
+@pytest.mark.parametrize('fmt,m,bb', [((8, 'k', 32), 8, 8), ((4, 'k', 32), 4, 16), ((8, 'k', 128), 1, 8), ((4, 'k', 32), 16, 8),
+                                      ((4, 'v', 16), 8, 8), ((8, 'v', 16), 4, 16), ((8, 'v', 16), 1, 8), ('bf16', 8, 8),
+                                      ('bf16', 4, 16)])
+def test_head_dim_80(DK, DV, H, G, fmt, m, bb):
+    """head_dim 80 = two and a half row blocks: Nemotron-3-Nano's heads (96 x 80 x d_state 128, the model of the
+    reference's end-to-end Mamba2 run, docs/vllm.md:108 there) and the odd head of its tests (d_state 96, head_dim 80,
+    tests/test_mamba2.py:24).  The last block's empty half is neither read nor written."""
+    if fmt != 'bf16' and fmt[1] == 'k' and DK % fmt[2]:
+        pytest.skip('Mamba2: a key group divides d_state')
+    T = 4 if m == 1 else 34 if m == 16 else 20
+    check(run_decode(fmt, m, bb, B=2, H=H, G=G, DK=DK, DV=DV, T=T), f'mamba2 {DK}x{DV} {fmt} m={m} buf{bb}', T, m)
+
+
 def test_dt_options_and_bf16_inputs():
     """No D, no dt_bias, dt given pre-activated (dt_softplus=False), a dt clamp; bf16 x / B / C."""
     check(run_decode((8, 'k', 128), 4, 8, T=8, use_D=False, use_bias=False), 'no D, no bias', 8, 4)
