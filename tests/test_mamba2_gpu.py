@@ -179,10 +179,12 @@ def test_against_reference_golden_vectors(golden, name):
 
 
 # ---------------------------------------------------------------------------------------------------------------
-H, G, DK, DV = 8, 2, 128, 64
+SHAPE = H, G, DK, DV = 8, 2, 128, 64
+NANO = 12, 2, 128, 80                                   # Nemotron-3-Nano's head shape, fewer heads
 
 
-def _setup(fmt, m, bb, seed=0):
+def _setup(fmt, m, bb, seed=0, shape=None):
+    H, G, DK, DV = shape or SHAPE
     gen = torch.Generator().manual_seed(seed)
     lay = Mamba2SlotLayout(quantizer(fmt), H, G, DK, DV, m=m, buffer_bits=bb)
     raw = torch.randint(0, 256, (8, lay.nbytes + 4096), dtype=torch.uint8, generator=gen).to(DEV)
@@ -197,10 +199,13 @@ def _setup(fmt, m, bb, seed=0):
     return lay, raw, blob, views, slots, refs, (A, D, dtb)
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32), 'bf16'])
+@pytest.mark.parametrize('fmt,shape', [((8, 'k', 128), SHAPE), ((4, 'k', 32), SHAPE), ('bf16', SHAPE),
+                                       ((8, 'k', 128), NANO), ((4, 'k', 32), NANO), ((8, 'v', 16), NANO), ('bf16', NANO)],
+                         ids=lambda v: str(v).replace(' ', ''))
 @pytest.mark.parametrize('m,bb', [(8, 8), (2, 16)])
-def test_slot_step_matches_lockstep_per_sequence(fmt, m, bb):
-    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup(fmt, m, bb)
+def test_slot_step_matches_lockstep_per_sequence(fmt, shape, m, bb):
+    H, G, DK, DV = shape
+    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup(fmt, m, bb, shape=shape)
     outside = raw.clone()
     sched = torch.Generator().manual_seed(1)
     gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
@@ -240,10 +245,12 @@ def test_slot_step_matches_lockstep_per_sequence(fmt, m, bb):
     assert torch.equal(raw[keep], outside[keep])
 
 
-def test_read_is_the_state_the_next_step_reads():
+@pytest.mark.parametrize('shape', [SHAPE, NANO], ids=str)
+def test_read_is_the_state_the_next_step_reads(shape):
     """read() + one textbook fp32 Mamba2 step == the kernel's next output (reference: tests/test_mamba2.py:273-300)."""
     m = 8
-    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup((8, 'k', 32), m, 8)
+    H, G, DK, DV = shape
+    lay, raw, blob, views, slots, refs, (A, D, dtb) = _setup((8, 'k', 32), m, 8, shape=shape)
     gens = [torch.Generator().manual_seed(10 + i) for i in range(len(slots))]
     idx = torch.tensor(slots, device=DEV, dtype=torch.int32)
     for t in range(13):
