@@ -104,6 +104,15 @@ def test_wide_value_heads(fmt, m, bb):
     check(run_decode(fmt, m, bb, B=2, H=2, DK=128, DV=256, T=T), f'kda 128x256 {fmt} m={m} buf{bb}', T, m)
 
 
+@pytest.mark.parametrize('fmt', [(4, 'k', 32), (4, 'v', 16), (8, 'k', 32), (8, 'v', 16), (8, 'k', 64), (4, 'v', 32), 'bf16'])
+@pytest.mark.parametrize('m,bb', [(8, 8), (4, 16), (1, 8), (16, 16)])
+def test_single_value_block_head(fmt, m, bb):
+    """3 heads of d_k 64, d_v 32: the 'small' head of the reference's KDA tests (tests/test_kda_kernels.py:21 there) --
+    one 32-row block per tile, so the pass, the fold and the re-read all run their first-and-last iteration at once."""
+    T = 4 if m == 1 else 34 if m == 16 else 20
+    check(run_decode(fmt, m, bb, B=2, H=3, DK=64, DV=32, T=T), f'kda 64x32 {fmt} m={m} buf{bb}', T, m)
+
+
 def test_bf16_inputs():
     check(run_decode((4, 'k', 32), 8, 8, T=16, dtype=torch.bfloat16), 'kda bf16 inputs', 16, 8)
 
@@ -248,14 +257,14 @@ def test_read_is_the_state_the_next_step_reads():
     assert rel < 1e-5, rel
 
 
-def _random_configs(n, seed=59):
+def _random_configs(n, seed=59, shapes=((128, 128), (96, 96), (64, 64), (128, 256))):
     import random
     rng = random.Random(seed)
     fmts = [(4, 'k', 32), (4, 'k', 64), (8, 'k', 32), (8, 'k', 128), (4, 'v', 32), (4, 'v', 16), (8, 'v', 64), 'bf16']
     out = []
     while len(out) < n:
         fmt = rng.choice(fmts)
-        DK, DV = rng.choice([(128, 128), (96, 96), (64, 64), (128, 256)])
+        DK, DV = rng.choice(list(shapes))
         if fmt != 'bf16' and (DK if fmt[1] == 'k' else DV) % fmt[2]:      # KDA: a group divides its axis (kda.py:55-64)
             continue
         out.append(dict(fmt=fmt, DK=DK, DV=DV, m=rng.choice([1, 2, 4, 8, 16]), bb=rng.choice([8, 16]),
@@ -264,7 +273,8 @@ def _random_configs(n, seed=59):
     return out
 
 
-@pytest.mark.parametrize('cfg', _random_configs(12), ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}")
+@pytest.mark.parametrize('cfg', _random_configs(12) + _random_configs(6, seed=61, shapes=((64, 32), (128, 256))),
+                         ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}")
 def test_random_configurations(cfg):
     """Seeded random combinations of format, head shape, buffer, head count and input dtype; the task's bounds."""
     T = max(2 * cfg['m'] + 1, 5)

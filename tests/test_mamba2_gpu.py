@@ -272,14 +272,14 @@ def test_read_is_the_state_the_next_step_reads(shape):
     assert torch.equal(got, unpack_vk(c, s, quantizer((8, 'k', 32)), DK).view_as(S))
 
 
-def _random_configs(n, seed=31):
+def _random_configs(n, seed=31, shapes=((128, 64), (128, 128), (64, 64))):
     import random
     rng = random.Random(seed)
     fmts = [(4, 'k', 32), (4, 'k', 64), (8, 'k', 32), (8, 'k', 128), (4, 'v', 32), (8, 'v', 16), (8, 'v', 64), 'bf16']
     out = []
     while len(out) < n:
         fmt = rng.choice(fmts)
-        DK, DV = rng.choice([(128, 64), (128, 128), (64, 64)])
+        DK, DV = rng.choice(list(shapes))
         if fmt != 'bf16' and ((fmt[1] == 'k' and fmt[2] > DK) or (fmt[1] == 'v' and DV % fmt[2])):
             continue
         G = rng.choice([1, 2, 3])
@@ -290,7 +290,7 @@ def _random_configs(n, seed=31):
     return out
 
 
-@pytest.mark.parametrize('cfg', _random_configs(12), ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}g{c['G']}")
+@pytest.mark.parametrize('cfg', _random_configs(12) + _random_configs(6, seed=37, shapes=((128, 80), (96, 80))), ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}g{c['G']}")
 def test_random_configurations(cfg):
     """Seeded random combinations of format, head shape, buffer, head / group counts (also 7 heads per group), D /
     dt_bias present or not and input dtype; the task's bounds (99.9 % of entries and codes identical, none off by more than a step)."""
