@@ -105,3 +105,48 @@ def test_decode_loop_with_joins_leaves_and_chunked_prefill(fmt):
     assert worst < 1e-2, worst                             # the task's bound on o
     assert torch.equal(blob[0], null_before)               # the null slot was never written
     assert {s.name for s in active} == {'B', 'C', 'D'} and len(free) == 0
+
+
+@pytest.mark.parametrize('m,bb', [(4, 8), (2, 16)])
+def test_external_function_on_the_unpacked_state(m, bb):
+    """The plugin's ``external:`` mode (/root/reference/src/statequant/integrations/vllm_plugin.py:400-410 there): the
+    state stays unpacked fp32 in the slot (``SlotLayout('fp32')``) and, right after a step, a user function is applied
+    through the views to the rows whose buffer just folded -- the fixed-shape form used under graphs (function on
+    every row, kept where folded).  The next step must read what the function left.  The function here is continuous
+    (clamp and scale), so a last-bit difference between kernel and oracle does not grow."""
+    fn = lambda S: S.clamp(-0.8, 0.8) * 0.9                 # noqa: E731
+    lay = SlotLayout('fp32', HV, HK, D, D, m=m, buffer_bits=bb)
+    gen = torch.Generator().manual_seed(23)
+    views = lay.views(lay.alloc(5, DEV))
+    slots = torch.tensor([4, 0, 2], dtype=torch.int32)       # the middle row is padding (null slot)
+    live = [0, 2]
+    S0 = torch.randn(2, HV, D, D, generator=gen) * 0.5
+    lay.write(views, slots[live].to(DEV), S0.to(DEV))
+    ref = ST.GDNOracle(S0.reshape(-1, D, D), ST.IDENT, m=m, hv=HV, hk=HK, buffer_bits=bb)
+    idx = slots.to(DEV)
+    null_before = views['S'][0].clone()
+    applied = 0
+    for t in range(3 * m + 1):
+        q, k, v = torch.randn(3, HK, D, generator=gen), torch.randn(3, HK, D, generator=gen), torch.randn(3, HV, D, generator=gen)
+        g, beta = -torch.rand(3, HV, generator=gen) * 0.2, torch.rand(3, HV, generator=gen)
+        out = torch.empty(3, HV, D, device=DEV)
+        lay.step(views, idx, q.to(DEV), k.to(DEV), v.to(DEV), out, D ** -0.5, g=g.to(DEV), beta=beta.to(DEV))
+        folded = (views['NPTR'][idx.long(), 0] == 0) & (idx > 0)
+        S = views['S'][idx.long()]
+        views['S'][idx.long()] = torch.where(folded[:, None, None, None], fn(S), S)
+        want = ref.step(q[live].reshape(-1, D), k[live].reshape(-1, D), v[live].reshape(-1, D), g[live].reshape(-1),
+                        beta[live].reshape(-1), D ** -0.5).view(2, HV, D)
+        if ref.n == 0:
+            ref.S0 = fn(ref.S0)
+            applied += 1
+            assert folded.cpu().tolist() == [True, False, True]
+        else:
+            assert not folded.any()
+        got = out.cpu()[live]
+        assert ((got - want).abs().max() / want.abs().max()).item() < 1e-4, t
+        assert float(out[1].abs().max()) == 0.0
+    assert applied == 3
+    got = views['S'][slots[live].long().to(DEV)].cpu().reshape(-1, D, D)
+    assert ((got - ref.S0).abs().max() / ref.S0.abs().max()).item() < 1e-4
+    assert float(got.abs().max()) <= 0.8 * 0.9 * 1.5         # the clamp took hold (steps after the fold add little)
+    assert torch.equal(views['S'][0], null_before)
