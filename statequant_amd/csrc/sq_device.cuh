@@ -15,6 +15,15 @@
 namespace sq {
 
 constexpr int WAVE = 64;
+
+// Ordering point for LDS traffic between the lanes of ONE wavefront (the step kernels run one wavefront per tile): the
+// LDS executes a wavefront's instructions in issue order, so a read issued after a write sees it; what is needed is
+// that the compiler keeps that order.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 constexpr int CPL = 16;                       // state columns per lane
 constexpr float FP16_TINY = 5.960464477539063e-08f;   // 2^-24: floor of a stored fp16 scale
 

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     float ubs[T::MMAX];
 #pragma unroll
     for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(F.ubs_raw), i) : 1.0f;
-    __syncthreads();
+    wave_sync();
     float x[2][CPL];
     lds_piece<T>(lds_q, l.cg, x[0]);
     lds_piece<T>(lds_kn, l.cg, x[1]);
@@ -272,7 +272,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
         float f[T::MMAX];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) f[i] = lane_bcast(decf, i);
-        __syncthreads();                                  // the front end's LDS is dead from here on
+        wave_sync();                                  // the front end's LDS is dead from here on
         fold_stage_values<T>(uo, f, m, l, lds_u);
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
             if (i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
         }
         fold_stage_key<T>(kr, m - 1, l, lds_k);
-        __syncthreads();
+        wave_sync();
         if constexpr (T::AXV) fold_tile_v<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
         else fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
     }

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     float ubs[T::MMAX];
 #pragma unroll
     for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(ubs_raw), i) : 1.0f;
-    __syncthreads();
+    wave_sync();
 
     // ---- buffer coefficients with the per-channel decay ratio folded into the buffered key ----
     float cqk[2][T::MMAX];
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
         float f[T::MMAX];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) f[i] = 1.0f;            // the decay ratio sits on the keys, per channel
-        __syncthreads();                                          // the front end's LDS is dead from here on
+        wave_sync();                                          // the front end's LDS is dead from here on
         fold_stage_values<T>(uo, f, m, l, lds_u);
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
             const int e = l.lane + WAVE * t;
             if (e < T::LPRP * CPL) lds_c[kpos<T>(e)] = e < DK ? expf(gn[t]) : 0.0f;     // = A
         }
-        __syncthreads();
+        wave_sync();
         if constexpr (T::AXV) fold_tile_v<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
         else fold_tile<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
     }

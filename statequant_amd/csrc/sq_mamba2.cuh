@@ -132,7 +132,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     float ubs[T::MMAX];
 #pragma unroll
     for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(ubs_raw), i) : 1.0f;
-    __syncthreads();
+    wave_sync();
     float x[1][CPL];
     lds_piece<T>(lds_cv, l.cg, x[0]);
 
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         float f[T::MMAX];
 #pragma unroll
         for (int i = 0; i < T::MMAX; ++i) f[i] = lane_bcast(decf, i);
-        __syncthreads();
+        wave_sync();
         fold_stage_values<T>(uo, f, m, l, lds_u);
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
             if (i < m - 1) stage_kpiece<T>(lds_k, i, l, kb);
         }
         fold_stage_key<T>(kr, m - 1, l, lds_k);
-        __syncthreads();
+        wave_sync();
         if constexpr (T::AXV) fold_tile_v<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
         else fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, Sh, SCh, l);
     }

@@ -376,7 +376,7 @@ __device__ __forceinline__ void float_pass(const uint8_t* lane_base, Window<T>& 
             const int e = l.lane + WAVE * t;
             if (e < T::LPRP * CPL) xf[v * T::KROW + kpos<T>(e)] = xe[v][t];
         }
-    __syncthreads();
+    wave_sync();
     float xc[NV][T::SPL];
 #pragma unroll
     for (int v = 0; v < NV; ++v) float_cols<T>(xf + v * T::KROW, scg, xc[v]);
@@ -402,7 +402,7 @@ __device__ __forceinline__ void float_pass(const uint8_t* lane_base, Window<T>& 
             }
         }
     }
-    __syncthreads();
+    wave_sync();
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
@@ -457,7 +457,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
     };
     if constexpr (!T::AXV) {
         fetch_planes();
-        __syncthreads();                                     // the planes' region now carries the row blocks
+        wave_sync();                                     // the planes' region now carries the row blocks
     }
 
 #pragma unroll
@@ -476,7 +476,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
                 }
             }
             stage_planes<T, NV * T::VH>(xr, l, lds_b, lds_xs);
-            __syncthreads();
+            wave_sync();
             fetch_planes();
         }
         if (l.cg < T::LPR) {
@@ -485,21 +485,21 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
                 store_row<T::BITS>(lds_a + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES, w.a[rb & 1][t]);
         }
         if (rb + 2 < T::NRB) window_load<T>(lane_base, rb + 2, w);
-        __syncthreads();
+        wave_sync();
         v16i acc = {0};
 #pragma unroll
         for (int ks = 0; ks < T::NKS; ++ks) {
             const RawRow<T::BITS> r = load_row<T::BITS>(lds_a + j * T::A_PITCH + (2 * ks + kb) * T::LANE_BYTES);
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), bop[ks], acc, 0, 0, 0);
         }
-        __syncthreads();                                     // every lane has its codes: the sums may take their place
+        wave_sync();                                     // every lane has its codes: the sums may take their place
         if (j < NCOL) {
             int4* dst = reinterpret_cast<int4*>(lds_c + j * T::MR + 4 * kb);
 #pragma unroll
             for (int a = 0; a < 4; ++a)
                 dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
         }
-        __syncthreads();
+        wave_sync();
         if (kb < NV) {
             const int row = rb * T::MR + j;
             float s = 0.0f;
@@ -521,7 +521,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
             }
             lds_own[kb * T::UROW + row] = s;
         }
-        __syncthreads();
+        wave_sync();
     }
 #pragma unroll
     for (int v = 0; v < NV; ++v)
@@ -865,7 +865,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
                 aop[cs][t] = slot < m ? v : 0.0f;
             }
     }
-    __syncthreads();                                         // lds_k becomes the block buffer
+    wave_sync();                                         // lds_k becomes the block buffer
     uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
     uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
 
@@ -901,7 +901,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             const float v = lds_u[(slot < m ? slot : 0) * T::UROW + row];
             bop[t] = slot < m ? v : 0.0f;
         }
-        __syncthreads();
+        wave_sync();
 
         v16f acc[NCS];
 #pragma unroll
@@ -954,14 +954,14 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             store_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES,
                                quantize_row<T::BITS>(a16, rs[(cs * T::MK) / T::GROUP]));
         }
-        __syncthreads();
+        wave_sync();
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
                 store_rows<T>(lane_base, rb * T::MR + t * T::RG,
                               load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
         }
-        __syncthreads();
+        wave_sync();
     }
 }
 }
@@ -1004,7 +1004,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         ident[2] = t / 4 == 2 ? one : 0;
         ident[3] = t / 4 == 3 ? one : 0;
     }
-    __syncthreads();                                         // lds_k becomes the block buffer
+    wave_sync();                                         // lds_k becomes the block buffer
     uint8_t* blk = reinterpret_cast<uint8_t*>(lds_k);
     uint8_t* lane_base = const_cast<uint8_t*>(lane_codes<T>(head, l));
 
@@ -1060,7 +1060,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
             const float v = lds_u[(slot < m ? slot : 0) * T::UROW + rb * T::MR + j];
             dop[t] = slot < m ? v : 0.0f;
         }
-        __syncthreads();
+        wave_sync();
 
         v16f acc[NCS];
 #pragma unroll
@@ -1100,7 +1100,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
                     sc_head[(grp * VH + hf) * T::DK + 32 * cs + j] = f32_to_f16(sc);
             }
         }
-        __syncthreads();                                     // every lane has its codes: the block takes the new ones
+        wave_sync();                                     // every lane has its codes: the block takes the new ones
         if (!last_phase) continue;
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) {
@@ -1118,14 +1118,14 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
                 }
             }
         }
-        __syncthreads();
+        wave_sync();
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
                 store_rows<T>(lane_base, rb * T::MR + t * T::RG,
                               load_row<T::BITS>(blk + (t * T::RG + l.rg) * T::A_PITCH + l.cg * T::LANE_BYTES));
         }
-        __syncthreads();
+        wave_sync();
     }
 }
 
