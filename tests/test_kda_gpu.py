@@ -113,6 +113,27 @@ def test_single_value_block_head(fmt, m, bb):
     check(run_decode(fmt, m, bb, B=2, H=3, DK=64, DV=32, T=T), f'kda 64x32 {fmt} m={m} buf{bb}', T, m)
 
 
+@pytest.mark.parametrize('bb', [8, 16])
+def test_bf16_control_tracks_the_fp32_recurrence(bb):
+    """The bf16 state (the control arm) against the textbook fp32 recurrence over 64 tokens, to bf16 / int8-buffer
+    accuracy -- the reference's own bounds for this comparison (tests/test_kda_kernels.py:151-172 there)."""
+    H, DK, DV = 4, 128, 128
+    gen = torch.Generator().manual_seed(5)
+    S0 = torch.randn(2 * H, DV, DK, generator=gen)
+    S = S0.to(torch.bfloat16).float()
+    ker = PackedKDAState(S0.to(DEV), 'bf16', m=8, hv=H, buffer_bits=bb, out_dtype=torch.float32)
+    rel2 = 0.0
+    for t in range(64):
+        q, k, v, g, beta = kda_token(gen, 2, H, DK, DV)
+        want = ST.kda_recurrence(S, q.reshape(-1, DK), k.reshape(-1, DK), v.reshape(-1, DV), g.reshape(-1, DK),
+                                 beta.reshape(-1))
+        got = ker.step(q.to(DEV), k.to(DEV), v.to(DEV), g.to(DEV), beta.to(DEV)).cpu().reshape(-1, DV)
+        rel2 = max(rel2, ((got - want).norm() / want.norm()).item())
+    st = ((ker.dequantize().cpu().view_as(S) - S).norm() / S.norm()).item()
+    print(f'\nkda bf16 state buf{bb} vs fp32 recurrence: rel l2 {rel2:.2e}, state {st:.2e}')
+    assert rel2 < (1.5e-2 if bb == 8 else 5e-3) and st < 1e-2
+
+
 def test_bf16_inputs():
     check(run_decode((4, 'k', 32), 8, 8, T=16, dtype=torch.bfloat16), 'kda bf16 inputs', 16, 8)
 

@@ -118,6 +118,32 @@ def test_head_dim_80(DK, DV, H, G, fmt, m, bb):
     check(run_decode(fmt, m, bb, B=2, H=H, G=G, DK=DK, DV=DV, T=T), f'mamba2 {DK}x{DV} {fmt} m={m} buf{bb}', T, m)
 
 
+def test_large_gqa_one_group():
+    """Mamba-2 / Falcon-H1 / Granite style: one B / C group shared by all 64 heads (tests/test_mamba2.py:115-132 there)."""
+    check(run_decode((4, 'k', 64), 8, 8, B=2, H=64, G=1, DK=128, DV=64, T=12), 'mamba2 64 heads, 1 group', 12, 8)
+
+
+@pytest.mark.parametrize('DK,DV,H,G', [(128, 64, 8, 2), (96, 80, 6, 2)])
+@pytest.mark.parametrize('bb', [8, 16])
+def test_bf16_control_tracks_the_fp32_recurrence(DK, DV, H, G, bb):
+    """The bf16 state (the control arm) against the textbook fp32 recurrence over 64 tokens, to bf16 / int8-buffer
+    accuracy -- the reference's own bounds for this comparison (tests/test_mamba2.py:156-174 there)."""
+    gen = torch.Generator().manual_seed(5)
+    S0 = torch.randn(2, H, DV, DK, generator=gen)
+    S = S0.to(torch.bfloat16).float()
+    ker = PackedMamba2State(S0.to(DEV), 'bf16', m=8, hv=H, hk=G, buffer_bits=bb, out_dtype=torch.float32)
+    A, D, dtb = params(gen, H)
+    rel2 = 0.0
+    for t in range(64):
+        x, dt, Bm, C = m2_token(gen, 2, H, G, DK, DV)
+        want = ST.mamba2_recurrence(S, x, dt, Bm, C, A, D, dtb, True, None).reshape(2, H, DV)
+        got = ker.step(x.to(DEV), dt.to(DEV), Bm.to(DEV), C.to(DEV), A.to(DEV), D.to(DEV), dtb.to(DEV), True).cpu()
+        rel2 = max(rel2, ((got.view_as(want) - want).norm() / want.norm()).item())
+    st = ((ker.dequantize().cpu().view_as(S) - S).norm() / S.norm()).item()
+    print(f'\nmamba2 {DK}x{DV} bf16 state buf{bb} vs fp32 recurrence: rel l2 {rel2:.2e}, state {st:.2e}')
+    assert rel2 < (1.5e-2 if bb == 8 else 5e-3) and st < 1e-2
+
+
 def test_dt_options_and_bf16_inputs():
     """No D, no dt_bias, dt given pre-activated (dt_softplus=False), a dt clamp; bf16 x / B / C."""
     check(run_decode((8, 'k', 128), 4, 8, T=8, use_D=False, use_bias=False), 'no D, no bias', 8, 4)

@@ -150,3 +150,84 @@ def test_graph_replay_matches_eager():
         assert torch.equal(blobs[0], blobs[1]), f'state differs after replay {rep}'
         for s in range(m):
             assert torch.equal(outs[0][s], outs[1][s]), (rep, s)
+
+
+def _replay_with_changing_slot_tables(lay, call, feed, S0, tables, idx, rounds=5):
+    """Capture ONE padded-batch step, replay it with the slot table and the inputs rewritten in place between replays
+    (padding rows at the null slot and at -1, sequences whose counters diverge), next to an eager twin on a second
+    blob; blobs and outputs must stay bit-identical (the reference's graph tests: tests/test_kda_kernels.py:313-345,
+    tests/test_mamba2.py:350-385 there)."""
+    blobs = [lay.alloc(8, DEV) for _ in range(2)]
+    views = [lay.views(b) for b in blobs]
+    live = torch.tensor(sorted({s for t in tables for s in t if s > 0}), device=DEV)
+    for v in views:
+        lay.write(v, live, S0[:len(live)])
+    outs = [torch.zeros_like(feed(None)) for _ in range(2)]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        call(views[0], outs[0])                              # warm-up on the capture stream: idx all padding
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            call(views[0], outs[0])
+    torch.cuda.synchronize()
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for r, tab in enumerate(tables * rounds):
+        idx.copy_(torch.tensor(tab, dtype=torch.int32))
+        feed(gen)
+        graph.replay()
+        call(views[1], outs[1])
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), (r, tab)
+        assert torch.equal(blobs[0], blobs[1]), (r, tab)
+    n = views[0]['NPTR'][live, 0].tolist()
+    assert len(set(n)) > 1, n                                # the sequences really were out of step
+
+
+TABLES = [[5, 2, 7, 0], [2, 0, -1, 0], [7, 5, 0, 0], [5, 7, 2, -1], [0, 0, 5, 0]]
+
+
+@pytest.mark.parametrize('fmt', [(4, 'k', 64), (8, 'v', 32), 'bf16'])
+def test_kda_graph_replay_with_changing_slot_tables(fmt):
+    from statequant_amd.kernels import KDASlotLayout
+    H, K, Vd, R = 4, 128, 128, 4
+    lay = KDASlotLayout(fmt if fmt == 'bf16' else sq.Quantizer(*fmt), H, K, Vd, m=4, buffer_bits=8)
+    idx = torch.zeros(R, device=DEV, dtype=torch.int32)
+    proj = torch.zeros(R, 2 * H * K + H * Vd, device=DEV, dtype=torch.bfloat16)   # q / k / v: slices of one projection
+    q, k, v = proj[:, :H * K].view(R, H, K), proj[:, H * K:2 * H * K].view(R, H, K), proj[:, 2 * H * K:].view(R, H, Vd)
+    g, beta = torch.zeros(R, H, K, device=DEV), torch.zeros(R, H, device=DEV)
+
+    def feed(gen):
+        if gen is not None:
+            proj.copy_(torch.randn(proj.shape, device=DEV, generator=gen))
+            g.copy_(-5 * torch.sigmoid(torch.randn(g.shape, device=DEV, generator=gen) * 2 - 3))
+            beta.copy_(torch.sigmoid(torch.randn(beta.shape, device=DEV, generator=gen)))
+        return torch.zeros(R, H, Vd, device=DEV, dtype=torch.bfloat16)
+
+    S0 = torch.randn(3, H, Vd, K, device=DEV) * 0.4
+    _replay_with_changing_slot_tables(lay, lambda vw, o: lay.step(vw, idx, q, k, v, g, beta, o), feed, S0, TABLES, idx)
+
+
+@pytest.mark.parametrize('fmt,P', [((8, 'k', 128), 64), ((4, 'k', 32), 80), ('bf16', 64)])
+def test_mamba2_graph_replay_with_changing_slot_tables(fmt, P):
+    from statequant_amd.kernels import Mamba2SlotLayout
+    H, G, N, R = 8, 2, 128, 4
+    lay = Mamba2SlotLayout(fmt if fmt == 'bf16' else sq.Quantizer(*fmt), H, G, N, P, m=4, buffer_bits=8)
+    idx = torch.zeros(R, device=DEV, dtype=torch.int32)
+    x = torch.zeros(R, H, P, device=DEV, dtype=torch.bfloat16)
+    dt = torch.zeros(R, H, device=DEV)
+    Bm, Cm = torch.zeros(R, G, N, device=DEV), torch.zeros(R, G, N, device=DEV)
+    A = -torch.exp(torch.rand(H, device=DEV) * 2)
+    D, dtb = torch.randn(H, device=DEV), torch.randn(H, device=DEV) * 0.3
+
+    def feed(gen):
+        if gen is not None:
+            x.copy_(torch.randn(x.shape, device=DEV, generator=gen))
+            dt.copy_(torch.randn(dt.shape, device=DEV, generator=gen) * 0.5 - 2)
+            Bm.copy_(torch.randn(Bm.shape, device=DEV, generator=gen))
+            Cm.copy_(torch.randn(Cm.shape, device=DEV, generator=gen))
+        return torch.zeros(R, H, P, device=DEV)
+
+    S0 = torch.randn(3, H, P, N, device=DEV) * 0.4
+    _replay_with_changing_slot_tables(lay, lambda vw, o: lay.step(vw, idx, x, dt, Bm, Cm, o, A, D, dtb), feed, S0,
+                                      TABLES, idx)
