@@ -251,7 +251,7 @@ class PackedGDNState:
     def stored_bytes(self):
         """Resident bytes: state payload + scales, the buffer, the decays (fold.py:371-378)."""
         nb = lambda t: t.numel() * t.element_size()          # noqa: E731
-        per = dict(state=nb(self.codes) + nb(self.scales),
+        per = dict(state=nb(self.codes) + (nb(self.scales) if self.fmt is not None else 0),   # bf16 state: no scales
                    buffer=nb(self.KB) + nb(self.UB) + ((nb(self.KBS) + nb(self.UBS)) if self.qbuf else 0),
                    decay=nb(self.GB) + nb(self.GCUR) + nb(self.NPTR))
         per['total'] = sum(per.values())

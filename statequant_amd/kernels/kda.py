@@ -141,7 +141,7 @@ class PackedKDAState:
     def stored_bytes(self):
         nb = lambda t: t.numel() * t.element_size()          # noqa: E731
         T = self.T
-        per = dict(state=nb(T['S']) + nb(T['SC']),
+        per = dict(state=nb(T['S']) + (nb(T['SC']) if self.fmt is not None else 0),          # bf16 state: no scales
                    buffer=nb(T['KB']) + nb(T['UB']) + ((nb(T['KBS']) + nb(T['UBS'])) if self.qbuf else 0),
                    decay=nb(T['GB']) + nb(T['GCUR']) + nb(T['NPTR']))
         per['total'] = sum(per.values())

@@ -377,6 +377,28 @@ def test_strided_inputs_like_the_serving_engine():
     assert torch.equal(o1, o2)
 
 
+def test_stored_bytes():
+    """Resident-byte accounting of the lockstep classes (tests/test_kernels.py:190-196 there), the unquantized control
+    included (no scales)."""
+    from statequant_amd.kernels import PackedKDAState, PackedMamba2State
+    B, hv, hk, d = 2, 4, 2, 128
+    BH = B * hv
+    S0 = torch.zeros(BH, d, d, device=DEV)
+    st = PackedGDNState(S0, sq.Quantizer(4, 'k', 64), m=8, hv=hv, hk=hk)
+    b = st.stored_bytes()
+    assert b['state'] == BH * d * d // 2 + BH * d * (d // 64) * 2
+    assert b['buffer'] == B * hk * 8 * d + BH * 8 * d + 2 * (B * hk * 8 + BH * 8)
+    assert b['total'] == b['state'] + b['buffer'] + b['decay']
+    assert torch.equal(st.dequantize(), S0)
+    assert PackedGDNState(S0, 'bf16', m=8, hv=hv, hk=hk, buffer_bits=16).stored_bytes()['state'] == BH * d * d * 2
+    k = PackedKDAState(S0, 'bf16', m=8, hv=hv, buffer_bits=16).stored_bytes()
+    assert k['state'] == BH * d * d * 2 and k['buffer'] == 2 * BH * 8 * d * 2
+    assert k['decay'] == BH * 8 * d * 4 + BH * d * 4 + BH * 4
+    m2 = PackedMamba2State(S0, sq.Quantizer(8, 'k', 32), m=8, hv=hv, hk=hk).stored_bytes()
+    assert m2['state'] == BH * d * d + BH * d * (d // 32) * 2
+    assert m2['buffer'] == B * hk * 8 * d + BH * 8 * d + 2 * (B * hk * 8 + BH * 8)
+
+
 def test_empty_batch_and_errors():
     lay = SlotLayout(quantizer((4, 'k', 64)), HV, HK, D, D)
     blob = lay.alloc(2, DEV)
