@@ -282,6 +282,7 @@ def test_fp32_slot_state_follows_the_unrounded_oracle(m, bb):
     slots = torch.tensor([3, 1])
     S0 = torch.randn(2, HV, D, D, generator=gen) * 0.5
     lay.write(views, slots.to(DEV), S0.to(DEV))
+    assert torch.equal(views['S'][slots.to(DEV)].cpu(), S0)          # write stores an fp32 state as it is
     ref = ST.GDNOracle(S0.reshape(-1, D, D), ST.IDENT, m=m, hv=HV, hk=HK, buffer_bits=bb)
     idx = slots.to(torch.int32).to(DEV)
     for t in range(2 * m + 3):

@@ -265,3 +265,16 @@ def test_ctypes_structs_match_the_c_header(tmp_path):
         T = pairs[name]
         assert int(size) == ctypes.sizeof(T), name
         assert [int(o) for o in offs] == [getattr(T, f).offset for f, _ in T._fields_], name
+
+
+def test_unsupported_dims_refused_and_olmo_bytes():
+    """The constructor's refusals and the OLMo-Hybrid-7B byte counts (tests/test_kernels_nonpow2.py:308-321 there)."""
+    with pytest.raises(AssertionError, match='value group'):
+        SlotLayout(sq.Quantizer(4, 'v', 128), 4, 2, 96, 192)
+    with pytest.raises(AssertionError, match='multiple of 32'):
+        SlotLayout('bf16', 4, 2, 96, 80)
+    b = SlotLayout(sq.Quantizer(4, 'k', 64), 30, 30, 96, 192, m=8, buffer_bits=8).breakdown()
+    assert b['S'] == 30 * 192 * 48 and b['SC'] == 30 * 192 * 2 * 2
+    assert b['KB'] == 30 * 8 * 96 and b['UB'] == 30 * 8 * 192
+    from statequant_amd.kernels import Mamba2SlotLayout
+    assert Mamba2SlotLayout('bf16', 96, 8, 128, 80, m=8, buffer_bits=8).breakdown()['S'] == 96 * 80 * 128 * 2
