@@ -22,10 +22,13 @@ FORMATS = {'int4-k-g64': (4, 'k', 64), 'int8-k-g32': (8, 'k', 32), 'int8-k-g128'
 VALUE_AXIS = {'int8-v-g32': (8, 'v', 32), 'int4-v-g32': (4, 'v', 32)}
 
 
-def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.float32, S0_scale=0.5, DV=None):
+def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.float32, S0_scale=0.5, DV=None,
+               shape_state=None, shape_token=None):
     DV = DV or D
     gen = torch.Generator().manual_seed(seed)
     S0 = torch.randn(B * HV, DV, D, generator=gen) * S0_scale                    # value-major
+    if shape_state is not None:
+        shape_state(S0.view(B, HV, DV, D))
     ker = PackedGDNState(S0.transpose(1, 2).to(DEV), quantizer(fmt), m=m, hv=HV, hk=HK, buffer_bits=bb,
                          out_dtype=torch.float32)
     ref = ST.GDNOracle(S0, fmt, m=m, hv=HV, hk=HK, buffer_bits=bb, auto_fold=False)
@@ -34,6 +37,8 @@ def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.flo
     scale = D ** -0.5
     for t in range(T):
         q, k, v, g, beta = gdn_token(gen, B, HV, HK, D, DV, dtype)
+        if shape_token is not None:
+            shape_token(q, k, v)
         slot = ker.n
         o = ker.step(q.reshape(B * HK, D).to(DEV), k.reshape(B * HK, D).to(DEV), v.reshape(B * HV, DV).to(DEV),
                      g.reshape(-1).to(DEV), beta.reshape(-1).to(DEV), scale).cpu()
@@ -376,6 +381,29 @@ def test_strided_inputs_like_the_serving_engine():
     lay.step(views, idx, q, k, v, o1, D ** -0.5, g=g, beta=beta)
     lay.step(v2, idx, q.contiguous(), k.contiguous(), v.contiguous(), o2, D ** -0.5, g=g, beta=beta)
     assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize('fmt', [(4, 'k', 32), (8, 'k', 64), (8, 'v', 32), (4, 'v', 16), 'bf16'])
+@pytest.mark.parametrize('bb', [8, 16])
+def test_zero_and_tiny_groups_through_the_fold(fmt, bb):
+    """States the re-quantization has to treat specially, kept that way through two folds: a head that stays all zero
+    (zero state, zero v: every scale at its floor, codes 0), a head at 1e-6 of the usual magnitude (scales in the fp16
+    subnormal range), and heads whose first 64 key columns stay zero (zero groups next to live ones; the keys of that
+    key head are zero there).  The packing of such states is pinned on the CPU against the reference's golden vectors;
+    this is the in-step fold."""
+    def shape_state(S):                                    # [B, HV, d_v, d_k]
+        S[:, 0] = 0.0
+        S[:, 1] *= 1e-6
+        S[:, 2:, :, :64] = 0.0
+
+    def shape_token(q, k, v):                              # q, k [B, HK, d_k]; v [B, HV, d_v]
+        v[:, 0] = 0.0
+        v[:, 1] *= 1e-6
+        k[:, 1, :64] = 0.0
+
+    m, T = 4, 9
+    tal = run_decode(fmt, m, bb, T=T, shape_state=shape_state, shape_token=shape_token)
+    check(tal, f'edge groups {fmt} buf{bb}', T, m)
 
 
 def test_stored_bytes():
