@@ -23,7 +23,7 @@ def kda_token(gen, B, H, DK, DV, dtype=torch.float32):
             -torch.nn.functional.softplus(r(B, H, DK)), torch.sigmoid(r(B, H)))
 
 
-def run_decode(fmt, m, bb, B=2, H=4, DK=128, DV=128, T=24, seed=1, dtype=torch.float32):
+def run_decode(fmt, m, bb, B=2, H=4, DK=128, DV=128, T=24, seed=1, dtype=torch.float32, shape_token=None):
     gen = torch.Generator().manual_seed(seed)
     S0 = torch.randn(B * H, DV, DK, generator=gen) * 0.5
     ker = PackedKDAState(S0.to(DEV), quantizer(fmt), m=m, hv=H, buffer_bits=bb, out_dtype=torch.float32)
@@ -32,6 +32,8 @@ def run_decode(fmt, m, bb, B=2, H=4, DK=128, DV=128, T=24, seed=1, dtype=torch.f
     tal = Tally()
     for t in range(T):
         q, k, v, g, beta = kda_token(gen, B, H, DK, DV, dtype)
+        if shape_token is not None:
+            shape_token(q, k, v, g, beta)
         slot = ker.n
         o = ker.step(q.to(DEV), k.to(DEV), v.to(DEV), g.to(DEV), beta.to(DEV)).cpu().reshape(B * H, DV)
         r = ref.step(q.reshape(B * H, DK), k.reshape(B * H, DK), v.reshape(B * H, DV), g.reshape(B * H, DK),
@@ -132,6 +134,21 @@ def test_bf16_control_tracks_the_fp32_recurrence(bb):
     st = ((ker.dequantize().cpu().view_as(S) - S).norm() / S.norm()).item()
     print(f'\nkda bf16 state buf{bb} vs fp32 recurrence: rel l2 {rel2:.2e}, state {st:.2e}')
     assert rel2 < (1.5e-2 if bb == 8 else 5e-3) and st < 1e-2
+
+
+@pytest.mark.parametrize('fmt,m,bb', [((4, 'k', 32), 8, 8), ((8, 'k', 64), 16, 16), ((4, 'v', 32), 16, 8), ('bf16', 16, 8)])
+def test_strong_per_channel_decays(fmt, m, bb):
+    """The reference's safe gate at its lower bound (tests/test_kda_kernels.py:33-41 there: g = -5 sigmoid(.)) on a
+    quarter of the channels at every token: over a full buffer of 16 the cumulative log decay reaches -80, so
+    exp(-G) of the buffered keys is near 5e34 and exp(G) near 2e-35 -- both still fp32 normal numbers -- and channels
+    that do not decay at all (g = 0) sit next to them."""
+    def shape_token(q, k, v, g, beta):                     # g [B, H, d_k]
+        g[..., 0::4] = -5.0
+        g[..., 1::4] = 0.0
+
+    T = 2 * m + 3
+    tal = run_decode(fmt, m, bb, T=T, shape_token=shape_token)
+    check(tal, f'kda strong decays {fmt} m={m} buf{bb}', T, m)
 
 
 def test_bf16_inputs():
