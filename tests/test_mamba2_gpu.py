@@ -118,6 +118,14 @@ def test_head_dim_80(DK, DV, H, G, fmt, m, bb):
     check(run_decode(fmt, m, bb, B=2, H=H, G=G, DK=DK, DV=DV, T=T), f'mamba2 {DK}x{DV} {fmt} m={m} buf{bb}', T, m)
 
 
+@pytest.mark.parametrize('fmt,m,bb', [((8, 'k', 128), 8, 8), ((4, 'k', 64), 4, 16), ((8, 'k', 32), 1, 8), ((4, 'k', 32), 16, 8),
+                                      ('bf16', 8, 8), ('bf16', 4, 16)])
+def test_d_state_256(fmt, m, bb):
+    """d_state 256, head_dim 64 (Falcon-H1's larger models): four 64-column pieces per state row."""
+    T = 4 if m == 1 else 34 if m == 16 else 20
+    check(run_decode(fmt, m, bb, B=2, H=4, G=2, DK=256, DV=64, T=T), f'mamba2 256x64 {fmt} m={m} buf{bb}', T, m)
+
+
 def test_large_gqa_one_group():
     """Mamba-2 / Falcon-H1 / Granite style: one B / C group shared by all 64 heads (tests/test_mamba2.py:115-132 there)."""
     check(run_decode((4, 'k', 64), 8, 8, B=2, H=64, G=1, DK=128, DV=64, T=12), 'mamba2 64 heads, 1 group', 12, 8)
@@ -207,6 +215,7 @@ def test_against_reference_golden_vectors(golden, name):
 # ---------------------------------------------------------------------------------------------------------------
 SHAPE = H, G, DK, DV = 8, 2, 128, 64
 NANO = 12, 2, 128, 80                                   # Nemotron-3-Nano's head shape, fewer heads
+WIDE = 4, 2, 256, 64                                    # d_state 256
 
 
 def _setup(fmt, m, bb, seed=0, shape=None):
@@ -226,7 +235,8 @@ def _setup(fmt, m, bb, seed=0, shape=None):
 
 
 @pytest.mark.parametrize('fmt,shape', [((8, 'k', 128), SHAPE), ((4, 'k', 32), SHAPE), ('bf16', SHAPE),
-                                       ((8, 'k', 128), NANO), ((4, 'k', 32), NANO), ((8, 'v', 16), NANO), ('bf16', NANO)],
+                                       ((8, 'k', 128), NANO), ((4, 'k', 32), NANO), ((8, 'v', 16), NANO), ('bf16', NANO),
+                                       ((8, 'k', 128), WIDE), ('bf16', WIDE)],
                          ids=lambda v: str(v).replace(' ', ''))
 @pytest.mark.parametrize('m,bb', [(8, 8), (2, 16)])
 def test_slot_step_matches_lockstep_per_sequence(fmt, shape, m, bb):
@@ -271,7 +281,7 @@ def test_slot_step_matches_lockstep_per_sequence(fmt, shape, m, bb):
     assert torch.equal(raw[keep], outside[keep])
 
 
-@pytest.mark.parametrize('shape', [SHAPE, NANO], ids=str)
+@pytest.mark.parametrize('shape', [SHAPE, NANO, WIDE], ids=str)
 def test_read_is_the_state_the_next_step_reads(shape):
     """read() + one textbook fp32 Mamba2 step == the kernel's next output (reference: tests/test_mamba2.py:273-300)."""
     m = 8
