@@ -51,6 +51,9 @@ WORKLOADS = {
     'gdn-bf16': ('gdn', 16, 128, 32, 16, 128, 128, 256, 24),
     'mamba2-int8-g128': ('mamba2', 8, 128, 128, 8, 128, 64, 128, 24),
     'kda-int4-g32': ('kda', 4, 32, 32, 32, 128, 128, 256, 24),
+    # Nemotron-3-Nano's layer (96 heads x head_dim 80 x d_state 128, 8 groups) and a d_state-256 layer (Falcon-H1 style)
+    'mamba2-nano-int8-g128': ('mamba2', 8, 128, 96, 8, 128, 80, 128, 24),
+    'mamba2-n256-int8-g128': ('mamba2', 8, 128, 128, 8, 256, 64, 64, 24),
     # the mixed-width GGA / STEP slot: bits = the plan's mean width, group = the FP8 window length
     'gga4-pw8': ('gga', 4, 8, 32, 16, 128, 128, 256, 24),
 }
