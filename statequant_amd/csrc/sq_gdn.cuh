@@ -32,11 +32,9 @@ struct GdnAddr {
     int32_t* np;
 };
 template <class T>
-__device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p) {
+__device__ __forceinline__ GdnAddr<T> gdn_addr(const GdnParams& p, const TileId& t, int32_t slot) {
     GdnAddr<T> a;
-    const TileId t = tile_id(p);
     a.b = t.b; a.h = t.h; a.hk = t.hk;
-    const int32_t slot = p.idx ? p.idx[a.b] : a.b;
     a.live = !(p.idx && slot <= 0);
     const uint32_t seq = a.live ? uint32_t(slot) : 0u;
     const uint32_t m = p.m, h = a.h, hk = a.hk;
@@ -71,17 +69,14 @@ struct GdnFront {
     uint32_t vr[T::NOWN];
     Window<T> win;
 };
+// The token's own operands: q, k, v and the gate.  Their addresses need the batch row only, not the slot, so they are
+// issued while the slot index is still on its way.
 template <class T>
-__device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& a, const LaneId& l, GdnFront<T>& f) {
+__device__ __forceinline__ void gdn_issue_inputs(const GdnParams& p, const TileId& a, const LaneId& l, GdnFront<T>& f) {
     constexpr int DK = T::DK, DV = T::DV;
-    const int m = p.m;
     const int gqa = p.gqa;
     const int hq = p.qk_per_key_head ? a.hk : a.h;
     const bool own_key = !p.qk_per_key_head && gqa > 1;          // the buffered key is the group's first head's
-    f.n = *a.np & (m - 1);
-    f.gcur = *a.gcp;
-    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
-    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(a.SCh), T::SC_ELEMS * 2, l.lane, f.st_sc);
     const uint32_t b = a.b, h = a.h;
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(hq) * DK);
     const void* kb = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(hq) * DK);
@@ -107,6 +102,17 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
         r = r < DV ? r : DV - 1;
         f.vr[t] = load_raw(vb, p.v_dt, r);
     }
+}
+
+// The slot's side: counters, the first blocks of the state tile, the scales, the live part of the decode buffer.
+template <class T>
+__device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& a, const LaneId& l, GdnFront<T>& f) {
+    constexpr int DV = T::DV;
+    const int m = p.m;
+    f.n = *a.np & (m - 1);
+    f.gcur = *a.gcp;
+    window_init<T>(lane_codes<T>(a.Sh, l), f.win);
+    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(a.SCh), T::SC_ELEMS * 2, l.lane, f.st_sc);
     // the buffer last, and only its live slots (the fill count is a scalar load issued first: by now it is here)
     const int nl = f.n > 0 ? f.n : 1;
     const int lm = l.lane < nl ? l.lane : nl - 1;
@@ -141,13 +147,16 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     constexpr int KT = KeyBuf<T>::KT;
     const bool own_key = !p.qk_per_key_head && gqa > 1;
     const LaneId l = lane_id<T>();
-    const GdnAddr<T> A = gdn_addr<T>(p);
+    const TileId tid = tile_id(p);
+    const int32_t slot = p.idx ? p.idx[tid.b] : tid.b;           // scalar load: on its way while the inputs are issued
+    GdnFront<T> F;
+    gdn_issue_inputs<T>(p, tid, l, F);
+    const GdnAddr<T> A = gdn_addr<T>(p, tid, slot);
     void* const outp = advance(p.out, p.out_dt, A.obase);
     if (!A.live) {                                                // padding row: zero output, touch nothing else
         for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
-    GdnFront<T> F;
     gdn_issue<T>(p, A, l, F);
     const int h = A.h;
     const int n = F.n;
