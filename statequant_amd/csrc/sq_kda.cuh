@@ -40,7 +40,29 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);          // scalar load: on its way while the inputs are issued
+    // the token's own operands first: their addresses need the batch row only, not the slot
+    uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
+    const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
+    const void* kb_ = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + h * DK);
+    const void* gb_ = advance(p.g, p.g_dt, uint64_t(b) * p.s_g + h * DK);
+#pragma unroll
+    for (int t = 0; t < T::NE; ++t) {
+        uint32_t e = l.lane + WAVE * t;
+        e = e < DK ? e : DK - 1;
+        qr[t] = load_raw(qb, p.q_dt, e);
+        kr_[t] = load_raw(kb_, p.k_dt, e);
+        gr[t] = load_raw(gb_, p.g_dt, e);
+    }
+    const uint32_t betar = load_raw_uniform(p.beta, p.beta_dt, uint64_t(b) * p.s_beta + h);
+    uint32_t vr[T::NOWN];
+    const void* vb = advance(p.v, p.v_dt, uint64_t(b) * p.s_v + h * DV);
+#pragma unroll
+    for (int t = 0; t < T::NOWN; ++t) {
+        uint32_t r = owned_row<T>(l, t);
+        r = r < DV ? r : DV - 1;
+        vr[t] = load_raw(vb, p.v_dt, r);
+    }
     void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
     if (p.idx && slot <= 0) {
         for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
@@ -61,35 +83,19 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     const uint8_t* lane_base = lane_codes<T>(Sh, l);
     const int cc = l.cg < T::LPR ? l.cg : T::LPR - 1;
 
-    // ---- issue every load: the state and the inputs first, the buffer last and only its live slots (the fill
-    // count is a scalar load issued first; by then it is here) ----
+    // ---- issue the slot's loads: the state first, the buffer last and only its live slots (the fill count is a
+    // scalar load issued first; by then it is here) ----
     const int n = *np & (m - 1);
     Window<T> win;
     window_init<T>(lane_base, win);
     Staged<T::SC_BYTES> st_sc;
     if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
-    uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     float gc[T::NE];
-    const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
-    const void* kb_ = advance(p.k, p.k_dt, uint64_t(b) * p.s_k + h * DK);
-    const void* gb_ = advance(p.g, p.g_dt, uint64_t(b) * p.s_g + h * DK);
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) {
         uint32_t e = l.lane + WAVE * t;
         e = e < DK ? e : DK - 1;
-        qr[t] = load_raw(qb, p.q_dt, e);
-        kr_[t] = load_raw(kb_, p.k_dt, e);
-        gr[t] = load_raw(gb_, p.g_dt, e);
         gc[t] = gch[e];
-    }
-    const uint32_t betar = load_raw_uniform(p.beta, p.beta_dt, uint64_t(b) * p.s_beta + h);
-    uint32_t vr[T::NOWN];
-    const void* vb = advance(p.v, p.v_dt, uint64_t(b) * p.s_v + h * DV);
-#pragma unroll
-    for (int t = 0; t < T::NOWN; ++t) {
-        uint32_t r = owned_row<T>(l, t);
-        r = r < DV ? r : DV - 1;
-        vr[t] = load_raw(vb, p.v_dt, r);
     }
     const int nl = n > 0 ? n : 1;
     uint16_t ubs_raw = 0;

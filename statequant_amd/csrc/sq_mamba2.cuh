@@ -36,34 +36,8 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
-    void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
-    if (p.idx && slot <= 0) {
-        for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
-        return;
-    }
-    const uint32_t seq = slot;
-
-    uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
-    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
-    BufAddr<T> buf;
-    buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
-    buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
-    buf.KBS = field(p.st.KBS, seq, p.st.sKBS, hk * um);
-    buf.UBS = field(p.st.UBS, seq, p.st.sUBS, h * um);
-    float* GBh = field(p.st.GB, seq, p.st.sGB, h * um);
-    float* gcp = field(p.st.GCUR, seq, p.st.sGC, h);
-    int32_t* np = field(p.st.NPTR, seq, p.st.sN, h);
-    const uint8_t* lane_base = lane_codes<T>(Sh, l);
-
-    // ---- issue every load: the state and the inputs first, the buffer last and only its live slots (the fill
-    // count is a scalar load issued first; by then it is here) ----
-    const int n = *np & (m - 1);
-    const float gcur = *gcp;
-    Window<T> win;
-    window_init<T>(lane_base, win);
-    Staged<T::SC_BYTES> st_sc;
-    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
+    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);          // scalar load: on its way while the inputs are issued
+    // the token's own operands first: their addresses need the batch row only, not the slot
     uint32_t cr[T::NE], br[T::NE];
     const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
     const void* bb = advance(p.B, p.B_dt, uint64_t(b) * p.s_B + hk * DK);
@@ -86,6 +60,33 @@ __global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params
         r = r < DV ? r : DV - 1;
         xr_raw[t] = load_raw(xb, p.x_dt, r);
     }
+    void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
+    if (p.idx && slot <= 0) {
+        for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
+        return;
+    }
+    const uint32_t seq = slot;
+
+    uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
+    uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
+    BufAddr<T> buf;
+    buf.KB = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
+    buf.UB = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
+    buf.KBS = field(p.st.KBS, seq, p.st.sKBS, hk * um);
+    buf.UBS = field(p.st.UBS, seq, p.st.sUBS, h * um);
+    float* GBh = field(p.st.GB, seq, p.st.sGB, h * um);
+    float* gcp = field(p.st.GCUR, seq, p.st.sGC, h);
+    int32_t* np = field(p.st.NPTR, seq, p.st.sN, h);
+    const uint8_t* lane_base = lane_codes<T>(Sh, l);
+
+    // ---- issue the slot's loads: the state first, the buffer last and only its live slots (the fill count is a
+    // scalar load issued first; by then it is here) ----
+    const int n = *np & (m - 1);
+    const float gcur = *gcp;
+    Window<T> win;
+    window_init<T>(lane_base, win);
+    Staged<T::SC_BYTES> st_sc;
+    if constexpr (!T::FLT) stage_load(reinterpret_cast<const uint8_t*>(SCh), T::SC_ELEMS * 2, l.lane, st_sc);
     const int nl = n > 0 ? n : 1;
     const int lm = l.lane < nl ? l.lane : nl - 1;
     uint16_t ubs_raw = 0;
