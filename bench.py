@@ -71,7 +71,7 @@ def describe_state(bits, group):
 
 # HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
 # over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
-MEASURED_TRAFFIC = {'gdn-int8-g128': 185326940, 'gga4-pw8': 184491520}
+MEASURED_TRAFFIC = {'gdn-int8-g128': 185332412, 'gga4-pw8': 184491520}
 
 
 def stored_bytes_per_slot(bits, group, hv, dk, dv):
