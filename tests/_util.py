@@ -40,7 +40,7 @@ class Tally:
 
     def __init__(self):
         self.worst_o = 0.0
-        self.buf_flips = self.buf_entries = 0
+        self.buf_flips = self.buf_entries = self.buf_scale_events = 0
         self.code_mism = self.code_n = self.scale_mism = 0
         self.code_far = 0                     # codes differing by more than one step
         self.worst_raw = 0.0
@@ -51,7 +51,15 @@ class Tally:
         self.worst_o = max(self.worst_o, ((o - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item())
 
     def entries(self, got, want):
-        self.buf_flips += (got != want).sum().item()
+        """Buffered vectors [..., d] as stored (dequantized).  A vector whose fp16 scale landed on the other side of a
+        rounding boundary (its absmax differs in the last fp32 bit) has most of its entries differ, each by less than
+        one code step; such a vector is counted once, as a scale event, not as d flipped entries."""
+        diff = got != want
+        per_vec = diff.sum(-1)
+        step = want.abs().amax(-1) / 127.0 * 1.01 + 1e-30
+        rescaled = (per_vec > 0.2 * want.shape[-1]) & ((got - want).abs().amax(-1) <= step)
+        self.buf_scale_events += int(rescaled.sum())
+        self.buf_flips += int(per_vec[~rescaled].sum())
         self.buf_entries += want.numel()
 
     def fold(self, codes, scales, ref, bits):
@@ -72,7 +80,8 @@ class Tally:
         return (f'[{tag}] max rel |o - o_oracle| {self.worst_o:.2e}; {self.folds} folds: codes differing '
                 f'{self.code_mism} of {self.code_n} ({100 * self.code_mism / max(self.code_n, 1):.5f}%), by more than '
                 f'1 LSB {self.code_far}, scales differing {self.scale_mism}; max rel |S - S_raw_oracle| '
-                f'{self.worst_raw:.2e}; buffer entries flipped {self.buf_flips} of {self.buf_entries}')
+                f'{self.worst_raw:.2e}; buffer entries flipped {self.buf_flips} of {self.buf_entries}, vectors with the scale one '
+                f'fp16 step off {self.buf_scale_events}')
 
 
 def code_diff(got, want, bits):

@@ -288,7 +288,7 @@ def _random_gga_configs(n, seed=77):
     return out
 
 
-@pytest.mark.parametrize('cfg', _random_gga_configs(16),
+@pytest.mark.parametrize('cfg', _random_gga_configs(16) + _random_gga_configs(12, seed=303),   # 303: bf16 tokens with exact ties
                          ids=lambda c: f"d{c['D']}-hv{c['HV']}hk{c['HK']}-{'pw%d' % c['m'] if c['pw'] else 'nopw'}-b{c['B']}")
 def test_random_configurations(cfg):
     """Seeded random plans (any mix of widths, also all pivots or none), head counts, window lengths (also not powers
@@ -324,6 +324,14 @@ def test_random_configurations(cfg):
         if pw:
             P, V, n = pk.window(Vp, live)
             assert torch.equal(n.cpu().long(), ora.n[li]), t
-            assert ((P.cpu() * nonp - ora.P[li]).abs() > 1e-6 * P.abs().amax().cpu()).float().mean().item() < 2e-3, t
+            # left factors: FP8 codes of beta k and of the propagated vectors.  An entry may sit on the other side of a
+            # rounding tie, one FP8 step away, never further.  With bf16 tokens exact ties are common (a code is
+            # 448 k_i / k_max, a ratio of two 8-bit significands), so more entries may do so than with fp32 tokens.
+            Pk, Po = P.cpu() * nonp, ora.P[li]
+            d = (Pk - Po).abs()
+            off = d > 1e-6 * Pk.abs().amax()
+            one_step = 0.126 * torch.maximum(Pk.abs(), Po.abs()) + Po.abs().amax(-1, keepdim=True) * (2.0 ** -9 / 448) * 1.01
+            assert not (off & (d > one_step)).any(), t
+            assert off.float().mean().item() < (3e-2 if cfg['bf16'] else 2e-3), t
             assert torch.equal(V.cpu() * nonp, ora.V[li] * nonp), t
     assert not Vp['blob'][0].any()

@@ -311,7 +311,8 @@ def _random_configs(n, seed=59, shapes=((128, 128), (96, 96), (64, 64), (128, 25
     return out
 
 
-@pytest.mark.parametrize('cfg', _random_configs(12) + _random_configs(6, seed=61, shapes=((64, 32), (128, 256))),
+@pytest.mark.parametrize('cfg', _random_configs(12) + _random_configs(6, seed=61, shapes=((64, 32), (128, 256)))
+                         + _random_configs(12, seed=101),     # 101: holds a buffered vector whose scale sits on an fp16 boundary
                          ids=lambda c: f"{c['fmt']}-{c['DK']}x{c['DV']}-m{c['m']}-h{c['H']}")
 def test_random_configurations(cfg):
     """Seeded random combinations of format, head shape, buffer, head count and input dtype; the task's bounds."""

@@ -17,6 +17,7 @@ def verdict(t, tag):
     assert t.code_far == 0
     assert t.code_mism <= 1e-4 * t.code_n, (t.code_mism, t.code_n)
     assert t.buf_flips <= 1e-3 * t.buf_entries, (t.buf_flips, t.buf_entries)
+    assert t.buf_scale_events * 64 <= 1e-2 * t.buf_entries, (t.buf_scale_events, t.buf_entries)   # <= 1 % of the vectors
 
 
 @pytest.mark.parametrize('fmt,m,bb', [((8, 'k', 128), 8, 8), ((4, 'k', 64), 8, 8), ((4, 'k', 32), 16, 16), ((8, 'v', 32), 8, 8),
