@@ -12,8 +12,10 @@
 
 namespace sq {
 
+// Occupancy target: four wavefronts per SIMD; the d_state-256 tile does not fit 128 registers, and asked for two it
+// is compiled at 234 without spills (asked for four the compiler gives up at 364, one wavefront per SIMD).
 template <class T>
-__global__ __launch_bounds__(WAVE, 4) void mamba2_step_kernel(const Mamba2Params p) {
+__global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(const Mamba2Params p) {
     using L = LdsPlan<T, 1, 1>;
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_cv = reinterpret_cast<float*>(lds + L::X);
