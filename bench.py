@@ -49,6 +49,7 @@ WORKLOADS = {
     'gdn-int4v-g32': ('gdn', 4, -32, 32, 16, 128, 128, 256, 24),
     'gdn-int8v-g32': ('gdn', 8, -32, 32, 16, 128, 128, 256, 24),
     'gdn-bf16': ('gdn', 16, 128, 32, 16, 128, 128, 256, 24),
+    'gdn-olmo-int4-g64': ('gdn', 4, 64, 30, 30, 96, 192, 256, 24),        # OLMo-Hybrid-7B's layer: 30 heads, 96 x 192
     'mamba2-int8-g128': ('mamba2', 8, 128, 128, 8, 128, 64, 128, 24),
     'kda-int4-g32': ('kda', 4, 32, 32, 32, 128, 128, 256, 24),
     # Nemotron-3-Nano's layer (96 heads x head_dim 80 x d_state 128, 8 groups) and a d_state-256 layer (Falcon-H1 style)
