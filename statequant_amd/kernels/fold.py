@@ -173,7 +173,10 @@ def _require_kernel(family, st):
 # ---------------------------------------------------------------------------------------------------------------
 # lockstep state
 # ---------------------------------------------------------------------------------------------------------------
-class PackedGDNState:
+from ._lockstep import LockstepState  # noqa: E402
+
+
+class PackedGDNState(LockstepState):
     """One layer's packed recurrent state and decode buffer for B sequences stepped in lockstep (fold.py:280-424).
 
     S            [BH, d_k, d_v] (or [B, H, d_k, d_v]) float state to start from
@@ -191,71 +194,37 @@ class PackedGDNState:
 
     def __init__(self, S, fmt, m=8, hv=None, hk=None, buffer_bits=8, out_dtype=torch.bfloat16,
                  block_v=None, warps=None, fused=None, fused_warps=None):
-        S = _flat(S)
-        _hip.require_gpu(S, 'PackedGDNState')
-        BH, DK, DV = S.shape
-        dev = S.device
-        self.BH, self.DK, self.DV, self.m = BH, DK, DV, m
+        from ._lockstep import describe_format, power_of_two
+        key_major = _flat(S)                                                     # [B * H, d_k, d_v]
+        _hip.require_gpu(key_major, 'PackedGDNState')
+        rows, dk, dv = key_major.shape
+        heads = hv if hv else rows
+        key_heads = hk if hk else heads
+        if heads % key_heads or rows % heads:
+            raise AssertionError(f'{rows} state rows, {heads} value heads, {key_heads} key heads do not divide')
+        if not power_of_two(m):
+            raise AssertionError('m must be a power of two')
+        if buffer_bits not in (8, 16):
+            raise AssertionError(f'buffer_bits {buffer_bits}: 8 (int8) or 16 (bf16)')
         self.fmt = packed_format(fmt)
         self.bits = _bits(self.fmt)
-        self.HV = hv or BH
-        self.HK = hk or self.HV
-        assert self.HV % self.HK == 0 and BH % self.HV == 0, (BH, self.HV, self.HK)
-        self.gqa, self.B = self.HV // self.HK, BH // self.HV
-        assert m >= 1 and m & (m - 1) == 0, 'm must be a power of two'
-        check_dims(self.fmt, DK, DV)
-        assert buffer_bits in (8, 16)
-        self.buffer_bits, self.qbuf = buffer_bits, buffer_bits == 8
-        self.axk = self.fmt is not None and self.fmt.axis == 'k'
-        self.group = self.fmt.group if self.fmt is not None else 32
-        self.fused = True
+        check_dims(self.fmt, dk, dv)
+        self.axk, self.group = describe_format(self.fmt, self.bits, default_group=32)
+        self.BH, self.B, self.HV, self.HK, self.gqa = rows, rows // heads, heads, key_heads, heads // key_heads
+        self.DK, self.DV, self.m = dk, dv, m
+        self.buffer_bits, self.qbuf, self.fused = buffer_bits, buffer_bits == 8, True
         _require_kernel('gdn', self)
-
-        codes, scales = pack(S, self.fmt)
-        self.codes, self.scales = codes.clone(), scales.clone()
-        bdt = torch.int8 if self.qbuf else torch.bfloat16
-        z = lambda *shape, dtype: torch.zeros(*shape, device=dev, dtype=dtype)      # noqa: E731
-        self.KB = z(self.B * self.HK, m, DK, dtype=bdt)
-        self.UB = z(BH, m, DV, dtype=bdt)
-        self.KBS = z(self.B * self.HK, m, dtype=torch.float16)
-        self.UBS = z(BH, m, dtype=torch.float16)
-        self.GB = z(BH, m, dtype=torch.float32)
-        self.GCUR = z(BH, dtype=torch.float32)
-        self.NPTR = z(self.B, self.HV, dtype=torch.int32)          # one counter copy per (sequence, value head)
-        self.O = z(BH, DV, dtype=out_dtype)
-        HV, HK = self.HV, self.HK
-        self._T = dict(S=self.codes, SC=self.scales, KB=self.KB, KBS=self.KBS, UB=self.UB, UBS=self.UBS, GB=self.GB,
-                       GCUR=self.GCUR, NPTR=self.NPTR)
-        # per-sequence strides of the lockstep layout: contiguous sequences
-        self._strides = (HV * self.codes[0].numel(), HV * self.scales[0].numel(), HK * m * DK, HK * m,
-                         HV * m * DV, HV * m, HV * m, HV)
-        self._lay = _hip.make_layout(self)
+        self._allocate(*pack(key_major, self.fmt), decay_shape=(), out_shape=(rows, dv), out_dtype=out_dtype)
+        self._T = self.T
 
     @torch.no_grad()
     def load(self, S):
         """Replace the state in place and empty the buffer."""
-        c, sc = pack(_flat(S), self.fmt)
-        self.codes.copy_(c)
-        self.scales.copy_(sc)
-        for t in (self.KB, self.UB, self.KBS, self.UBS, self.GB, self.GCUR, self.NPTR):
-            t.zero_()
+        self._reset(*pack(_flat(S), self.fmt))
 
     def dequantize(self):
         """The stored state S_0 (without the buffered tokens) as fp32 [BH, d_k, d_v]."""
         return unpack(self.codes, self.scales, self.fmt, self.DK)
-
-    @property
-    def n(self):
-        return int(self.NPTR.reshape(-1)[0])
-
-    def stored_bytes(self):
-        """Resident bytes: state payload + scales, the buffer, the decays (fold.py:371-378)."""
-        nb = lambda t: t.numel() * t.element_size()          # noqa: E731
-        per = dict(state=nb(self.codes) + (nb(self.scales) if self.fmt is not None else 0),   # bf16 state: no scales
-                   buffer=nb(self.KB) + nb(self.UB) + ((nb(self.KBS) + nb(self.UBS)) if self.qbuf else 0),
-                   decay=nb(self.GB) + nb(self.GCUR) + nb(self.NPTR))
-        per['total'] = sum(per.values())
-        return per
 
     def step(self, q, k, v, g, beta, scale):
         BH, HV, HK = self.BH, self.HV, self.HK

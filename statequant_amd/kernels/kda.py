@@ -17,43 +17,48 @@ import ctypes
 import torch
 
 from . import _hip
+from ._lockstep import LockstepState, describe_format, power_of_two
 from .fold import _bits, _require_kernel, pack_vk, packed_format, unpack_vk
 from .slots import SlotLayout, _order_ptr, field_table, slot_state, state_fields
 
 
+def _unit(x):
+    """Rows of x scaled to unit length, the epsilon inside the square root (as the kernels normalise q and k)."""
+    xf = x.float()
+    return xf * torch.rsqrt(xf.square().sum(dim=-1, keepdim=True) + 1e-6)
+
+
 def kda_recurrence(S, q, k, v, g, beta, scale=None):
-    """One plain fp32 KDA step on S [BH, d_v, d_k] (value-major, updated in place); q, k raw [BH, d_k] (normalised
-    here), v [BH, d_v], g [BH, d_k] log decay, beta [BH].  Returns o [BH, d_v] fp32 (kda.py:44-52)."""
-    scale = q.shape[-1] ** -0.5 if scale is None else scale
-    nrm = lambda x: x.float() / torch.sqrt((x.float() ** 2).sum(-1, keepdim=True) + 1e-6)     # noqa: E731
-    qn, kn = nrm(q) * scale, nrm(k)
-    S.mul_(torch.exp(g.float()).unsqueeze(1))
-    u = beta.float().unsqueeze(1) * (v.float() - torch.einsum('bvk,bk->bv', S, kn))
-    S.add_(u.unsqueeze(2) * kn.unsqueeze(1))
-    return torch.einsum('bvk,bk->bv', S, qn)
-
-
-def _check(fmt, dk, dv, hv, hk, m, buffer_bits):
-    """kda.py:55-64, with the power-of-two restriction on the head dims lifted."""
-    assert dk >= 16 and dk % 2 == 0 and dv >= 16, (dk, dv)
-    assert hk == hv, 'KDA: key heads must equal value heads'
-    assert m >= 1 and m & (m - 1) == 0 and m <= 32, 'm must be a power of two <= 32'
-    assert buffer_bits in (8, 16), buffer_bits
-    if fmt is not None:
-        g = fmt.group
-        assert g >= 2 and g & (g - 1) == 0, f'group {g} must be a power of two'
-        assert (dk if fmt.axis == 'k' else dv) % g == 0, f'group {g} must divide d_{fmt.axis} ({dk}, {dv})'
-        assert fmt.axis == 'v' or dk // g <= 64, 'at most 64 key groups'
+    """The unquantized per-channel gated delta rule, one token, on S [BH, d_v, d_k] in place (kda.py:44-52): every key
+    channel decays by exp(g), then the delta write beta (v - S k) k^T, then o = S q.  q, k raw [BH, d_k]; v [BH, d_v];
+    g [BH, d_k] log decay; beta [BH].  Returns o [BH, d_v] fp32."""
+    kn = _unit(k)
+    qn = _unit(q) * (q.shape[-1] ** -0.5 if scale is None else scale)
+    S *= g.float().exp()[:, None, :]
+    err = v.float() - (S * kn[:, None, :]).sum(-1)
+    S += (beta.float()[:, None] * err)[:, :, None] * kn[:, None, :]
+    return (S * qn[:, None, :]).sum(-1)
 
 
 def _common(st, fmt, hv, hk, dk, dv, m, buffer_bits):
+    """Geometry and format attributes of a KDA state / layout (kda.py:55-64; head dims need not be powers of two)."""
     st.fmt = packed_format(fmt)
     st.bits = _bits(st.fmt)
+    st.axk, st.group = describe_format(st.fmt, st.bits, default_group=16)
+    if hk != hv:
+        raise AssertionError('KDA: key heads must equal value heads')
+    if not (power_of_two(m) and m <= 32):
+        raise AssertionError('m must be a power of two <= 32')
+    if buffer_bits not in (8, 16):
+        raise AssertionError(f'buffer_bits {buffer_bits}: 8 (int8) or 16 (bf16)')
+    assert dk >= 16 and dk % 2 == 0 and dv >= 16, (dk, dv)
+    if st.fmt is not None:
+        axis_len = dk if st.axk else dv
+        assert st.group >= 2 and power_of_two(st.group), f'group {st.group} must be a power of two'
+        assert axis_len % st.group == 0, f'group {st.group} must divide d_{st.fmt.axis} ({dk}, {dv})'
+        assert not st.axk or dk // st.group <= 64, 'at most 64 key groups'
     st.HV, st.HK, st.DK, st.DV, st.m = hv, hk, dk, dv, m
-    _check(st.fmt, dk, dv, hv, hk, m, buffer_bits)
     st.buffer_bits, st.qbuf = buffer_bits, buffer_bits == 8
-    st.axk = st.fmt is not None and st.fmt.axis == 'k'
-    st.group = st.fmt.group if st.fmt is not None else 16
 
 
 def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_stride, order=None):
@@ -76,7 +81,7 @@ def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_s
     return out
 
 
-class PackedKDAState:
+class PackedKDAState(LockstepState):
     """One KDA layer's packed state and decode buffer for B sequences in lockstep (kda.py:208-282).
 
     S [B, H, d_v, d_k] (or [B*H, d_v, d_k]); fmt, m, hv (= H), buffer_bits as ``PackedGDNState``.
@@ -85,67 +90,25 @@ class PackedKDAState:
 
     def __init__(self, S, fmt, m=8, hv=None, buffer_bits=8, out_dtype=torch.bfloat16, sbv=None, fbv=None,
                  warps=None):
-        S = S.float().reshape(-1, S.shape[-2], S.shape[-1])
-        _hip.require_gpu(S, 'PackedKDAState')
-        BH, DV, DK = S.shape
-        hv = hv or BH
-        assert BH % hv == 0
-        _common(self, fmt, hv, hv, DK, DV, m, buffer_bits)
+        flat = S.float().flatten(0, -3) if S.dim() > 3 else S.float()           # [B * H, d_v, d_k]
+        _hip.require_gpu(flat, 'PackedKDAState')
+        heads = hv if hv else flat.shape[0]
+        if flat.shape[0] % heads:
+            raise AssertionError(f'{flat.shape[0]} state rows are not a multiple of {heads} heads')
+        _common(self, fmt, heads, heads, flat.shape[2], flat.shape[1], m, buffer_bits)
         _require_kernel('kda', self)
-        self.BH, self.B = BH, BH // hv
-        dev = S.device
-        c, s = pack_vk(S, self.fmt)
-        bdt = torch.int8 if self.qbuf else torch.bfloat16
-        self.T = dict(S=c.clone(), SC=s.clone(),
-                      KB=torch.zeros(BH, m, DK, device=dev, dtype=bdt),
-                      UB=torch.zeros(BH, m, DV, device=dev, dtype=bdt),
-                      KBS=torch.zeros(BH, m, device=dev, dtype=torch.float16),
-                      UBS=torch.zeros(BH, m, device=dev, dtype=torch.float16),
-                      GB=torch.zeros(BH, m, DK, device=dev), GCUR=torch.zeros(BH, DK, device=dev),
-                      NPTR=torch.zeros(self.B, hv, device=dev, dtype=torch.int32))
-        self.O = torch.zeros(self.B, hv, DV, device=dev, dtype=out_dtype)
-        T = self.T
-        self._strides = (hv * T['S'][0].numel(), hv * T['SC'][0].numel(), hv * m * DK, hv * m, hv * m * DV, hv * m,
-                         hv * m * DK, hv * DK)
-        self._lay = _hip.make_layout(self)
-
-    def __getattr__(self, name):
-        T = self.__dict__.get('T')
-        if T is not None and name in T:
-            return T[name]
-        raise AttributeError(name)
-
-    @property
-    def codes(self):
-        return self.T['S']
-
-    @property
-    def scales(self):
-        return self.T['SC']
-
-    @property
-    def n(self):
-        return int(self.T['NPTR'].reshape(-1)[0])
+        self.BH, self.B = flat.shape[0], flat.shape[0] // heads
+        self._allocate(*pack_vk(flat, self.fmt), decay_shape=(self.DK,), out_shape=(self.B, heads, self.DV),
+                       out_dtype=out_dtype)                                     # one decay per key channel
 
     @torch.no_grad()
     def load(self, S):
-        c, s = pack_vk(S.float().reshape(self.BH, self.DV, self.DK), self.fmt)
-        self.T['S'].copy_(c)
-        self.T['SC'].copy_(s)
-        for k in ('KB', 'UB', 'KBS', 'UBS', 'GB', 'GCUR', 'NPTR'):
-            self.T[k].zero_()
+        """Replace the state (any shape that flattens to [B * H, d_v, d_k]) and empty the buffer."""
+        self._reset(*pack_vk(S.float().reshape(self.BH, self.DV, self.DK), self.fmt))
 
     def dequantize(self):
-        return unpack_vk(self.T['S'], self.T['SC'], self.fmt, self.DK)
-
-    def stored_bytes(self):
-        nb = lambda t: t.numel() * t.element_size()          # noqa: E731
-        T = self.T
-        per = dict(state=nb(T['S']) + (nb(T['SC']) if self.fmt is not None else 0),          # bf16 state: no scales
-                   buffer=nb(T['KB']) + nb(T['UB']) + ((nb(T['KBS']) + nb(T['UBS'])) if self.qbuf else 0),
-                   decay=nb(T['GB']) + nb(T['GCUR']) + nb(T['NPTR']))
-        per['total'] = sum(per.values())
-        return per
+        """The stored state (without the buffered tokens), fp32 [B * H, d_v, d_k]."""
+        return unpack_vk(self.codes, self.scales, self.fmt, self.DK)
 
     def step(self, q, k, v, g, beta, scale=None):
         Bn, HV, DK, DV = self.B, self.HV, self.DK, self.DV

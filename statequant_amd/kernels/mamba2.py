@@ -16,57 +16,58 @@ import ctypes
 import torch
 
 from . import _hip
+from ._lockstep import LockstepState, describe_format, power_of_two
 from .fold import _bits, _require_kernel, pack_vk, packed_format, unpack_vk
 from .slots import SlotLayout, _order_ptr, field_table, slot_state, state_fields
 
 
-def _gate(dt, A, dt_bias=None, dt_softplus=False, dt_limit=None):
-    """dt (raw [B, H]) -> (dt, log decay g = A dt), fp32, as the kernel (mamba2.py:45-54)."""
-    dt = dt.float()
-    if dt_bias is not None:
-        dt = dt + dt_bias.float()
+def _activated_dt(dt, A, dt_bias, dt_softplus, dt_limit):
+    """Raw dt [B, H] -> (dt after bias / softplus / clamp, log decay A dt), fp32 -- the kernel's gate in torch
+    (mamba2.py:45-54).  softplus switches to the identity above 20, as the kernels do."""
+    t = dt.float() if dt_bias is None else dt.float() + dt_bias.float()
     if dt_softplus:
-        dt = torch.where(dt <= 20., torch.log(1. + torch.exp(dt)), dt)
-    if dt_limit is not None and tuple(dt_limit) != (0., float('inf')):
-        dt = dt.clamp(dt_limit[0], dt_limit[1])
-    return dt, A.float() * dt
+        t = torch.where(t > 20.0, t, torch.log(torch.exp(t.clamp(max=20.0)) + 1.0))
+    lo, hi = (0.0, float('inf')) if dt_limit is None else (float(dt_limit[0]), float(dt_limit[1]))
+    if (lo, hi) != (0.0, float('inf')):
+        t = torch.clamp(t, min=lo, max=hi)
+    return t, t * A.float()
 
 
 def mamba2_recurrence(S, x, dt, B, C, A, D=None, dt_bias=None, dt_softplus=False, dt_limit=None):
-    """One plain fp32 Mamba2 step on S [B, H, d_v, d_k] (updated in place); x [B, H, d_v], dt [B, H], B / C
-    [B, G, d_k], A / D / dt_bias [H].  Returns y [B, H, d_v] fp32 (mamba2.py:57-70)."""
-    H, G = dt.shape[1], B.shape[1]
-    dt, g = _gate(dt, A, dt_bias, dt_softplus, dt_limit)
-    Bh = B.float().repeat_interleave(H // G, 1)
-    Ch = C.float().repeat_interleave(H // G, 1)
-    u = dt.unsqueeze(-1) * x.float()
-    S.mul_(torch.exp(g)[..., None, None]).add_(u.unsqueeze(-1) * Bh.unsqueeze(-2))
-    y = torch.einsum('bhvk,bhk->bhv', S, Ch)
-    if D is not None:
-        y = y + D.float()[:, None] * x.float()
-    return y
-
-
-def _check_dims(fmt, dk, dv):
-    assert dk >= 16 and dk % 2 == 0, dk
-    if fmt is not None:
-        g = fmt.group
-        assert g & (g - 1) == 0, f'group {g} must be a power of two'
-        assert (dk if fmt.axis == 'k' else dv) % g == 0, f'group {g} must divide d_{fmt.axis} ({dk}, {dv})'
+    """The unquantized recurrence, one token, on S [B, H, d_v, d_k] in place (mamba2.py:57-70):
+    S <- exp(A dt) S + (dt x) B^T, y = S C + D x.  x [B, H, d_v], dt [B, H], B / C [B, G, d_k] (G groups, each shared
+    by H / G heads), A / D / dt_bias [H].  Returns y [B, H, d_v] fp32."""
+    heads, groups = dt.shape[1], B.shape[1]
+    step, log_decay = _activated_dt(dt, A, dt_bias, dt_softplus, dt_limit)
+    share = heads // groups
+    key = torch.repeat_interleave(B.float(), share, dim=1)              # [B, H, d_k]
+    query = torch.repeat_interleave(C.float(), share, dim=1)
+    xf = x.float()
+    S *= log_decay.exp()[:, :, None, None]
+    S += torch.einsum('bhv,bhk->bhvk', step[..., None] * xf, key)
+    y = (S * query[:, :, None, :]).sum(-1)
+    return y if D is None else y + xf * D.float().view(1, heads, 1)
 
 
 def _common(st, fmt, hv, hk, dk, dv, m, buffer_bits):
+    """Geometry and format attributes of a Mamba2 state / layout (names as the launch helpers read them)."""
     st.fmt = packed_format(fmt)
     st.bits = _bits(st.fmt)
-    st.HV, st.HK, st.DK, st.DV, st.m = hv, hk, dk, dv, m
-    assert hv % hk == 0, (hv, hk)
-    st.gqa = hv // hk
-    assert m >= 1 and m & (m - 1) == 0 and m <= 32, 'm must be a power of two <= 32'
-    _check_dims(st.fmt, dk, dv)
-    assert buffer_bits in (8, 16)
+    st.axk, st.group = describe_format(st.fmt, st.bits, default_group=16)
+    if hv % hk:
+        raise AssertionError(f'{hv} heads do not split into {hk} groups')
+    if not (power_of_two(m) and m <= 32):
+        raise AssertionError('m must be a power of two <= 32')
+    if buffer_bits not in (8, 16):
+        raise AssertionError(f'buffer_bits {buffer_bits}: 8 (int8) or 16 (bf16)')
+    assert dk >= 16 and dk % 2 == 0, dk
+    if st.fmt is not None:
+        axis_len = dk if st.axk else dv
+        assert power_of_two(st.group), f'group {st.group} must be a power of two'
+        assert axis_len % st.group == 0, f'group {st.group} must divide d_{st.fmt.axis} ({dk}, {dv})'
+    st.HV, st.HK, st.gqa = hv, hk, hv // hk
+    st.DK, st.DV, st.m = dk, dv, m
     st.buffer_bits, st.qbuf = buffer_bits, buffer_bits == 8
-    st.axk = st.fmt is not None and st.fmt.axis == 'k'
-    st.group = st.fmt.group if st.fmt is not None else 16
 
 
 def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx, T, strides, nptr_stride,
@@ -94,7 +95,7 @@ def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limi
     return out
 
 
-class PackedMamba2State:
+class PackedMamba2State(LockstepState):
     """One Mamba2 layer's packed state and decode buffer for B sequences in lockstep (mamba2.py:259-335).
 
     S [B, H, d_v, d_k] (or [B*H, d_v, d_k]); fmt, m, hv (= H), hk (= G groups), buffer_bits as ``PackedGDNState``.
@@ -103,68 +104,26 @@ class PackedMamba2State:
 
     def __init__(self, S, fmt, m=8, hv=None, hk=None, buffer_bits=8, out_dtype=torch.bfloat16, sbv=None, fbv=None,
                  warps=None):
-        S = S.float().reshape(-1, S.shape[-2], S.shape[-1])
-        _hip.require_gpu(S, 'PackedMamba2State')
-        BH, DV, DK = S.shape
-        hv = hv or BH
-        hk = hk or hv
-        assert BH % hv == 0
-        _common(self, fmt, hv, hk, DK, DV, m, buffer_bits)
+        flat = S.float().flatten(0, -3) if S.dim() > 3 else S.float()           # [B * H, d_v, d_k]
+        _hip.require_gpu(flat, 'PackedMamba2State')
+        heads = hv if hv else flat.shape[0]
+        groups = hk if hk else heads
+        if flat.shape[0] % heads:
+            raise AssertionError(f'{flat.shape[0]} state rows are not a multiple of {heads} heads')
+        _common(self, fmt, heads, groups, flat.shape[2], flat.shape[1], m, buffer_bits)
         _require_kernel('mamba2', self)
-        self.BH, self.B = BH, BH // hv
-        dev = S.device
-        c, s = pack_vk(S, self.fmt)
-        bdt = torch.int8 if self.qbuf else torch.bfloat16
-        self.T = dict(S=c.clone(), SC=s.clone(),
-                      KB=torch.zeros(self.B * hk, m, DK, device=dev, dtype=bdt),
-                      UB=torch.zeros(BH, m, DV, device=dev, dtype=bdt),
-                      KBS=torch.zeros(self.B * hk, m, device=dev, dtype=torch.float16),
-                      UBS=torch.zeros(BH, m, device=dev, dtype=torch.float16),
-                      GB=torch.zeros(BH, m, device=dev), GCUR=torch.zeros(BH, device=dev),
-                      NPTR=torch.zeros(self.B, hv, device=dev, dtype=torch.int32))
-        self.O = torch.zeros(self.B, hv, DV, device=dev, dtype=out_dtype)
-        T = self.T
-        self._strides = (hv * T['S'][0].numel(), hv * T['SC'][0].numel(), hk * m * DK, hk * m, hv * m * DV, hv * m,
-                         hv * m, hv)
-        self._lay = _hip.make_layout(self)
-
-    def __getattr__(self, name):
-        T = self.__dict__.get('T')
-        if T is not None and name in T:
-            return T[name]
-        raise AttributeError(name)
-
-    @property
-    def codes(self):
-        return self.T['S']
-
-    @property
-    def scales(self):
-        return self.T['SC']
-
-    @property
-    def n(self):
-        return int(self.T['NPTR'].reshape(-1)[0])
+        self.BH, self.B = flat.shape[0], flat.shape[0] // heads
+        self._allocate(*pack_vk(flat, self.fmt), decay_shape=(), out_shape=(self.B, heads, self.DV),
+                       out_dtype=out_dtype)
 
     @torch.no_grad()
     def load(self, S):
-        c, s = pack_vk(S.float().reshape(self.BH, self.DV, self.DK), self.fmt)
-        self.T['S'].copy_(c)
-        self.T['SC'].copy_(s)
-        for k in ('KB', 'UB', 'KBS', 'UBS', 'GB', 'GCUR', 'NPTR'):
-            self.T[k].zero_()
+        """Replace the state (any shape that flattens to [B * H, d_v, d_k]) and empty the buffer."""
+        self._reset(*pack_vk(S.float().reshape(self.BH, self.DV, self.DK), self.fmt))
 
     def dequantize(self):
-        return unpack_vk(self.T['S'], self.T['SC'], self.fmt, self.DK)
-
-    def stored_bytes(self):
-        nb = lambda t: t.numel() * t.element_size()          # noqa: E731
-        T = self.T
-        per = dict(state=nb(T['S']) + (nb(T['SC']) if self.fmt is not None else 0),          # bf16 state: no scales
-                   buffer=nb(T['KB']) + nb(T['UB']) + ((nb(T['KBS']) + nb(T['UBS'])) if self.qbuf else 0),
-                   decay=nb(T['GB']) + nb(T['GCUR']) + nb(T['NPTR']))
-        per['total'] = sum(per.values())
-        return per
+        """The stored state (without the buffered tokens), fp32 [B * H, d_v, d_k]."""
+        return unpack_vk(self.codes, self.scales, self.fmt, self.DK)
 
     def step(self, x, dt, B, C, A, D=None, dt_bias=None, dt_softplus=False, dt_limit=None):
         Bn, HV, HK = self.B, self.HV, self.HK
