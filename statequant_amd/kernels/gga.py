@@ -38,17 +38,19 @@ class GGAPlan:
 
 
 def head_bytes(b, dk, dv, group=32):
-    """Stored bytes of one head at width b: codes + row factors (2 bit: group rows) + column factors; fp16 pivots
-    (vllm_gga.py:174-180)."""
+    """Bytes one head occupies at width b (vllm_gga.py:174-180): an fp16 pivot stores its dk x dv values; a coded head
+    stores b-bit codes plus fp16 factors -- one row factor per row (2-bit heads: one per row and group of `group`
+    value columns) and one column factor per column."""
+    values = dk * dv
     if b == 16:
-        return 2 * dk * dv
-    if b == 2:
-        return dk * dv // 4 + 2 * dk * (dv // group) + 2 * dv
-    return dk * dv * b // 8 + 2 * dk + 2 * dv
+        return values * 2
+    row_factors = dk * (dv // group) if b == 2 else dk
+    return (values * b) // 8 + 2 * (row_factors + dv)
 
 
-def _al(n):
-    return -(-n // _ALIGN) * _ALIGN
+def _al(nbytes):
+    """nbytes rounded up to the slot alignment."""
+    return (nbytes + _ALIGN - 1) // _ALIGN * _ALIGN
 
 
 class GGAPacked:
@@ -57,38 +59,43 @@ class GGAPacked:
     per_layer = True
 
     def __init__(self, method, hv, hk, dk, dv, pw=False, m=8):
-        assert dk & (dk - 1) == 0 and dv & (dv - 1) == 0 and dv % 32 == 0, (dk, dv)
-        assert method.group == 32, 'two-bit heads keep one row factor per 32 value columns'
-        self.method, self.HV, self.HK, self.DK, self.DV = method, hv, hk, dk, dv
-        self.pw, self.m, self.gqa = pw, m, hv // hk
-        assert hv % hk == 0
+        for d in (dk, dv):
+            if d & (d - 1):
+                raise AssertionError((dk, dv))
+        assert dv % 32 == 0, (dk, dv)
+        assert hv % hk == 0, (hv, hk)
+        self.method = method
+        self.HV, self.HK, self.gqa = hv, hk, hv // hk
+        self.DK, self.DV = dk, dv
+        self.pw, self.m = pw, m
+        # per layer: where each head starts inside the slot (after the 16 counter bytes), its width, the impact factors
         self.tables, self.bytes_per_layer = {}, {}
-        for layer, (b, w) in method.plan.items():
-            b = [int(x) for x in b]
-            assert len(b) == hv and set(b) <= set(WIDTHS), b
-            assert tuple(w.shape) == (hv, dk), (tuple(w.shape), hv, dk)
-            offs, off = [], 16                                  # counters first
-            for x in b:
-                offs.append(off)
-                off += _al(head_bytes(x, dk, dv, method.group))
-            self.tables[layer] = (offs, b, w)
-            self.bytes_per_layer[layer] = off
+        for layer, (widths, impact) in method.plan.items():
+            widths = [int(x) for x in widths]
+            assert len(widths) == hv and all(x in WIDTHS for x in widths), (layer, widths)
+            sizes = [_al(head_bytes(x, dk, dv, method.group)) for x in widths]
+            starts = [16 + sum(sizes[:i]) for i in range(hv)]
+            self.tables[layer] = (starts, widths, impact)
+            self.bytes_per_layer[layer] = 16 + sum(sizes)
+        # the windows follow the largest layer's heads: per head m left and m right FP8 vectors and their 2 m scales
         self.QOFF = _al(max(self.bytes_per_layer.values()))
-        self.QSZ = m * (dk + dv + 8)
-        self.nbytes = self.QOFF + (hv * self.QSZ if pw else 0)
+        self.QSZ = m * (dk + dv) + 2 * m * 4
+        self.nbytes = self.QOFF + hv * self.QSZ * int(bool(pw))
         self._dev = {}
 
     def __repr__(self):
-        return (f'GGAPacked({self.method.name}{"+PW-S%d" % self.m if self.pw else ""}, hv={self.HV}, hk={self.HK}, '
-                f'dk={self.DK}, dv={self.DV}, {self.nbytes} B/slot = max over layers; mean '
-                f'{self.bits_per_value():.3f} b/value)')
+        window = f'+PW-S{self.m}' if self.pw else ''
+        return (f'GGAPacked({self.method.name}{window}, hv={self.HV}, hk={self.HK}, dk={self.DK}, dv={self.DV}, '
+                f'{self.nbytes} B/slot = max over layers; mean {self.bits_per_value():.3f} b/value)')
 
     def bits_per_value(self):
         """Mean stored bits per state value over the layers (without the 16-byte counters), window included."""
-        n = self.HV * self.DK * self.DV
-        st = sum(sum(head_bytes(x, self.DK, self.DV, self.method.group) for x in t[1]) for t in self.tables.values())
-        q = self.HV * self.QSZ * len(self.tables) if self.pw else 0
-        return 8 * (st + q) / (n * len(self.tables))
+        layers = len(self.tables)
+        head_total = 0
+        for _, widths, _ in self.tables.values():
+            head_total += sum(head_bytes(x, self.DK, self.DV, self.method.group) for x in widths)
+        window_total = layers * self.HV * self.QSZ if self.pw else 0
+        return 8.0 * (head_total + window_total) / (layers * self.HV * self.DK * self.DV)
 
     def supported(self):
         """Whether ``libsqhip.so`` has kernels for these head dims and window length."""
@@ -101,13 +108,14 @@ class GGAPacked:
         return self
 
     def _plan(self, layer, dev):
-        key = (layer, dev)
-        if key not in self._dev:
-            offs, b, w = self.tables[layer]
-            self._dev[key] = (torch.tensor(offs, dtype=torch.int32, device=dev),
-                              torch.tensor(b, dtype=torch.int32, device=dev),
-                              w.to(dev, torch.float32).contiguous())
-        return self._dev[key]
+        """(head offsets int32 [HV], widths int32 [HV], impact factors fp32 [HV, d_k]) of a layer on device dev."""
+        cached = self._dev.get((layer, dev))
+        if cached is None:
+            starts, widths, impact = self.tables[layer]
+            as_i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=dev)      # noqa: E731
+            cached = (as_i32(starts), as_i32(widths), impact.to(device=dev, dtype=torch.float32).contiguous())
+            self._dev[(layer, dev)] = cached
+        return cached
 
     def views(self, blob):
         assert blob.dtype == torch.uint8 and blob.dim() == 2 and blob.shape[1] >= self.nbytes
@@ -177,33 +185,40 @@ class GGAPacked:
     def window(self, views, idx):
         """The queued pairs of slots idx as reconstructed fp32 (P [n, m, HV, d_k], V [n, m, HV, d_v]) in ring order
         from the oldest, and the counts n [n]; dead entries zeroed."""
-        li = idx.long()
-        blob = views['blob'][li]
         m, HV, DK, DV = self.m, self.HV, self.DK, self.DV
-        ct = blob[:, :16].view(torch.int32)
-        n, hd = ct[:, 0], ct[:, 1]
-        Qb = blob[:, self.QOFF:self.QOFF + HV * self.QSZ].reshape(-1, HV, self.QSZ)
-        Pc = Qb[..., :m * DK].contiguous().view(torch.float8_e4m3fn).float().view(-1, HV, m, DK)
-        Vc = Qb[..., m * DK:m * (DK + DV)].contiguous().view(torch.float8_e4m3fn).float().view(-1, HV, m, DV)
-        sc = Qb[..., m * (DK + DV):].contiguous().view(torch.float32).view(-1, HV, 2, m)
-        Pf = Pc * sc[:, :, 0, :, None]
-        Vf = Vc * sc[:, :, 1, :, None]
-        order = (hd[:, None] + torch.arange(m, device=li.device)[None, :]) % m          # oldest first
-        Pf = torch.gather(Pf, 2, order[:, None, :, None].expand(-1, HV, -1, DK)).transpose(1, 2)
-        Vf = torch.gather(Vf, 2, order[:, None, :, None].expand(-1, HV, -1, DV)).transpose(1, 2)
-        live = (torch.arange(m, device=li.device)[None, :] < n[:, None])[:, :, None, None]
-        return torch.where(live, Pf, 0.), torch.where(live, Vf, 0.), n
+        rows = views['blob'].index_select(0, idx.long())
+        counters = rows[:, :8].contiguous().view(torch.int32)                  # n, ring position of the oldest
+        count, oldest = counters[:, 0], counters[:, 1]
+        win = rows[:, self.QOFF:self.QOFF + HV * self.QSZ].unflatten(1, (HV, self.QSZ))
+
+        def fp8_block(lo, width):                                              # [n, HV, m, width] decoded codes
+            raw = win[:, :, lo:lo + m * width].contiguous()
+            return raw.view(torch.float8_e4m3fn).to(torch.float32).unflatten(2, (m, width))
+
+        scales = win[:, :, m * (DK + DV):].contiguous().view(torch.float32).unflatten(2, (2, m))
+        left = fp8_block(0, DK) * scales[:, :, 0].unsqueeze(-1)
+        right = fp8_block(m * DK, DV) * scales[:, :, 1].unsqueeze(-1)
+        # ring order -> age order, then entries beyond the count are dropped
+        steps = torch.arange(m, device=rows.device)
+        ring = torch.remainder(oldest.unsqueeze(1) + steps, m)                  # [n, m]
+        alive = (steps.unsqueeze(0) < count.unsqueeze(1)).view(-1, m, 1, 1)
+
+        def by_age(x):                                                          # [n, HV, m, d] -> [n, m, HV, d]
+            picked = torch.stack([x[i, :, ring[i]] for i in range(x.shape[0])]) if x.shape[0] else x
+            return picked.transpose(1, 2) * alive
+
+        return by_age(left), by_age(right), count
 
     @torch.no_grad()
     def read(self, views, idx, layer=None):
         """Logical state (stored + window), value-major fp32 [P, HV, d_v, d_k]."""
-        S = self.stored(views, idx, layer)
-        if self.pw and idx.shape[0]:
-            P, V, _ = self.window(views, idx)
-            _, bits, _ = self._plan(layer, idx.device)
-            nonp = (bits != 16)[None, :, None, None].float()
-            S = S + torch.einsum('bmhk,bmhv->bhkv', P, V) * nonp
-        return S.transpose(-1, -2)
+        state = self.stored(views, idx, layer)                                 # [P, HV, d_k, d_v]
+        if self.pw and idx.numel():
+            left, right, _ = self.window(views, idx)
+            widths = self._plan(layer, idx.device)[1]
+            coded = (widths != 16).to(state.dtype).view(1, -1, 1, 1)           # pivots keep no window
+            state = state + coded * torch.einsum('pmhk,pmhv->phkv', left, right)
+        return state.mT
 
     @torch.no_grad()
     def write(self, views, idx, S, layer=None):
