@@ -20,16 +20,16 @@ FP16_TINY = 2.0 ** -24          # smallest fp16 subnormal: floor of a stored fp1
 
 
 class Format:
-    """A storage format for one state tensor: ``fake`` (store/load round trip) and ``bits_per_value``."""
+    """What every storage format offers: ``fake(S)`` -- S after one store / load round trip, same shape and dtype --
+    and ``bits_per_value(d_k, d_v)``, payload and side information together.  Calling a format applies ``fake``."""
 
     def fake(self, S: torch.Tensor) -> torch.Tensor:
-        raise NotImplementedError
+        raise NotImplementedError(type(self).__name__)
 
     def bits_per_value(self, d_k: int, d_v: int) -> float:
-        raise NotImplementedError
+        raise NotImplementedError(type(self).__name__)
 
-    def __call__(self, S: torch.Tensor) -> torch.Tensor:
-        return self.fake(S)
+    __call__ = lambda self, S: self.fake(S)                 # noqa: E731
 
 
 @dataclass(frozen=True)
@@ -81,12 +81,20 @@ class Quantizer(Format):
     scale_dtype: str = 'fp32'
 
     def __post_init__(self):
-        assert self.axis in AXES, f'axis must be one of {AXES}, got {self.axis!r}'
-        assert 2 <= self.bits <= 15, f'bits must be in 2..15, got {self.bits}'
-        assert self.zero_point in ('int', 'fp') and self.rounding in ('rtn', 'sr')
-        assert self.rotation in (None, 'hadamard')
-        assert self.scale_bits in (8, 16)
-        assert self.scale_dtype in ('fp32', 'fp16') and (self.scale_dtype == 'fp32' or self.scale_bits == 16)
+        problems = []
+        if self.axis not in AXES:
+            problems.append(f'axis must be one of {AXES}, got {self.axis!r}')
+        if not 2 <= self.bits <= 15:
+            problems.append(f'bits must be in 2..15, got {self.bits}')
+        if self.zero_point not in ('int', 'fp') or self.rounding not in ('rtn', 'sr'):
+            problems.append(f'zero_point {self.zero_point!r} / rounding {self.rounding!r}')
+        if self.rotation not in (None, 'hadamard'):
+            problems.append(f'rotation {self.rotation!r}')
+        if self.scale_bits not in (8, 16) or self.scale_dtype not in ('fp32', 'fp16'):
+            problems.append(f'scale_bits {self.scale_bits} / scale_dtype {self.scale_dtype!r}')
+        elif self.scale_dtype == 'fp16' and self.scale_bits != 16:
+            problems.append('fp16 scales are 16-bit scales')
+        assert not problems, '; '.join(problems)
 
     def _cast_scale(self, scale):
         """quantizer.py:159-164 (16-bit scales only)."""
@@ -120,10 +128,14 @@ class Quantizer(Format):
         return out.to(S.dtype)
 
     def bits_per_value(self, d_k, d_v):
-        side = self.scale_bits
+        """Payload bits plus the per-group side information (scale, and a zero point for affine grids) spread over the
+        group's values; a ragged last group counts as a whole group."""
+        per_group = self.scale_bits
         if self.affine:
-            side += self.bits if self.zero_point == 'int' else self.scale_bits
+            per_group += self.bits if self.zero_point == 'int' else self.scale_bits
         if self.axis == 'head':
-            return self.bits + side / (d_k * d_v)
-        n = d_k if self.axis == 'k' else d_v
-        return self.bits + side * -(-n // self.group) / n
+            groups, values = 1, d_k * d_v
+        else:
+            values = d_k if self.axis == 'k' else d_v
+            groups = (values + self.group - 1) // self.group
+        return self.bits + per_group * groups / values
