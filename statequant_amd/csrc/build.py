@@ -14,6 +14,7 @@ import concurrent.futures as cf
 import hashlib
 import itertools
 import os
+import re
 import subprocess
 import sys
 
@@ -26,7 +27,9 @@ ARCH = 'gfx950'
 # -ffp-contract=off: every fused multiply-add in the kernels is written explicitly, as in the reference's kernels.
 # The packed-fp32 target feature is switched off on purpose (plain v_fma / v_mul only).
 HIPCC_FLAGS = ['--offload-arch=' + ARCH, '-O3', '-std=c++17', '-fPIC', '-ffp-contract=off',
-               '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops', '-Wno-unused-command-line-argument']
+               '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops', '-Wno-unused-command-line-argument',
+               # scalar kernel arguments ahead of a parameter struct arrive in registers (no load at wave start)
+               '-mllvm', '-amdgpu-kernarg-preload-count=16']
 
 
 def _cases():
@@ -69,6 +72,8 @@ def _cases():
 CASES = _cases()
 GGA_SHAPES = [(128, 128), (64, 64)]                  # (d_k, d_v) of the mixed-width GGA / STEP slot (sq_gga.cuh)
 PARAMS = {'gdn': 'GdnParams', 'kda': 'KdaParams', 'mamba2': 'Mamba2Params'}
+# families with a workgroup-per-key-head kernel (sq_<family>_quad.cuh) -> value heads per workgroup that are built
+QUAD_FAMILIES = {'gdn': (2, 1)}
 CHUNK = 6                                            # instances per translation unit
 
 
@@ -76,6 +81,52 @@ def _tile(c):
     bits, dk, dv, group, qbuf, mmax, axv = c
     return (f'Tile<{bits}, {dk}, {dv}, {group}, {"true" if qbuf else "false"}, {mmax}'
             + (', true>' if axv else '>'))
+
+
+# Run-time conditions of the workgroup-per-key-head kernels, per family (part of the generated dispatch unit).
+QUAD_OK = {'gdn': [
+    '// q, k per key head (or ungrouped keys), rows that 32-bit vector loads can address',
+    'static bool gdn_quad_ok(const GdnParams& p) {',
+    '    if (!p.qk_per_key_head && p.gqa > 1) return false;',
+    '    auto ok = [](const void* ptr, uint32_t stride, int dt) {',
+    '        return dt == 0 || ((reinterpret_cast<uintptr_t>(ptr) % 4) == 0 && stride % 2 == 0);',
+    '    };',
+    '    return ok(p.q, p.s_q, p.q_dt) && ok(p.k, p.s_k, p.k_dt);',
+    '}']}
+
+
+def quad_variants(fam, c):
+    """[(row blocks per wavefront, value heads per workgroup, wavefronts per SIMD the register allocation aims
+    for)], widest head group first, of the workgroup-per-key-head kernels (sq_quad.cuh) for a case; empty where only
+    the one-wavefront kernels (sq_tile.cuh) serve it: value-axis groups, the float state, rows that are not a power
+    of two in size, d_k above 128, more than four scale groups per row."""
+    bits, dk, dv, group, qbuf, mmax, axv = c
+    if fam not in QUAD_FAMILIES or axv or bits not in (4, 8):
+        return []
+    rb = dk * bits // 8
+    if rb & (rb - 1) or not 32 <= rb <= 128 or dk > 128 or dv % 32 or (bits == 4 and dk % 64):
+        return []
+    if -(-dk // group) > 4:
+        return []
+    nrb = dv // 32
+    nb = 2 if nrb % 2 == 0 else 1
+    be = 1 if qbuf else 2
+    out = []
+    for gh in QUAD_FAMILIES[fam]:
+        nw = gh * nrb // nb
+        if nw > 16:
+            continue
+        lds = gh * dv * rb + mmax * dk * be + gh * mmax * dv * be + 2 * dk * 4 + dk * 8 + 512
+        wgs = min(160 * 1024 // lds, 32 // nw)
+        if wgs < 1:
+            continue
+        out.append((nb, gh, max(1, min(7, -(-wgs * nw // 4)))))
+    return out
+
+
+def _quad_name(fam, c, v):
+    nb, gh, wpe = v
+    return f'launch_{fam}_quad<{_tile(c)}, {nb}, {gh}, {wpe}>'
 
 
 def _write_if_changed(path, text):
@@ -95,6 +146,14 @@ def generate():
                            for c in rows[k:k + CHUNK])
             path = os.path.join(OUT, f'inst_{fam}_{k // CHUNK:02d}.hip')
             _write_if_changed(path, f'// generated by build.py\n#include "../sq_{fam}.cuh"\nnamespace sq {{\n{body}}}\n')
+            units.append(path)
+    for fam, rows in CASES.items():
+        qrows = [(c, v) for c in rows for v in quad_variants(fam, c)]
+        for k in range(0, len(qrows), CHUNK):
+            body = ''.join(f'template int {_quad_name(fam, c, v)}(const {PARAMS[fam]}&, hipStream_t);\n'
+                           for c, v in qrows[k:k + CHUNK])
+            path = os.path.join(OUT, f'inst_{fam}q_{k // CHUNK:02d}.hip')
+            _write_if_changed(path, f'// generated by build.py\n#include "../sq_{fam}_quad.cuh"\nnamespace sq {{\n{body}}}\n')
             units.append(path)
     # pack / read: instances by (bits, d_k, group, value-axis[, buffer, per-channel decay]); d_v and m are run-time there
     rowfmt = sorted({(c[0], c[1], c[3], c[6]) for rows in CASES.values() for c in rows})
@@ -116,7 +175,7 @@ def generate():
                       + ''.join(f'template int launch_gga<GgaTile<{dk}, {dv}>>(const GgaParams&, int, hipStream_t);\n'
                                 for dk, dv in GGA_SHAPES) + '}\n')
     units.append(path)
-    d = ['// generated by build.py: layout -> compiled kernel instance', '#include "../sq_convert.cuh"',
+    d = ['// generated by build.py: layout -> compiled kernel instance', '#include <stdlib.h>', '#include "../sq_convert.cuh"',
          'namespace sq {',
          'int launch_fold_first(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,',
          '                      hipStream_t stream) {',
@@ -126,12 +185,21 @@ def generate():
     for fam, rows in CASES.items():
         P = PARAMS[fam]
         d.append(f'template <class T> int launch_{fam}(const {P}&, hipStream_t);')
+        if fam in QUAD_FAMILIES:
+            d.append(f'template <class T, int NB, int GH, int WPE> int launch_{fam}_quad(const {P}&, hipStream_t);')
+            d += QUAD_OK[fam]
         d.append(f'int dispatch_{fam}(const {P}& p, hipStream_t stream, bool run) {{')
+        if fam in QUAD_FAMILIES:
+            d.append(f'    const bool quad = !getenv("SQ_NO_QUAD") && (!run || {fam}_quad_ok(p));')
+            d.append('    const int ghmax = getenv("SQ_GH1") ? 1 : 64;')
         # smallest sufficient buffer bound first
         for c in sorted(rows, key=lambda c: c[5]):
             bits, dk, dv, group, qbuf, mmax, axv = c
-            d.append(f'    if (p.bits == {bits} && p.dk == {dk} && p.dv == {dv} && p.group == {group} && p.axv == {axv} '
-                     f'&& p.qbuf == {qbuf} && p.m <= {mmax}) return run ? launch_{fam}<{_tile(c)}>(p, stream) : 0;')
+            cond = (f'p.bits == {bits} && p.dk == {dk} && p.dv == {dv} && p.group == {group} && p.axv == {axv} '
+                    f'&& p.qbuf == {qbuf} && p.m <= {mmax}')
+            for v in quad_variants(fam, c):
+                d.append(f'    if (quad && p.gqa % {v[1]} == 0 && {v[1]} <= ghmax && {cond}) return run ? {_quad_name(fam, c, v)}(p, stream) : 0;')
+            d.append(f'    if ({cond}) return run ? launch_{fam}<{_tile(c)}>(p, stream) : 0;')
         d.append('    return -1;\n}')
     d.append('template <int BITS, int DK, int GROUP, bool AXV> int launch_pack(const PackParams&, hipStream_t);')
     d.append('int dispatch_pack(const PackParams& p, hipStream_t stream, bool run) {')
@@ -173,12 +241,39 @@ def _stamp():
     return h.hexdigest()
 
 
-def _compile(src):
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"([^"]+)"', re.M)
+
+
+def _unit_hash(src, seen=None):
+    """Hash of a translation unit with every header it includes by "quotes", transitively, and the flags."""
+    seen = {} if seen is None else seen
+    todo = [os.path.abspath(src)]
+    while todo:
+        path = todo.pop()
+        if path in seen or not os.path.exists(path):
+            continue
+        text = open(path).read()
+        seen[path] = text
+        todo += [os.path.normpath(os.path.join(os.path.dirname(path), inc)) for inc in _INCLUDE.findall(text)]
+    h = hashlib.sha256(' '.join(HIPCC_FLAGS).encode())
+    for path in sorted(seen):
+        h.update(path.encode())
+        h.update(seen[path].encode())
+    return h.hexdigest()
+
+
+def _compile(src, force=False):
+    """Compile one unit unless its object is current (same sources, headers and flags as when it was built)."""
     obj = os.path.join(OUT, os.path.splitext(os.path.basename(src))[0] + '.o')
+    tag, want = obj + '.hash', _unit_hash(src)
+    if not force and os.path.exists(obj) and os.path.exists(tag) and open(tag).read() == want:
+        return obj
     cmd = ['hipcc', *HIPCC_FLAGS, '-c', src, '-o', obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode:
         raise RuntimeError(f'{" ".join(cmd)}\n{r.stdout}\n{r.stderr}')
+    with open(tag, 'w') as f:
+        f.write(want)
     return obj
 
 
@@ -196,7 +291,7 @@ def build(jobs=None, force=False, verbose=True):
         n = sum(len(r) for r in CASES.values())
         print(f'[build] hipcc {ARCH}: {n} kernel instances in {len(units)} translation units, {jobs} jobs')
     with cf.ThreadPoolExecutor(jobs) as ex:
-        objs = list(ex.map(_compile, units))
+        objs = list(ex.map(lambda u: _compile(u, force), units))
     cmd = ['hipcc', '--offload-arch=' + ARCH, '-shared', '-fPIC', '-o', LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode:

@@ -1,0 +1,495 @@
+// Gated DeltaNet packed decode step, one workgroup per (batch row, key head): the GH value heads of the key head
+// share q, k, the buffered keys and everything computed from them; every wavefront owns NB 32-row blocks of one
+// value head's state (int4 / int8 codes, key-axis scale groups; geometry and building blocks in sq_quad.cuh).
+//
+// Same arithmetic per head as the one-wavefront kernel of sq_gdn.cuh (the reference's fused Triton step,
+// /root/reference/src/statequant/kernels/_fused_triton.py:48-190).  Division of labour inside the workgroup:
+//   issue            every wavefront: its row blocks, their scales, its rows of v and of the buffered values, its
+//                    share of the buffered keys, its head's decays and counters -- all in flight before any is used
+//   roles            one wavefront each: q (l2 norm, scale, digit planes);  k (l2 norm, digit planes);  per head the
+//                    gates and decays;  then everything lands in LDS                                       [barrier]
+//   per wavefront    its row blocks' S0 q, S0 k on the matrix core;  K_i . q, K_i . k of its share of the slots;
+//                    one wavefront: k . q and this token's buffered key                                    [barrier]
+//                    buffer term, u, o for its rows;  max |u| of the head                                  [barrier]
+//                    append;  with a full buffer: fold of its row blocks out of LDS, stored back           [barrier]
+// Requires q and k given per key head (or one value head per key head): with per-value-head q / k and grouped keys
+// the one-wavefront kernel runs instead.
+#pragma once
+#include "sq_gdn.cuh"
+#include "sq_quad.cuh"
+
+namespace sq {
+
+// NE consecutive elements of a float vector of run-time dtype, one load per lane: raw[t] = element NE lane + t as
+// `load_raw` leaves it (fp32 bits, or the 16-bit pattern).  The vector's base must be 4-byte aligned.
+template <int NE>
+__device__ __forceinline__ void load_vec(const void* base, int dt, int lane, uint32_t (&raw)[NE]) {
+    if (dt == F32) {
+        if constexpr (NE == 1) raw[0] = reinterpret_cast<const uint32_t*>(base)[lane];
+        else if constexpr (NE == 2) {
+            const v2u x = reinterpret_cast<const v2u*>(base)[lane];
+            raw[0] = x.x; raw[1] = x.y;
+        } else {
+            const v4u x = reinterpret_cast<const v4u*>(base)[lane];
+            raw[0] = x.x; raw[1] = x.y; raw[2] = x.z; raw[3] = x.w;
+        }
+    } else {
+        if constexpr (NE == 1) raw[0] = reinterpret_cast<const uint16_t*>(base)[lane];
+        else if constexpr (NE == 2) {
+            const uint32_t x = reinterpret_cast<const uint32_t*>(base)[lane];
+            raw[0] = x & 0xFFFFu; raw[1] = x >> 16;
+        } else {
+            const v2u x = reinterpret_cast<const v2u*>(base)[lane];
+            raw[0] = x.x & 0xFFFFu; raw[1] = x.x >> 16; raw[2] = x.y & 0xFFFFu; raw[3] = x.y >> 16;
+        }
+    }
+}
+
+// Everything a wavefront loads for one item, as issued loads (raw bits; nothing here waits for memory).
+template <class T, class Q>
+struct GdnLoads {
+    v4u cw[Q::NB][Q::NLD];                 // its row blocks
+    uint16_t sc[Q::NB][T::NG];             // scales of rows (block bi, lane % 32)
+    Raw4<T::QBUF> uraw[Q::UT], kraw[Q::KT];
+    uint16_t kbs[Q::KT], ubs;
+    float gbl, gcur;
+    int np;
+    uint32_t xr[Q::NE], xr2[Q::NE], g0, g1, g2, g3, vr;
+};
+
+template <class T, int NB, int GH, int WPE>
+__global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
+void gdn_quad_kernel(const int32_t* idx, const int32_t* order, int per_xcd, int rows_per_xcd, int hv, int hv_shift,
+                     const GdnParams p) {
+    // the leading arguments (copies of fields of `p`) are what the slot index load needs: as separate scalar
+    // arguments they are preloaded into registers at wave launch, so that load goes out first thing
+    using Q = Quad<T, NB, GH>;
+    using L = QuadLds<T, NB, GH, 2, 2>;
+    constexpr int DK = T::DK, DV = T::DV, NW = Q::NW, NWH = Q::NWH, MM = T::MMAX, NE = Q::NE, NG = T::NG;
+    constexpr int RQ = 1 % NW, RK = 3 % NW, RX = 2 % NW;          // which wavefront plays which shared role
+    __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
+    uint8_t* lds_kbr = lds + L::KBR;
+    float* lds_xn = reinterpret_cast<float*>(lds + L::XN);
+    uint8_t* lds_pl = lds + L::PL;
+    float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
+    float* lds_dots = reinterpret_cast<float*>(lds + L::DOTS);
+    float* lds_kbsf = reinterpret_cast<float*>(lds + L::KBSF);
+    float* lds_red = reinterpret_cast<float*>(lds + L::RED);
+
+    const int lane0 = threadIdx.x & (WAVE - 1);
+    const int w = __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6);
+    const int hl = w / NWH, wh = w % NWH;                         // head of the group, wavefront of the head
+    const int m = p.m;
+    uint8_t* lds_ubr = lds + L::UBR + hl * (MM * DV * T::BE);     // this head's buffered values
+    float* lds_ubsf = reinterpret_cast<float*>(lds + L::UBSF) + hl * MM;
+    float* lds_scal = reinterpret_cast<float*>(lds + L::SCAL) + hl * 8;
+    float* lds_gsc = reinterpret_cast<float*>(lds + L::SCAL) + GH * 8;   // the group's scalars (k . q)
+    float* lds_gbf = reinterpret_cast<float*>(lds + L::GBF) + hl * MM;
+    uint16_t* lds_sc = reinterpret_cast<uint16_t*>(lds + L::SC) + hl * (DV * NG);
+    uint8_t* my_codes = lds + L::CODES + hl * Q::HEAD + wh * NB * Q::BLK;
+    static_assert((WAVE / Q::CPR) % (Q::SWD * Q::SWM) == 0 || Q::NLD == 1, "swizzle period");
+
+    // ---- this workgroup's item: (batch row, head group), dealt so that every XCD walks a contiguous range ----
+    const int ngrp = hv / GH;                                     // head groups per batch row
+    struct Item { int b, grp, slot; };
+    Item cur;
+    {
+        const int wg = blockIdx.x;
+        const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
+        cur.b = hv_shift >= 0 ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
+        cur.grp = item - cur.b * ngrp;
+        if (order) {
+            int pos = cur.b;
+            if (rows_per_xcd) {
+                const int x = pos / rows_per_xcd;
+                pos = (pos - x * rows_per_xcd) * 8 + x;
+            }
+            cur.b = order[pos];
+        }
+        cur.slot = idx ? idx[cur.b] : cur.b;
+    }
+    auto tile_of = [&](const Item& it) {
+        TileId t;
+        t.b = it.b;
+        t.h = it.grp * GH + hl;
+        t.hk = p.gqa_shift >= 0 ? t.h >> p.gqa_shift : t.h / p.gqa;
+        return t;
+    };
+
+    // ---- issue every load of an item: first the token's own operands (their addresses need the batch row only) ...
+    GdnLoads<T, Q> F;
+    auto issue = [&](const Item& it, int lane, int n32, int row) {
+        const TileId tid = tile_of(it);
+        const uint32_t b = tid.b, h = tid.h;
+        if constexpr (RQ == RK) {                                 // a single wavefront carries both vectors
+            if (w == RQ) {
+                load_vec<NE>(advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(tid.hk) * DK), p.q_dt, lane, F.xr);
+                load_vec<NE>(advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(tid.hk) * DK), p.k_dt, lane, F.xr2);
+            }
+        } else if (w == RQ || w == RK) {
+            const bool isq = w == RQ;
+            const void* base = isq ? advance(p.q, p.q_dt, uint64_t(b) * p.s_q + uint32_t(tid.hk) * DK)
+                                   : advance(p.k, p.k_dt, uint64_t(b) * p.s_k + uint32_t(tid.hk) * DK);
+            load_vec<NE>(base, isq ? p.q_dt : p.k_dt, lane, F.xr);
+        }
+        if (wh == 0) {
+            F.g0 = load_raw_uniform(p.a, p.a_dt, uint64_t(b) * p.s_a + h);
+            F.g1 = load_raw_uniform(p.bt, p.bt_dt, uint64_t(b) * p.s_bt + h);
+            F.g2 = load_raw_uniform(p.A_log, p.A_log_dt, h);
+            F.g3 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);
+        }
+        F.vr = load_raw(advance(p.v, p.v_dt, uint64_t(b) * p.s_v + h * DV), p.v_dt, uint32_t(row));
+    };
+    // ... and the slot's side (not for a padding row: nothing of a slot is touched then)
+    auto issue_slot = [&](const GdnAddr<T>& A, int lane, int n32) {
+        F.np = *A.np;
+        F.gcur = *A.gcp;
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+            for (int t = 0; t < Q::NLD; ++t)
+                F.cw[bi][t] = *reinterpret_cast<const v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16);
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) F.sc[bi][g] = A.SCh[uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g)];
+        // buffered values of this wavefront's rows, every slot: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
+#pragma unroll
+        for (int t = 0; t < Q::UT; ++t) {
+            const uint32_t i = lane / Q::LU + Q::SU * t;
+            const uint32_t ic = i < uint32_t(m) ? i : uint32_t(m) - 1;
+            F.uraw[t] = load_raw4<T::QBUF>(A.buf.UB + (ic * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE);
+        }
+        // buffered keys, dealt over the workgroup: lane (slot = SPP (NW t + w) + lane / LPS, columns 4 (lane % LPS) ..)
+#pragma unroll
+        for (int t = 0; t < Q::KT; ++t) {
+            const uint32_t i = Q::SPP * (NW * t + w) + lane / Q::LPS;
+            const uint32_t ic = i < uint32_t(m) ? i : uint32_t(m) - 1;
+            F.kraw[t] = load_raw4<T::QBUF>(A.buf.KB + (ic * DK + 4 * (lane % Q::LPS)) * T::BE);
+            F.kbs[t] = T::QBUF ? A.buf.KBS[ic] : uint16_t(0);
+        }
+        // per slot of this head, lane i: cumulative decay and value scale
+        const uint32_t li = uint32_t(lane) < uint32_t(m) ? lane : 0;
+        F.gbl = A.GBh[li];
+        F.ubs = T::QBUF ? A.buf.UBS[li] : uint16_t(0);
+    };
+
+    {
+        const int lane = lane0;
+        const int n32 = lane & 31, kb = lane >> 5;
+        // the row of the head this lane finishes after the pass (NB = 2: the wavefront's halves take a block each)
+        const int row = (wh * NB + (NB == 2 ? kb : 0)) * T::MR + n32;
+        const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);    // chunk `lane` of a 1 KB piece in the LDS image
+        issue(cur, lane, n32, row);
+        const TileId tid = tile_of(cur);
+        const GdnAddr<T> A = gdn_addr<T>(p, tid, cur.slot);
+        void* const outp = advance(p.out, p.out_dt, A.obase);
+        if (!A.live) {                                   // padding row: zero output, touch nothing else
+            for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(outp, p.out_dt, r, 0.0f);
+            return;
+        }
+        issue_slot(A, lane, n32);
+        // every load of the item is in flight from here on: keep the compiler from sinking any of them to its use,
+        // and from scheduling a use (a conversion, with its wait) up among them
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        {
+        // ---- shared roles (their inputs were issued first) ----
+        auto role_vector = [&](const uint32_t (&raw)[NE], int dt, float post, int v) {
+            float xe[NE], ss = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NE; ++t) {
+                xe[t] = raw_to_f(raw[t], dt);
+                ss = __builtin_fmaf(xe[t], xe[t], ss);
+            }
+            const float nrm = sqrtf(lanes_sum<WAVE>(ss) + 1e-6f);
+#pragma unroll
+            for (int t = 0; t < NE; ++t) xe[t] = xe[t] / nrm * post;
+            if constexpr (NE == 1) lds_xn[v * DK + lane] = xe[0];
+            else if constexpr (NE == 2) *reinterpret_cast<float2*>(lds_xn + v * DK + 2 * lane) = make_float2(xe[0], xe[1]);
+            else *reinterpret_cast<float4*>(lds_xn + v * DK + 4 * lane) = make_float4(xe[0], xe[1], xe[2], xe[3]);
+            quad_stage_planes<T, NE>(xe, v, lane, lds_pl, lds_xs);
+        };
+        if constexpr (RQ == RK) {
+            if (w == RQ) {
+                role_vector(F.xr, p.q_dt, p.scale, 0);
+                role_vector(F.xr2, p.k_dt, 1.0f, 1);
+            }
+        } else {
+            if (w == RQ) role_vector(F.xr, p.q_dt, p.scale, 0);
+            if (w == RK) role_vector(F.xr, p.k_dt, 1.0f, 1);
+        }
+        if (wh == 0) {                                   // this head's gates and decays
+            float g, beta;
+            if (p.gate) {
+                const float x = raw_to_f(F.g0, p.a_dt) + raw_to_f(F.g3, p.dt_bias_dt);
+                const float sp = x <= 20.0f ? logf(1.0f + expf(x)) : x;
+                g = -expf(raw_to_f(F.g2, p.A_log_dt)) * sp;
+                beta = 1.0f / (1.0f + expf(-raw_to_f(F.g1, p.bt_dt)));
+            } else {
+                g = raw_to_f(F.g0, p.a_dt);
+                beta = raw_to_f(F.g1, p.bt_dt);
+            }
+            if (lane == 0) {
+                lds_scal[0] = beta;
+                lds_scal[1] = expf(F.gcur);
+                lds_scal[2] = expf(g);
+                lds_scal[3] = F.gcur + g;
+            }
+        }
+        // ---- the loads land: LDS images of the row blocks, scales, raw buffer pieces ----
+        const int n = F.np & (m - 1);
+        const float gcur = F.gcur;
+        const uint32_t vr = F.vr;
+        uint16_t scw[NB][NG];
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                scw[bi][g] = F.sc[bi][g];
+                if (kb == 0) lds_sc[((wh * NB + bi) * T::MR + n32) * NG + g] = F.sc[bi][g];
+            }
+#pragma unroll
+        for (int t = 0; t < Q::UT; ++t) {
+            const int i = lane / Q::LU + Q::SU * t;
+            if (i < m) store_raw4<T::QBUF>(lds_ubr + (i * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE, F.uraw[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < Q::KT; ++t) {
+            const int i = Q::SPP * (NW * t + w) + lane / Q::LPS;
+            if (i < m) {
+                store_raw4<T::QBUF>(lds_kbr + (i * DK + 4 * (lane % Q::LPS)) * T::BE, F.kraw[t]);
+                if (T::QBUF && lane % Q::LPS == 0) lds_kbsf[i] = f16_to_f32(F.kbs[t]);
+            }
+        }
+        if (wh == 0 && lane < m) {
+            lds_gbf[lane] = F.gbl;
+            if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
+        }
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+            for (int t = 0; t < Q::NLD; ++t)
+                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+        const bool full = n == m - 1;
+        lds_barrier();
+
+        // ---- every wavefront: state pass over its row blocks ----
+        float sq, sk;                                    // (S0 q)[row], (S0 k)[row], scales applied
+        {
+            v4i aop[T::NKS];
+            quad_fetch_planes<T, 2>(lds_pl, lane, aop);
+            float xs[NG];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) xs[g] = lds_xs[kb * NG + g];
+            float own[NB];
+#pragma unroll
+            for (int bi = 0; bi < NB; ++bi) {
+                float sc[NG];
+#pragma unroll
+                for (int g = 0; g < NG; ++g) sc[g] = f16_to_f32(scw[bi][g]);
+                own[bi] = quad_block_pass<Q, T>(my_codes + bi * Q::BLK, aop, xs, sc, lane);
+            }
+            if constexpr (NB == 2) {                     // lane (n, kb) takes over row n of block kb: both sums
+                const auto r = __builtin_amdgcn_permlane32_swap(as_u32(own[0]), as_u32(own[1]), false, false);
+                sq = as_f32(r[0]);
+                sk = as_f32(r[1]);
+            } else {
+                const Pair qk = pair32(own[0]);
+                sq = qk.lo;
+                sk = qk.hi;
+            }
+        }
+        // ---- K_i . q, K_i . k of this wavefront's share of the slots ----
+        {
+            float x[2][4];
+#pragma unroll
+            for (int v = 0; v < 2; ++v) {
+                const float4 f = *reinterpret_cast<const float4*>(lds_xn + v * DK + 4 * (lane % Q::LPS));
+                x[v][0] = f.x; x[v][1] = f.y; x[v][2] = f.z; x[v][3] = f.w;
+            }
+#pragma unroll
+            for (int t = 0; t < Q::KT; ++t) {
+                const int i = Q::SPP * (NW * t + w) + lane / Q::LPS;
+                const int ic = i < m ? i : m - 1;
+                float kf[4];
+                decode_raw4<T::QBUF>(load_raw4<T::QBUF>(lds_kbr + (ic * DK + 4 * (lane % Q::LPS)) * T::BE), kf);
+                if constexpr (T::QBUF) {
+                    const float s = lds_kbsf[ic];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) kf[c] = kf[c] * s;
+                }
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    float pr = kf[0] * x[v][0];
+#pragma unroll
+                    for (int c = 1; c < 4; ++c) pr = __builtin_fmaf(kf[c], x[v][c], pr);
+                    pr = lanes_sum<Q::LPS>(pr);
+                    if (lane % Q::LPS == 0 && i < MM) lds_dots[v * MM + i] = pr;
+                }
+            }
+        }
+        // ---- k . q ----
+        if (w == RK) {
+            float kqp = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NE; ++t) kqp = __builtin_fmaf(lds_xn[DK + NE * lane + t], lds_xn[NE * lane + t], kqp);
+            kqp = lanes_sum<WAVE>(kqp);
+            if (lane == 0) lds_gsc[0] = kqp;
+        }
+        lds_barrier();                                   // the raw keys of slot n may be overwritten from here on
+
+        // ---- the buffered key of this token: the rounded k, for this workgroup's folds and (first head group of
+        //      the key head only) for the slot ----
+        if (w == RX) {
+            float kxe[NE], kmax = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NE; ++t) {
+                kxe[t] = lds_xn[DK + NE * lane + t];
+                kmax = fmaxf(kmax, fabsf(kxe[t]));
+            }
+            float ks = 1.0f;
+            if constexpr (T::QBUF) ks = fp16_scale(lanes_max<WAVE>(kmax), 127.0f);
+            const bool write = tid.h - hl == tid.hk * p.gqa;
+            if (T::QBUF && lane == 0) {
+                lds_kbsf[n] = ks;
+                if (write) A.buf.KBS[n] = f32_to_f16(ks);
+            }
+            if constexpr (T::QBUF) {
+                uint32_t pk = 0;
+#pragma unroll
+                for (int t = 0; t < NE; ++t) pk |= (uint32_t(int(round_buf(kxe[t], ks))) & 0xFFu) << (8 * t);
+                uint8_t* dl = lds_kbr + n * DK + NE * lane;
+                uint8_t* dg = A.buf.KB + n * DK + NE * lane;
+                if constexpr (NE == 1) { *dl = uint8_t(pk); if (write) *dg = uint8_t(pk); }
+                else if constexpr (NE == 2) {
+                    *reinterpret_cast<uint16_t*>(dl) = uint16_t(pk);
+                    if (write) *reinterpret_cast<uint16_t*>(dg) = uint16_t(pk);
+                } else {
+                    *reinterpret_cast<uint32_t*>(dl) = pk;
+                    if (write) *reinterpret_cast<uint32_t*>(dg) = pk;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < NE; ++t) {
+                    const uint16_t hb = f32_to_bf16(kxe[t]);
+                    reinterpret_cast<uint16_t*>(lds_kbr)[n * DK + NE * lane + t] = hb;
+                    if (write) reinterpret_cast<uint16_t*>(A.buf.KB)[n * DK + NE * lane + t] = hb;
+                }
+            }
+        }
+
+        // ---- this wavefront's rows: buffer term, u, o ----
+        const float beta = lds_scal[0], alpha = lds_scal[1], a = lds_scal[2], gnew = lds_scal[3];
+        const float kq = lds_gsc[0];
+        // coefficients of the head's slots, lane i: c_x[i] = exp(gcur - G_i) (K_i . x), times the slot's value scale;
+        // dead slots (i >= n) may hold anything: select, never multiply
+        const int li = lane < m ? lane : 0;
+        float cq, ck;
+        {
+            const float dec = expf(gcur - lds_gbf[li]);
+            const float dq = lds_dots[li], dk_ = lds_dots[MM + li];
+            const float us_i = T::QBUF ? lds_ubsf[li] : 1.0f;
+            const bool alive = lane < n;
+            cq = alive ? (T::QBUF ? (dec * dq) * us_i : dec * dq) : 0.0f;
+            ck = alive ? (T::QBUF ? (dec * dk_) * us_i : dec * dk_) : 0.0f;
+        }
+        float accq = alpha * sq, acck = alpha * sk;
+#pragma unroll
+        for (int i = 0; i < MM; ++i) {
+            if (i < n) {                                 // wave-uniform
+                const float uv = lds_raw<T::QBUF>(lds_ubr, i * DV + row);
+                accq = __builtin_fmaf(uv, lane_bcast(cq, i), accq);
+                acck = __builtin_fmaf(uv, lane_bcast(ck, i), acck);
+            }
+        }
+        const float vt = raw_to_f(vr, p.v_dt);
+        const float u = beta * __builtin_fmaf(-a, acck, vt);
+        const float o = __builtin_fmaf(kq, u, a * accq);
+        if (NB == 2 || kb == 0) store_f(outp, p.out_dt, row, o);
+
+        // ---- append ----
+        float us = 1.0f;
+        if constexpr (T::QBUF) {
+            float amax = lanes_max<WAVE>(fabsf(u));
+            if constexpr (NWH > 1) {
+                if (lane == 0) lds_red[w] = amax;
+                lds_barrier();
+#pragma unroll
+                for (int ww = 0; ww < NWH; ++ww) amax = fmaxf(amax, lds_red[hl * NWH + ww]);
+            }
+            us = fp16_scale(amax, 127.0f);
+            if (wh == 0 && lane == 0) { A.buf.UBS[n] = f32_to_f16(us); lds_ubsf[n] = us; }
+        }
+        if (NB == 2 || kb == 0) {
+            if constexpr (T::QBUF) {
+                const int8_t c = int8_t(int(round_buf(u, us)));
+                reinterpret_cast<int8_t*>(A.buf.UB)[n * DV + row] = c;
+                reinterpret_cast<int8_t*>(lds_ubr)[n * DV + row] = c;
+            } else {
+                const uint16_t hb = f32_to_bf16(u);
+                reinterpret_cast<uint16_t*>(A.buf.UB)[n * DV + row] = hb;
+                reinterpret_cast<uint16_t*>(lds_ubr)[n * DV + row] = hb;
+            }
+        }
+        if (wh == 0 && lane == 0) {
+            A.GBh[n] = gnew;
+            *A.gcp = full ? 0.0f : gnew;                 // advance
+            *A.np = full ? 0 : n + 1;
+        }
+
+        // ---- fold ----
+        if (full) {
+            lds_barrier();                               // `full` is the same in every head of a slot
+            constexpr int MT4 = (MM + 3) / 4, CL = DK / 4;
+            const int fn = lane & 15, fq = lane >> 4;
+            // decay ratios a_m / a_i of the lane's slots 4 t + q (this token: 1)
+            float decf[MT4];
+#pragma unroll
+            for (int t = 0; t < MT4; ++t) {
+                const int sl = 4 * t + fq;
+                decf[t] = sl < m - 1 ? expf(gnew - lds_gbf[sl < m - 1 ? sl : 0]) : 1.0f;
+            }
+            const float cmul = expf(gnew);
+            const int fg = (fq * CL) / T::KGROUP;
+#pragma unroll
+            for (int bi = 0; bi < NB; ++bi) {
+                uint8_t* blk = my_codes + bi * Q::BLK;
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const int frow = (wh * NB + bi) * T::MR + 16 * hf + fn;
+                    float bop[MT4];
+#pragma unroll
+                    for (int t = 0; t < MT4; ++t) {
+                        const int sl = 4 * t + fq;
+                        const int sc_ = sl < m ? sl : 0;
+                        float uv = lds_raw<T::QBUF>(lds_ubr, sc_ * DV + frow);
+                        if constexpr (T::QBUF) uv = uv * lds_ubsf[sc_];
+                        uv = decf[t] * uv;
+                        bop[t] = sl < m ? uv : 0.0f;
+                    }
+                    quad_fold_half<Q, T, false>(blk, hf, lds_kbr, lds_kbsf, nullptr, nullptr, bop, cmul, m,
+                                                f16_to_f32(lds_sc[frow * NG + fg]), A.SCh + frow * NG + fg, lane);
+                }
+                wave_sync();
+#pragma unroll
+                for (int t = 0; t < Q::NLD; ++t)
+                    *reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16) =
+                        *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0);
+            }
+        }
+        }
+    }
+}
+
+template <class T, int NB, int GH, int WPE>
+int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
+    GdnParams p = p0;
+    p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
+    if (p.per_xcd == 0) p.rows_per_xcd = 0;
+    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
+                       0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
+    return int(hipGetLastError());
+}
+
+}  // namespace sq

@@ -1,0 +1,411 @@
+// The state tile of one (sequence, value head) shared by the wavefronts of one workgroup: every wavefront owns NB of
+// the tile's 32-row blocks.  Shared by the Gated DeltaNet, KDA and Mamba2 step kernels for int4 / int8 codes with
+// key-axis scale groups and a power-of-two row size.
+//
+// What this buys over one wavefront per tile (sq_tile.cuh, kept for the other formats):
+//   * a tile's life is a quarter as long, so the launch's ramp-up and tail shrink and the dispatcher balances the
+//     compute units with a finer grain;
+//   * a row block stays in LDS from the state pass to the fold, so a folding tile reads its codes from memory once;
+//   * the front end (normalisation, digit planes, gates, buffer coefficients) is split across the wavefronts instead
+//     of running back to back in one.
+//
+// Row dot products run on the matrix core as in sq_tile.cuh (codes against three signed 8-bit digit planes of the
+// fixed-point read-out vectors, exact int32 sums), with the operands' roles swapped: the digit planes are the first
+// operand (result row 8 g + 4 v + d = scale group g, vector v, digit d) and the codes the second (result column =
+// state row).  v_mfma_i32_32x32x32_i8 leaves result rows 8 a + 4 kb + b of column n in lane (n, kb), element
+// 4 a + b -- so lane (state row n, vector kb) ends up with exactly the three digits of all of its row's groups, and
+// the sums never travel through LDS.
+//
+// LDS image of a row block: the rows as stored, 16-byte chunks XOR-swizzled inside a row so that both the row-shaped
+// writes (lanes along a row) and the operand-shaped reads (lanes down a column of chunks) are conflict free without
+// padding.
+#pragma once
+#include "sq_tile.cuh"
+#include "sq_params.h"
+
+namespace sq {
+
+// Compute units of the current device (queried once per process and device; 256 on an MI355X).
+inline int quad_compute_units() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (!cached[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// LDS-only release / acquire around a workgroup barrier: the state codes still in flight from global memory (plain
+// register loads) are not waited for.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <class T, int NB_, int GH_ = 1>
+struct Quad {
+    static_assert(!T::FLT && !T::AXV && !T::RAGV, "int4 / int8 codes with key-axis groups, whole row blocks");
+    static constexpr int NB = NB_;                         // row blocks per wavefront
+    static constexpr int GH = GH_;                         // value heads of one key head per workgroup
+    static_assert(T::NRB % NB == 0 && (NB == 1 || NB == 2), "one or two row blocks per wavefront");
+    static constexpr int NWH = T::NRB / NB;                // wavefronts per head
+    static constexpr int NW = GH * NWH;                    // wavefronts per workgroup
+    static constexpr int THREADS = NW * WAVE;
+    static_assert(THREADS <= 1024, "workgroup size");
+    static constexpr int RW = NB * T::MR;                  // rows per wavefront
+    static constexpr int RB = T::ROW_BYTES;
+    static_assert((RB & (RB - 1)) == 0 && RB >= 32 && RB <= 256, "row size: a power of two in 32..256 bytes");
+    static_assert(T::BITS == 8 || T::DK % 64 == 0, "int4: d_k a multiple of 64");
+    static constexpr int CPR = RB / 16;                    // 16-byte chunks per row
+    static constexpr int BLK = T::MR * RB;                 // bytes of a row block
+    static constexpr int HEAD = T::DV * RB;                // bytes of a head's codes
+    static constexpr int NLD = BLK / 1024;                 // wavefront loads per row block
+    static constexpr int SWM = CPR < 8 ? CPR : 8;          // swizzle: chunk c of row r sits at chunk c ^ ((r / SWD) % SWM)
+    static constexpr int SWD = 8 / SWM;
+    static_assert(T::NG <= 4, "at most four scale groups per row (result rows 8 g + 4 v + d)");
+    // a d_k vector in a wavefront: lane l holds the NE consecutive elements NE l ..
+    static constexpr int NE = T::DK / WAVE;
+    static_assert(NE * WAVE == T::DK && NE >= 1 && NE <= 4, "d_k: 64, 128 or 256");
+    // buffer passes: keys 4 columns per lane (slots dealt over the workgroup's wavefronts), values 4 rows per lane
+    static constexpr int LPS = T::DK / 4;                  // lanes per buffered key
+    static constexpr int SPP = WAVE / LPS;                 // keys per wavefront and pass
+    static constexpr int KT = (T::MMAX + NW * SPP - 1) / (NW * SPP);
+    static constexpr int LU = RW / 4;                      // lanes per buffered value piece of this wavefront's rows
+    static constexpr int SU = WAVE / LU;
+    static constexpr int UT = (T::MMAX + SU - 1) / SU;
+};
+
+// Byte offset, inside a row block's LDS image, of chunk c of row r.
+template <class Q>
+__device__ __forceinline__ int swz(int r, int c) { return r * Q::RB + ((c ^ ((r / Q::SWD) % Q::SWM)) << 4); }
+
+template <class T, int NB, int GH, int NX, int NV>
+struct QuadLds {
+    using Q = Quad<T, NB, GH>;
+    static constexpr int CODES = 0;                                    // [GH][DV] rows, swizzled
+    static constexpr int KBR = CODES + GH * Q::HEAD;                   // buffered keys, raw [m][DK]
+    static constexpr int UBR = KBR + T::MMAX * T::DK * T::BE;          // buffered values, raw [GH][m][DV]
+    static constexpr int XN = UBR + GH * T::MMAX * T::DV * T::BE;      // read-out vectors, fp32 [NX][DK]
+    static constexpr int PL = XN + NX * T::DK * 4;                     // digit planes [k-step][half][8][16]
+    static constexpr int XS = PL + T::DK * 8;                          // [NV][NG] exponent factors
+    static constexpr int DOTS = XS + round_up(NV * T::NG * 4, 16);     // [NV][MMAX] K_i . x
+    static constexpr int KBSF = DOTS + NV * T::MMAX * 4;               // [MMAX] key scales as fp32
+    static constexpr int UBSF = KBSF + T::MMAX * 4;                    // [GH][MMAX] value scales as fp32
+    static constexpr int SCAL = UBSF + GH * T::MMAX * 4;               // [GH][8] scalars of a head + [8] of the group
+    static constexpr int RED = SCAL + (GH + 1) * 32;                   // one float per wavefront
+    static constexpr int GBF = RED + round_up(Q::NW * 4, 16);          // [GH][MMAX] cumulative decays of the slots
+    static constexpr int SC = GBF + GH * T::MMAX * 4;                  // [GH][DV][NG] fp16 scales of the rows
+    static constexpr int BYTES = SC + round_up(GH * T::DV * T::NG * 2, 16);
+};
+
+// Where column e of a read-out vector goes in the digit-plane region: the (k-step, lane half, byte) at which the
+// matrix core meets it with the codes.  int8: k-step ks, half kb carry columns 32 ks + 16 kb + [0, 16).  int4: a lane
+// reads whole 16-byte chunks (32 columns) and feeds them as two k-steps, so k-step ks, half kb carry columns
+// 32 (2 (ks / 2) + kb) + 16 (ks % 2) + [0, 16), in the nibble-split order of `operand`.
+template <class T>
+__device__ __forceinline__ int plane_addr(int e, int pl) {
+    int ks, kb, pos;
+    if constexpr (T::BITS == 8) {
+        ks = e / 32; kb = (e / 16) % 2; pos = e % 16;
+    } else {
+        const int p = e / 32;
+        kb = p % 2; ks = 2 * (p / 2) + (e % 32) / 16; pos = operand_pos<4>(e % 16);
+    }
+    return ((ks * 2 + kb) * 8 + pl) * 16 + pos;
+}
+template <class T>
+__device__ __forceinline__ constexpr int op_colbase(int ks, int kb) {
+    return T::BITS == 8 ? 32 * ks + 16 * kb : 32 * (2 * (ks / 2) + kb) + 16 * (ks % 2);
+}
+
+// Both values of a lane pair 16 / 32 lanes apart, in both lanes: {lower lane's, upper lane's}.
+struct Pair { float lo, hi; };
+__device__ __forceinline__ Pair pair32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(as_u32(v), as_u32(v), false, false);
+    return Pair{as_f32(r[0]), as_f32(r[1])};
+}
+__device__ __forceinline__ Pair pair16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(as_u32(v), as_u32(v), false, false);
+    return Pair{as_f32(r[0]), as_f32(r[1])};
+}
+// Sum / maximum over aligned blocks of N lanes, N a power of two up to 64; every lane of a block gets the result.
+template <int N>
+__device__ __forceinline__ float lanes_sum(float v) {
+    v = block_sum<(N < 16 ? N : 16)>(v);
+    if constexpr (N >= 32) { const Pair p = pair16(v); v = p.lo + p.hi; }
+    if constexpr (N >= 64) { const Pair p = pair32(v); v = p.lo + p.hi; }
+    return v;
+}
+template <int N>
+__device__ __forceinline__ float lanes_max(float v) {
+    v = block_max<(N < 16 ? N : 16)>(v);
+    if constexpr (N >= 32) { const Pair p = pair16(v); v = fmaxf(p.lo, p.hi); }
+    if constexpr (N >= 64) { const Pair p = pair32(v); v = fmaxf(p.lo, p.hi); }
+    return v;
+}
+
+// One read-out vector -> its three digit planes (plane slots 3 v .. 3 v + 2) and its exponent factors; xe[t] =
+// element NE lane + t.  Arithmetic as `stage_planes` in sq_tile.cuh: per scale group e = exponent of the largest
+// |x|, q = rint(x 2^(22 - e)) cut into three signed 8-bit digits.
+template <class T, int NE>
+__device__ __forceinline__ void quad_stage_planes(const float (&xe)[NE], int v, int lane, uint8_t* lds_pl,
+                                                  float* lds_xs) {
+    float mx = 0.0f;
+#pragma unroll
+    for (int t = 0; t < NE; ++t) mx = fmaxf(mx, fabsf(xe[t]));
+    constexpr int GL = T::KGROUP / NE;                       // lanes per scale group
+    static_assert(GL >= 1 && GL <= WAVE, "scale group inside a wavefront");
+    const float gmax = lanes_max<GL>(mx);
+    int ex = __builtin_amdgcn_frexp_expf(gmax);
+    ex = ex < -100 ? -100 : ex;
+    const float up = __builtin_ldexpf(1.0f, 22 - ex);
+    uint32_t d[NE];
+#pragma unroll
+    for (int t = 0; t < NE; ++t) {
+        const float f = __builtin_fmaf(xe[t], up, 12582912.0f);
+        d[t] = (as_u32(f) + 0x408080u) ^ 0x808080u;
+    }
+    const int e0 = NE * lane;
+    if constexpr (T::BITS == 8 && NE == 2) {                 // neighbouring columns are neighbouring operand bytes
+        uint8_t* at = lds_pl + plane_addr<T>(e0, 3 * v);
+        *reinterpret_cast<uint16_t*>(at) = uint16_t((d[0] & 0xFFu) | ((d[1] & 0xFFu) << 8));
+        *reinterpret_cast<uint16_t*>(at + 16) = uint16_t(((d[0] >> 8) & 0xFFu) | (d[1] & 0xFF00u));
+        *reinterpret_cast<uint16_t*>(at + 32) = uint16_t(((d[0] >> 16) & 0xFFu) | ((d[1] >> 8) & 0xFF00u));
+    } else {
+#pragma unroll
+        for (int t = 0; t < NE; ++t) {
+            uint8_t* at = lds_pl + plane_addr<T>(e0 + t, 3 * v);
+            at[0] = uint8_t(d[t]);
+            at[16] = uint8_t(d[t] >> 8);
+            at[32] = uint8_t(d[t] >> 16);
+        }
+    }
+    if (e0 % T::KGROUP == 0) lds_xs[v * T::NG + e0 / T::KGROUP] = __builtin_ldexpf(1.0f, ex - 22 - (T::BITS == 4 ? 4 : 0));
+}
+
+// The digit planes as the matrix core's first operand, per k-step: lane (i, kb) carries result row i = 8 g + 4 v + d,
+// i.e. digit d of vector v -- on the k-steps whose columns belong to scale group g, zero elsewhere (and zero in the
+// unused rows), so that ONE accumulation over all k-steps leaves every group's sums in its own result rows.
+template <class T, int NV>
+__device__ __forceinline__ void quad_fetch_planes(const uint8_t* lds_pl, int lane, v4i (&aop)[T::NKS]) {
+    const int i = lane & 31, kb = lane >> 5;
+    const int g = i >> 3, v = (i >> 2) & 1, d = i & 3;
+    const bool used = d < 3 && g < T::NG && v < NV;
+#pragma unroll
+    for (int ks = 0; ks < T::NKS; ++ks) {
+        const v4i x = *reinterpret_cast<const v4i*>(lds_pl + ((ks * 2 + kb) * 8 + 3 * v + (d < 3 ? d : 0)) * 16);
+        const bool mine = used && (kb == 0 ? op_colbase<T>(ks, 0) : op_colbase<T>(ks, 1)) / T::KGROUP == g;
+        aop[ks] = mine ? x : v4i{0, 0, 0, 0};
+    }
+}
+
+// Row sums of one 32-row block (its LDS image at `blk`): lane (n, kb) returns (S0 x_kb)[row n of the block] with the
+// row's scales applied group by group, in order.  xs[g] = the exponent factor of vector kb, group g; sc[g] = the
+// row's scales.
+template <class Q, class T>
+__device__ __forceinline__ float quad_block_pass(const uint8_t* blk, const v4i (&aop)[T::NKS], const float (&xs)[T::NG],
+                                                 const float (&sc)[T::NG], int lane) {
+    const int n = lane & 31, kb = lane >> 5;
+    v16i acc = {0};
+    if constexpr (T::BITS == 8) {
+#pragma unroll
+        for (int ks = 0; ks < T::NKS; ++ks) {
+            const RawRow<8> r = load_row<8>(blk + swz<Q>(n, 2 * ks + kb));
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop[ks], operand<8>(r), acc, 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int kp = 0; kp < T::NKS / 2; ++kp) {
+            const uint4 c = *reinterpret_cast<const uint4*>(blk + swz<Q>(n, 2 * kp + kb));
+            RawRow<4> lo, hi;
+            lo.v = make_uint2(c.x, c.y);
+            hi.v = make_uint2(c.z, c.w);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop[2 * kp], operand<4>(lo), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop[2 * kp + 1], operand<4>(hi), acc, 0, 0, 0);
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int g = 0; g < T::NG; ++g) {
+        const float f = __builtin_fmaf(float(acc[4 * g + 2]), 65536.0f,
+                                       __builtin_fmaf(float(acc[4 * g + 1]), 256.0f, float(acc[4 * g])));
+        const float term = (f * xs[g]) * sc[g];
+        s = g == 0 ? term : s + term;
+    }
+    return s;
+}
+
+// Native vector types for values that stay in registers across the load / use distance (the compiler keeps arrays of
+// HIP's uint4 / uint2 structs in scratch memory when an asm statement separates their loads from their uses).
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+
+// Raw buffered elements: four per lane.
+template <bool QBUF> struct Raw4;
+template <> struct Raw4<true> { uint32_t a; };
+template <> struct Raw4<false> { v2u a; };
+template <bool QBUF>
+__device__ __forceinline__ Raw4<QBUF> load_raw4(const uint8_t* p) {
+    Raw4<QBUF> r;
+    if constexpr (QBUF) r.a = *reinterpret_cast<const uint32_t*>(p);
+    else r.a = *reinterpret_cast<const v2u*>(p);
+    return r;
+}
+template <bool QBUF>
+__device__ __forceinline__ void store_raw4(uint8_t* p, const Raw4<QBUF>& r) {
+    if constexpr (QBUF) *reinterpret_cast<uint32_t*>(p) = r.a;
+    else *reinterpret_cast<v2u*>(p) = r.a;
+}
+template <bool QBUF>
+__device__ __forceinline__ void decode_raw4(const Raw4<QBUF>& r, float (&f)[4]) {
+    if constexpr (QBUF) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) f[b] = s8_to_f(r.a, b);
+    } else {
+        f[0] = as_f32(r.a.x << 16); f[1] = as_f32(r.a.x & 0xFFFF0000u);
+        f[2] = as_f32(r.a.y << 16); f[3] = as_f32(r.a.y & 0xFFFF0000u);
+    }
+}
+// One raw buffered element from LDS as fp32 (unscaled).
+template <bool QBUF>
+__device__ __forceinline__ float lds_raw(const uint8_t* base, int idx) {
+    if constexpr (QBUF) return float(reinterpret_cast<const int8_t*>(base)[idx]);
+    else return bf16_to_f32(reinterpret_cast<const uint16_t*>(base)[idx]);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// the fold of one row block held in LDS
+// ---------------------------------------------------------------------------------------------------------------
+// fp32 value of byte `b` of `w` taken as unsigned, times s, plus o (one conversion + one fma per code; with
+// w = codes ^ 0x80.. and o = -128 s this is (code x s) rounded once, bit-identical to convert-then-multiply).
+template <int B>
+__device__ __forceinline__ float ubyte_fma(uint32_t w, float s, float o) {
+    const float f = float((w >> (8 * B)) & 0xFFu);          // v_cvt_f32_ubyteB
+    return __builtin_fmaf(f, s, o);
+}
+
+// S = cmul S0 + sum_i du_i (x) kx_i over the m buffer slots, four slots per matrix-core issue in slot order
+// (v_mfma_f32_16x16x4_f32, fp32), re-quantized into the block's LDS image and its scales (reference:
+// _fused_triton.py:278-394 `_fold_head`).  Half a row block at a time: lane (n, q) -- n = lane % 16 the row of the
+// half, q = lane / 16 -- owns the quarter q of row n, CL = d_k / 4 consecutive columns, as CL / 4 accumulator tiles
+// of 4 columns: the instruction leaves result rows 4 q + b of result column n in lane (n, q), and the keys are fed
+// so that result row 4 q' + b of tile ct is state column q' CL + 4 ct + b.  A lane's codes are whole 16-byte (8-byte)
+// pieces of the LDS image, a scale group lies in 1, 2 or 4 lanes of a row (lanes 16 or 32 apart), and a 128-column
+// row needs 32 accumulator registers.
+//   lds_kbr / kbsf   buffered keys, raw, and their scales (slot m - 1: this token's, as stored)
+//   bop[t]           the lane's folded values: slot 4 t + q, row n (decay ratio x stored value)
+//   COLVEC           per-column factors on the old state (KDA) from lds_cv, and per-(slot, column) key factors from
+//                    lds_kd [m][DK]; else the scalar cmul
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <class Q, class T, bool COLVEC>
+__device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const uint8_t* lds_kbr, const float* lds_kbsf,
+                                               const float* lds_cv, const float* lds_kd,
+                                               const float (&bop)[(T::MMAX + 3) / 4], float cmul, int m, float s_old,
+                                               uint16_t* sc_out, int lane) {
+    constexpr int MT4 = (T::MMAX + 3) / 4;
+    constexpr int CL = T::DK / 4;                            // columns per lane
+    constexpr int NT = CL / 4;                               // accumulator tiles per lane
+    constexpr int NBY = Q::RB / 4;                           // bytes per lane
+    constexpr int NW32 = NBY / 4;                            // 32-bit words per lane
+    static_assert(CL % 16 == 0 && T::KGROUP % CL == 0 && T::KGROUP / CL <= 4, "a scale group is 1, 2 or 4 lanes wide");
+    constexpr int LPG = T::KGROUP / CL;
+    const int n = lane & 15, q = lane >> 4;
+    const int row = 16 * hf + n;
+
+    // the lane's bytes of the row
+    uint32_t w[NW32];
+    if constexpr (NBY >= 16) {
+#pragma unroll
+        for (int c = 0; c < NBY / 16; ++c) {
+            const uint4 x = *reinterpret_cast<const uint4*>(blk + swz<Q>(row, q * (NBY / 16) + c));
+            w[4 * c] = x.x; w[4 * c + 1] = x.y; w[4 * c + 2] = x.z; w[4 * c + 3] = x.w;
+        }
+    } else {
+        const uint2 x = *reinterpret_cast<const uint2*>(blk + swz<Q>(row, q >> 1) + 8 * (q & 1));
+        w[0] = x.x; w[1] = x.y;
+    }
+    // dequantize: (code x scale) x factor, one conversion + one fma per code
+    const float s = T::BITS == 8 ? s_old : s_old * 0.0625f;
+    const float sm = COLVEC ? s : s * cmul;
+    const float off = -128.0f * sm;
+    v4f acc[NT];
+    if constexpr (T::BITS == 8) {
+#pragma unroll
+        for (int d = 0; d < NW32; ++d) {
+            const uint32_t u = w[d] ^ 0x80808080u;
+            acc[d][0] = ubyte_fma<0>(u, sm, off); acc[d][1] = ubyte_fma<1>(u, sm, off);
+            acc[d][2] = ubyte_fma<2>(u, sm, off); acc[d][3] = ubyte_fma<3>(u, sm, off);
+        }
+    } else {
+        // a stored nibble is code + 8: moved to the high half of a byte it reads 16 code + 128 as an unsigned byte
+#pragma unroll
+        for (int d = 0; d < NW32; ++d) {                     // word d: columns 8 d .. 8 d + 7
+            const uint32_t lo = (w[d] << 4) & 0xF0F0F0F0u, hi = w[d] & 0xF0F0F0F0u;
+            acc[2 * d][0] = ubyte_fma<0>(lo, sm, off); acc[2 * d][1] = ubyte_fma<0>(hi, sm, off);
+            acc[2 * d][2] = ubyte_fma<1>(lo, sm, off); acc[2 * d][3] = ubyte_fma<1>(hi, sm, off);
+            acc[2 * d + 1][0] = ubyte_fma<2>(lo, sm, off); acc[2 * d + 1][1] = ubyte_fma<2>(hi, sm, off);
+            acc[2 * d + 1][2] = ubyte_fma<3>(lo, sm, off); acc[2 * d + 1][3] = ubyte_fma<3>(hi, sm, off);
+        }
+    }
+    if constexpr (COLVEC) {
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct) {
+            const float4 f = *reinterpret_cast<const float4*>(lds_cv + q * CL + 4 * ct);
+            acc[ct][0] *= f.x; acc[ct][1] *= f.y; acc[ct][2] *= f.z; acc[ct][3] *= f.w;
+        }
+    }
+    // the m rank-1 updates: first operand = keys (result row i = 4 q' + b <-> column q' CL + 4 ct + b), second = values
+    const int kcol = (n >> 2) * CL + (n & 3);
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+#pragma unroll
+        for (int t = 0; t < MT4; ++t) {
+            const int slot = 4 * t + q;
+            const int sl = slot < m ? slot : 0;
+            float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
+            if constexpr (T::QBUF) kv = kv * lds_kbsf[sl];
+            if constexpr (COLVEC) kv = kv * lds_kd[sl * T::DK + kcol + 4 * ct];
+            kv = slot < m ? kv : 0.0f;
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv, bop[t], acc[ct], 0, 0, 0);
+        }
+    }
+    // absmax of the lane's columns, then of its scale group
+    float mx = 0.0f;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) mx = fmaxf(mx, fabsf(acc[ct][b]));
+    if constexpr (LPG >= 2) { const Pair pm = pair16(mx); mx = fmaxf(pm.lo, pm.hi); }
+    if constexpr (LPG >= 4) { const Pair pm = pair32(mx); mx = fmaxf(pm.lo, pm.hi); }
+    const float sc = fp16_scale(mx, T::QMAX);
+    const float rs = 1.0f / sc;
+    if (q % LPG == 0) *sc_out = f32_to_f16(sc);
+    // new codes, back into the LDS image
+    if constexpr (NBY >= 16) {
+#pragma unroll
+        for (int c = 0; c < CL / 16; ++c) {                  // 16 columns per call
+            float a16[CPL];
+#pragma unroll
+            for (int e = 0; e < CPL; ++e) a16[e] = acc[4 * c + e / 4][e % 4];
+            const RawRow<T::BITS> r = quantize_row<T::BITS>(a16, rs);
+            if constexpr (T::BITS == 8) {
+                *reinterpret_cast<uint4*>(blk + swz<Q>(row, q * (NBY / 16) + c)) = r.v;
+            } else {                                         // 16 columns = 8 bytes = half a chunk
+                *reinterpret_cast<uint2*>(blk + swz<Q>(row, q * (NBY / 16) + c / 2) + 8 * (c & 1)) = r.v;
+            }
+        }
+    } else {
+        float a16[CPL];
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) a16[e] = acc[e / 4][e % 4];
+        const RawRow<T::BITS> r = quantize_row<T::BITS>(a16, rs);
+        *reinterpret_cast<uint2*>(blk + swz<Q>(row, q >> 1) + 8 * (q & 1)) = r.v;
+    }
+}
+
+}  // namespace sq
