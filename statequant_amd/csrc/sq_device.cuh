@@ -234,7 +234,9 @@ __device__ __forceinline__ RawRow<BITS> encode_row(const float (&c)[CPL]) {
 // a r + 1.5 2^23 (one fma: the exact product, rounded once, half to even, at integer granularity) leaves the code in
 // the low mantissa bits in two's complement; int4 adds its +8 storage bias in the same constant.  The clamp acts on
 // the biased float, the bytes / nibbles are gathered with byte permutes.
-template <int BITS>
+// CLAMP = false leaves the clamp out: for callers that know |a r| < qmax + 1/2 (a scale that is a NORMAL fp16
+// number lies within 2^-11 of absmax / qmax, so the largest quotient is qmax (1 + 2^-11) at most).
+template <int BITS, bool CLAMP = true>
 __device__ __forceinline__ RawRow<BITS> quantize_row(const float (&a)[CPL], float r) {
     constexpr float QMAX = float((1 << (BITS - 1)) - 1);
     constexpr float MAGIC = 12582912.0f + (BITS == 4 ? 8.0f : 0.0f);
@@ -242,7 +244,7 @@ __device__ __forceinline__ RawRow<BITS> quantize_row(const float (&a)[CPL], floa
 #pragma unroll
     for (int t = 0; t < CPL; ++t) {
         const float f = __builtin_fmaf(a[t], r, MAGIC);
-        u[t] = as_u32(__builtin_amdgcn_fmed3f(f, MAGIC - QMAX, MAGIC + QMAX));
+        u[t] = as_u32(CLAMP ? __builtin_amdgcn_fmed3f(f, MAGIC - QMAX, MAGIC + QMAX) : f);
     }
     RawRow<BITS> o;
     if constexpr (BITS == 8) {

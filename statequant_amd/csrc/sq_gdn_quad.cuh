@@ -59,7 +59,7 @@ struct GdnLoads {
 
 template <class T, int NB, int GH, int WPE>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void gdn_quad_kernel(const int32_t* idx, const int32_t* order, int per_xcd, int rows_per_xcd, int hv, int hv_shift,
+void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd, int hv, int hv_shift,
                      const GdnParams p) {
     // the leading arguments (copies of fields of `p`) are what the slot index load needs: as separate scalar
     // arguments they are preloaded into registers at wave launch, so that load goes out first thing
@@ -394,14 +394,17 @@ void gdn_quad_kernel(const int32_t* idx, const int32_t* order, int per_xcd, int 
             cq = alive ? (T::QBUF ? (dec * dq) * us_i : dec * dq) : 0.0f;
             ck = alive ? (T::QBUF ? (dec * dk_) * us_i : dec * dk_) : 0.0f;
         }
+        // every slot's value is fetched up front (one wait for all of them), dead slots then add c = 0 times a finite
+        // int8 value, or are skipped (bf16 values of a dead slot may be NaNs)
+        float uv[MM];
+#pragma unroll
+        for (int i = 0; i < MM; ++i) uv[i] = lds_raw<T::QBUF>(lds_ubr, (i < m ? i : 0) * DV + row);
         float accq = alpha * sq, acck = alpha * sk;
 #pragma unroll
         for (int i = 0; i < MM; ++i) {
-            if (i < n) {                                 // wave-uniform
-                const float uv = lds_raw<T::QBUF>(lds_ubr, i * DV + row);
-                accq = __builtin_fmaf(uv, lane_bcast(cq, i), accq);
-                acck = __builtin_fmaf(uv, lane_bcast(ck, i), acck);
-            }
+            const float u_i = T::QBUF ? uv[i] : (i < n ? uv[i] : 0.0f);
+            accq = __builtin_fmaf(u_i, lane_bcast(cq, i), accq);
+            acck = __builtin_fmaf(u_i, lane_bcast(ck, i), acck);
         }
         const float vt = raw_to_f(vr, p.v_dt);
         const float u = beta * __builtin_fmaf(-a, acck, vt);
@@ -452,6 +455,8 @@ void gdn_quad_kernel(const int32_t* idx, const int32_t* order, int per_xcd, int 
             }
             const float cmul = expf(gnew);
             const int fg = (fq * CL) / T::KGROUP;
+            float kop[DK / 16][MT4];
+            quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lane, kop);
 #pragma unroll
             for (int bi = 0; bi < NB; ++bi) {
                 uint8_t* blk = my_codes + bi * Q::BLK;
@@ -468,8 +473,8 @@ void gdn_quad_kernel(const int32_t* idx, const int32_t* order, int per_xcd, int 
                         uv = decf[t] * uv;
                         bop[t] = sl < m ? uv : 0.0f;
                     }
-                    quad_fold_half<Q, T, false>(blk, hf, lds_kbr, lds_kbsf, nullptr, nullptr, bop, cmul, m,
-                                                f16_to_f32(lds_sc[frow * NG + fg]), A.SCh + frow * NG + fg, lane);
+                    quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
+                                                A.SCh + frow * NG + fg, lane);
                 }
                 wave_sync();
 #pragma unroll

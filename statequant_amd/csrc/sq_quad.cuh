@@ -20,6 +20,8 @@
 // writes (lanes along a row) and the operand-shaped reads (lanes down a column of chunks) are conflict free without
 // padding.
 #pragma once
+#include <type_traits>
+
 #include "sq_tile.cuh"
 #include "sq_params.h"
 
@@ -302,11 +304,33 @@ __device__ __forceinline__ float ubyte_fma(uint32_t w, float s, float o) {
 //                    lds_kd [m][DK]; else the scalar cmul
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// The folded keys as the matrix core's first operand, once per wavefront (they are the same for every half block):
+// kop[ct][t] = kx_{4 t + q}[column (n / 4) CL + 4 ct + n % 4] for lane (n, q); 0 for slots >= m.
+template <class T, bool COLVEC>
+__device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const float* lds_kbsf, const float* lds_kd,
+                                               int m, int lane, float (&kop)[T::DK / 16][(T::MMAX + 3) / 4]) {
+    constexpr int MT4 = (T::MMAX + 3) / 4, CL = T::DK / 4, NT = CL / 4;
+    const int n = lane & 15, q = lane >> 4;
+    const int kcol = (n >> 2) * CL + (n & 3);
+#pragma unroll
+    for (int t = 0; t < MT4; ++t) {
+        const int slot = 4 * t + q;
+        const int sl = slot < m ? slot : 0;
+        const float ks = T::QBUF ? lds_kbsf[sl] : 1.0f;
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct) {
+            float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
+            if constexpr (T::QBUF) kv = kv * ks;
+            if constexpr (COLVEC) kv = kv * lds_kd[sl * T::DK + kcol + 4 * ct];
+            kop[ct][t] = slot < m ? kv : 0.0f;
+        }
+    }
+}
+
 template <class Q, class T, bool COLVEC>
-__device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const uint8_t* lds_kbr, const float* lds_kbsf,
-                                               const float* lds_cv, const float* lds_kd,
-                                               const float (&bop)[(T::MMAX + 3) / 4], float cmul, int m, float s_old,
-                                               uint16_t* sc_out, int lane) {
+__device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float (&kop)[T::DK / 16][(T::MMAX + 3) / 4],
+                                               const float* lds_cv, const float (&bop)[(T::MMAX + 3) / 4], float cmul,
+                                               float s_old, uint16_t* sc_out, int lane) {
     constexpr int MT4 = (T::MMAX + 3) / 4;
     constexpr int CL = T::DK / 4;                            // columns per lane
     constexpr int NT = CL / 4;                               // accumulator tiles per lane
@@ -316,17 +340,20 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const uint8
     constexpr int LPG = T::KGROUP / CL;
     const int n = lane & 15, q = lane >> 4;
     const int row = 16 * hf + n;
+    // where the lane's bytes of the row sit in the LDS image
+    const int at = NBY >= 16 ? swz<Q>(row, q * (NBY / 16)) : swz<Q>(row, q >> 1) + 8 * (q & 1);
+    const int at1 = NBY >= 32 ? swz<Q>(row, q * (NBY / 16) + 1) : at;      // its second chunk (int8, d_k 128)
+    static_assert(NBY <= 32, "at most two chunks per lane");
 
-    // the lane's bytes of the row
     uint32_t w[NW32];
     if constexpr (NBY >= 16) {
 #pragma unroll
         for (int c = 0; c < NBY / 16; ++c) {
-            const uint4 x = *reinterpret_cast<const uint4*>(blk + swz<Q>(row, q * (NBY / 16) + c));
+            const v4u x = *reinterpret_cast<const v4u*>(blk + (c == 0 ? at : at1));
             w[4 * c] = x.x; w[4 * c + 1] = x.y; w[4 * c + 2] = x.z; w[4 * c + 3] = x.w;
         }
     } else {
-        const uint2 x = *reinterpret_cast<const uint2*>(blk + swz<Q>(row, q >> 1) + 8 * (q & 1));
+        const v2u x = *reinterpret_cast<const v2u*>(blk + at);
         w[0] = x.x; w[1] = x.y;
     }
     // dequantize: (code x scale) x factor, one conversion + one fma per code
@@ -360,52 +387,47 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const uint8
         }
     }
     // the m rank-1 updates: first operand = keys (result row i = 4 q' + b <-> column q' CL + 4 ct + b), second = values
-    const int kcol = (n >> 2) * CL + (n & 3);
-#pragma unroll
-    for (int ct = 0; ct < NT; ++ct) {
-#pragma unroll
-        for (int t = 0; t < MT4; ++t) {
-            const int slot = 4 * t + q;
-            const int sl = slot < m ? slot : 0;
-            float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
-            if constexpr (T::QBUF) kv = kv * lds_kbsf[sl];
-            if constexpr (COLVEC) kv = kv * lds_kd[sl * T::DK + kcol + 4 * ct];
-            kv = slot < m ? kv : 0.0f;
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv, bop[t], acc[ct], 0, 0, 0);
-        }
-    }
-    // absmax of the lane's columns, then of its scale group
-    float mx = 0.0f;
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) mx = fmaxf(mx, fabsf(acc[ct][b]));
+        for (int t = 0; t < MT4; ++t)
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop[ct][t], bop[t], acc[ct], 0, 0, 0);
+    // absmax of the lane's columns (three-operand maxima), then of its scale group
+    float mx = 0.0f;
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct) {
+        mx = fmaxf(fmaxf(mx, fabsf(acc[ct][0])), fabsf(acc[ct][1]));
+        mx = fmaxf(fmaxf(mx, fabsf(acc[ct][2])), fabsf(acc[ct][3]));
+    }
     if constexpr (LPG >= 2) { const Pair pm = pair16(mx); mx = fmaxf(pm.lo, pm.hi); }
     if constexpr (LPG >= 4) { const Pair pm = pair32(mx); mx = fmaxf(pm.lo, pm.hi); }
     const float sc = fp16_scale(mx, T::QMAX);
     const float rs = 1.0f / sc;
     if (q % LPG == 0) *sc_out = f32_to_f16(sc);
-    // new codes, back into the LDS image
-    if constexpr (NBY >= 16) {
+    // new codes, back into the LDS image.  A scale in fp16's normal range cannot push a quotient past qmax + 1/2, so
+    // the clamp is only compiled into the path taken when some lane's scale is subnormal (or at its floor).
+    auto requantize = [&](auto clamp) {
+        constexpr bool CLAMP = decltype(clamp)::value;
+        if constexpr (NBY >= 16) {
 #pragma unroll
-        for (int c = 0; c < CL / 16; ++c) {                  // 16 columns per call
+            for (int c = 0; c < CL / 16; ++c) {              // 16 columns per call
+                float a16[CPL];
+#pragma unroll
+                for (int e = 0; e < CPL; ++e) a16[e] = acc[4 * c + e / 4][e % 4];
+                const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP>(a16, rs);
+                if constexpr (T::BITS == 8) *reinterpret_cast<uint4*>(blk + (c == 0 ? at : at1)) = r.v;
+                else *reinterpret_cast<uint2*>(blk + at + 8 * c) = r.v;      // 16 columns = half a chunk
+            }
+        } else {
             float a16[CPL];
 #pragma unroll
-            for (int e = 0; e < CPL; ++e) a16[e] = acc[4 * c + e / 4][e % 4];
-            const RawRow<T::BITS> r = quantize_row<T::BITS>(a16, rs);
-            if constexpr (T::BITS == 8) {
-                *reinterpret_cast<uint4*>(blk + swz<Q>(row, q * (NBY / 16) + c)) = r.v;
-            } else {                                         // 16 columns = 8 bytes = half a chunk
-                *reinterpret_cast<uint2*>(blk + swz<Q>(row, q * (NBY / 16) + c / 2) + 8 * (c & 1)) = r.v;
-            }
+            for (int e = 0; e < CPL; ++e) a16[e] = acc[e / 4][e % 4];
+            const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP>(a16, rs);
+            *reinterpret_cast<uint2*>(blk + at) = r.v;
         }
-    } else {
-        float a16[CPL];
-#pragma unroll
-        for (int e = 0; e < CPL; ++e) a16[e] = acc[e / 4][e % 4];
-        const RawRow<T::BITS> r = quantize_row<T::BITS>(a16, rs);
-        *reinterpret_cast<uint2*>(blk + swz<Q>(row, q >> 1) + 8 * (q & 1)) = r.v;
-    }
+    };
+    if (__builtin_amdgcn_ballot_w64(sc < 6.103515625e-05f) != 0) requantize(std::true_type{});
+    else requantize(std::false_type{});
 }
 
 }  // namespace sq
