@@ -73,7 +73,7 @@ CASES = _cases()
 GGA_SHAPES = [(128, 128), (64, 64)]                  # (d_k, d_v) of the mixed-width GGA / STEP slot (sq_gga.cuh)
 PARAMS = {'gdn': 'GdnParams', 'kda': 'KdaParams', 'mamba2': 'Mamba2Params'}
 # families with a workgroup-per-key-head kernel (sq_<family>_quad.cuh) -> value heads per workgroup that are built
-QUAD_FAMILIES = {'gdn': (2, 1)}
+QUAD_FAMILIES = {'gdn': (2, 1), 'mamba2': (4, 2, 1)}
 CHUNK = 6                                            # instances per translation unit
 
 
@@ -85,13 +85,21 @@ def _tile(c):
 
 # Run-time conditions of the workgroup-per-key-head kernels, per family (part of the generated dispatch unit).
 QUAD_OK = {'gdn': [
-    '// q, k per key head (or ungrouped keys), rows that 32-bit vector loads can address',
+    '// q, k per key head (or ungrouped keys), rows that 16-byte vector loads can address',
     'static bool gdn_quad_ok(const GdnParams& p) {',
     '    if (!p.qk_per_key_head && p.gqa > 1) return false;',
     '    auto ok = [](const void* ptr, uint32_t stride, int dt) {',
-    '        return dt == 0 || ((reinterpret_cast<uintptr_t>(ptr) % 4) == 0 && stride % 2 == 0);',
+    '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
     '    };',
     '    return ok(p.q, p.s_q, p.q_dt) && ok(p.k, p.s_k, p.k_dt);',
+    '}'],
+    'mamba2': [
+    '// B, C rows that 16-byte vector loads can address',
+    'static bool mamba2_quad_ok(const Mamba2Params& p) {',
+    '    auto ok = [](const void* ptr, uint32_t stride, int dt) {',
+    '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
+    '    };',
+    '    return ok(p.B, p.s_B, p.B_dt) && ok(p.C, p.s_C, p.C_dt);',
     '}']}
 
 
@@ -191,7 +199,7 @@ def generate():
         d.append(f'int dispatch_{fam}(const {P}& p, hipStream_t stream, bool run) {{')
         if fam in QUAD_FAMILIES:
             d.append(f'    const bool quad = !getenv("SQ_NO_QUAD") && (!run || {fam}_quad_ok(p));')
-            d.append('    const int ghmax = getenv("SQ_GH1") ? 1 : 64;')
+            d.append('    const int ghmax = getenv("SQ_GHMAX") ? atoi(getenv("SQ_GHMAX")) : 64;')
         # smallest sufficient buffer bound first
         for c in sorted(rows, key=lambda c: c[5]):
             bits, dk, dv, group, qbuf, mmax, axv = c

@@ -148,24 +148,24 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
             for (int t = 0; t < Q::NLD; ++t)
-                F.cw[bi][t] = *reinterpret_cast<const v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16);
+                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-            for (int g = 0; g < NG; ++g) F.sc[bi][g] = A.SCh[uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g)];
+            for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(A.SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
         // buffered values of this wavefront's rows, every slot: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
 #pragma unroll
         for (int t = 0; t < Q::UT; ++t) {
             const uint32_t i = lane / Q::LU + Q::SU * t;
             const uint32_t ic = i < uint32_t(m) ? i : uint32_t(m) - 1;
-            F.uraw[t] = load_raw4<T::QBUF>(A.buf.UB + (ic * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE);
+            F.uraw[t] = stream_raw4<T::QBUF>(A.buf.UB + (ic * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE);
         }
         // buffered keys, dealt over the workgroup: lane (slot = SPP (NW t + w) + lane / LPS, columns 4 (lane % LPS) ..)
 #pragma unroll
         for (int t = 0; t < Q::KT; ++t) {
             const uint32_t i = Q::SPP * (NW * t + w) + lane / Q::LPS;
             const uint32_t ic = i < uint32_t(m) ? i : uint32_t(m) - 1;
-            F.kraw[t] = load_raw4<T::QBUF>(A.buf.KB + (ic * DK + 4 * (lane % Q::LPS)) * T::BE);
+            F.kraw[t] = stream_raw4<T::QBUF>(A.buf.KB + (ic * DK + 4 * (lane % Q::LPS)) * T::BE);
             F.kbs[t] = T::QBUF ? A.buf.KBS[ic] : uint16_t(0);
         }
         // per slot of this head, lane i: cumulative decay and value scale
@@ -479,8 +479,8 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
                 wave_sync();
 #pragma unroll
                 for (int t = 0; t < Q::NLD; ++t)
-                    *reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16) =
-                        *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0);
+                    stream_store(reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16),
+                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
             }
         }
         }

@@ -241,10 +241,6 @@ __device__ __forceinline__ float quad_block_pass(const uint8_t* blk, const v4i (
     return s;
 }
 
-// Native vector types for values that stay in registers across the load / use distance (the compiler keeps arrays of
-// HIP's uint4 / uint2 structs in scratch memory when an asm statement separates their loads from their uses).
-typedef uint32_t v4u __attribute__((ext_vector_type(4)));
-typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 // Raw buffered elements: four per lane.
 template <bool QBUF> struct Raw4;
@@ -255,6 +251,13 @@ __device__ __forceinline__ Raw4<QBUF> load_raw4(const uint8_t* p) {
     Raw4<QBUF> r;
     if constexpr (QBUF) r.a = *reinterpret_cast<const uint32_t*>(p);
     else r.a = *reinterpret_cast<const v2u*>(p);
+    return r;
+}
+template <bool QBUF>
+__device__ __forceinline__ Raw4<QBUF> stream_raw4(const uint8_t* p) {       // the same through `stream_load`
+    Raw4<QBUF> r;
+    if constexpr (QBUF) r.a = stream_load(reinterpret_cast<const uint32_t*>(p));
+    else r.a = stream_load(reinterpret_cast<const v2u*>(p));
     return r;
 }
 template <bool QBUF>

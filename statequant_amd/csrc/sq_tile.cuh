@@ -310,7 +310,7 @@ __device__ __forceinline__ bool rows_inside(int first) { return !T::RAGV || firs
 template <class T>
 __device__ __forceinline__ RawRow<T::BITS> load_rows(const uint8_t* lane_base, int first) {
     if (!rows_inside<T>(first)) return zero_row<T::BITS>();
-    return load_row<T::BITS>(lane_base + first * T::ROW_BYTES);
+    return stream_row<T::BITS>(lane_base + first * T::ROW_BYTES);
 }
 template <class T>
 __device__ __forceinline__ void store_rows(uint8_t* lane_base, int first, const RawRow<T::BITS>& r) {
