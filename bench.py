@@ -10,15 +10,22 @@ of the fused step kernel through the C ABI (``SlotLayout.step`` -> ``sq_gdn_step
 state and advance in lockstep, so one step in m folds and re-quantizes every state tile (the reference's benchmark does
 the same: benchmarks/decode_state.py:41-66 there times graphs of m steps = one fold).
 
-Timing: W untimed warm-up steps, then exactly K steps between ``torch.cuda.synchronize()`` calls on the wall clock
-(``ms_per_step``), with HIP events on the launch stream around the same region.  The steps are replayed from a HIP
-graph of m steps (m x 24 kernel nodes) when K and W are multiples of m, otherwise launched eagerly.
+Timing: whole fold periods only.  K and W are rounded up to multiples of m (``config.steps_requested`` keeps K;
+``steps`` is what was timed), so every timed window holds exactly steps / m folds whatever K is; W untimed warm-up
+steps, then the timed steps between ``torch.cuda.synchronize()`` calls on the wall clock (``ms_per_step``), with HIP
+events on the launch stream around the same region.  The steps are replayed from a HIP graph of m steps (m x 24
+kernel nodes) unless ``--no-graph``.
 
 Prints ONE JSON line.  ``value`` = microseconds per layer per decode step (lower is better).  ``roofline`` prices the
 step kernel against HBM: achieved = algorithmic state bytes per launch / average launch duration, where the
 algorithmic bytes are (codes + scales) x (1 + 1/m) per slot (read every step, rewritten once per m steps) x slots.
+``roofline.total`` prices the same duration against every byte the step has to move (state, live buffer slots,
+appends, counters, inputs, output).  ``roofline.traffic`` is the HBM traffic per launch that profile_step.py measured
+with rocprofv3 counters (read from profiles/hbm_traffic.json: a separate run, not this one; null if none).
 ``cpu_baseline`` times the CPU oracle (a torch restatement of the reference's own CPU path) on this box's host cores
-on a bounded sample of the same workload; it is a reported baseline, not a target.
+on a bounded sample of the same workload, and ``cpu_baseline_c1`` the same oracle on the reference's own CPU-runnable
+configuration (4 sequences, 4 / 2 heads, d 64, int8 group 64, bf16 buffer, m 8, 64 steps); reported baselines, not
+targets.
 
 Secondary figures: ``--workload`` (the other formats and families; ``gga4-pw8`` is the mixed-width GGA / STEP slot,
 which re-fits every head at every token), ``--slots N`` (other batch sizes), ``--op write |
@@ -70,9 +77,15 @@ def describe_state(bits, group):
         return 'bf16, unquantized'
     return f'int{bits} {"value" if group < 0 else "key"}-axis group {abs(group)}, fp16 scales'
 
-# HBM bytes per launch of the step kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (average
-# over the steps of one fold period), scaled by a copy kernel of known size; None until measured (profiles/).
-MEASURED_TRAFFIC = {'gdn-int8-g128': 185332412, 'gga4-pw8': 184491520}
+
+def measured_traffic(workload):
+    """HBM bytes per launch (read + written, averaged over a fold period) that profile_step.py measured for the
+    workload with rocprofv3 FETCH_SIZE / WRITE_SIZE, from the table it keeps; None if it holds no such row."""
+    path = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+    if not os.path.exists(path):
+        return None
+    row = json.load(open(path)).get(workload)
+    return row['traffic'] if row else None
 
 
 def stored_bytes_per_slot(bits, group, hv, dk, dv):
@@ -85,6 +98,25 @@ def stored_bytes_per_slot(bits, group, hv, dk, dv):
 
 def state_bytes_per_slot(bits, group, hv, dk, dv, m):
     return stored_bytes_per_slot(bits, group, hv, dk, dv) * (1 + 1 / m)
+
+
+def total_bytes_per_slot(fam, bits, group, hv, hk, dk, dv, m, in_bytes=2, out_bytes=2, be=1):
+    """Every byte one decode step of one slot has to move, averaged over a fold period: the state as above; the live
+    part of the decode buffer ((m - 1) / 2 slots on average: values, keys, their scales, cumulative decays); the
+    append of one slot; counters and running decay read and written; the token's inputs and its output.  KDA keeps
+    the decays per key channel (fp32 [m, d_k] per head), which is why its total is far above its state bytes."""
+    live = (m - 1) / 2
+    gdim = dk if fam == 'kda' else 1                          # decay entries per (head, slot)
+    per_slot = hv * dv * be + hk * dk * be + (hv + hk) * 2 + hv * gdim * 4      # one buffer slot: u, k, scales, G
+    counters = 2 * (hv * gdim * 4 + hv * 4)                                     # GCUR, NPTR: read + write
+    if fam == 'gdn':
+        inputs = 2 * hk * dk * in_bytes + hv * dv * in_bytes + 2 * hv * 4
+    elif fam == 'kda':
+        inputs = 2 * hv * dk * in_bytes + hv * dk * 4 + hv * dv * in_bytes + hv * 4
+    else:
+        inputs = 2 * hk * dk * in_bytes + hv * dv * in_bytes + hv * 4 + 3 * hv * 4 / 128
+    return (state_bytes_per_slot(bits, group, hv, dk, dv, m) + live * per_slot + per_slot + counters + inputs
+            + hv * dv * out_bytes)
 
 
 def build(workload, m, device):
@@ -178,6 +210,28 @@ def cpu_baseline(workload, m, budget_s=20.0):
                       f'torch CPU oracle, {cores} threads'}
 
 
+def cpu_baseline_c1():
+    """The CPU oracle on the reference's own CPU-runnable configuration, whole: 4 sequences, 4 value / 2 key heads,
+    d_k = d_v = 64, int8 state in groups of 64, bf16 decode buffer of m = 8, 64 steps from a zero state, seed 0."""
+    from oracle import states as ST
+    B, hv, hk, d, m, steps = 4, 4, 2, 64, 8, 64
+    torch.set_num_threads(1)
+    gen = torch.Generator().manual_seed(0)
+    r = lambda *s: torch.randn(*s, generator=gen)          # noqa: E731
+    st = ST.GDNOracle(torch.zeros(B * hv, d, d), (8, 'k', 64), m=m, hv=hv, hk=hk, buffer_bits=16)
+    t_total = 0.0
+    for _ in range(steps):
+        args = (r(B * hk, d).bfloat16(), r(B * hk, d).bfloat16(), r(B * hv, d).bfloat16(),
+                -torch.nn.functional.softplus(r(B * hv)), torch.sigmoid(r(B * hv)), d ** -0.5)
+        t0 = time.perf_counter()
+        st.step(*args)
+        t_total += time.perf_counter() - t0
+    torch.set_num_threads(os.cpu_count() or 1)
+    return {'value': round(t_total / steps * 1e6, 1), 'unit': 'us per layer-step', 'cores': 1, 'kind': 'port',
+            'sample': f'reference CPU case: {B} sequences x {hv}/{hk} heads x {d} x {d}, int8 g64, bf16 buffer, m={m}, '
+                      f'{steps} steps from zero, torch CPU oracle, 1 thread'}
+
+
 def gga_plan(hv, dk, layers, seed=0):
     """A synthetic plan at a mean of 4 bits with one fp16 pivot per layer (charged 8 bits, as the method's allocator
     does): 12 x 2, 11 x 4, 6 x 6, 2 x 8 bits and the pivot over the 32 heads, shuffled per layer."""
@@ -224,7 +278,10 @@ def bench_gga(a, dev):
                 i = inputs[s * layers + L]
                 pk.step(views[L], idx, i['q'], i['k'], i['v'], out, dk ** -0.5, gate=(i['a'], i['b'], A_log, dtb), layer=L)
 
-    use_graph = not a.no_graph and a.steps % period_len == 0 and a.warmup % period_len == 0 and a.steps > 0
+    requested = (a.steps, a.warmup)
+    a.steps = max(-(-a.steps // period_len), 1) * period_len          # whole graphs of period_len steps
+    a.warmup = -(-a.warmup // period_len) * period_len
+    use_graph = not a.no_graph
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         period()
@@ -245,7 +302,7 @@ def bench_gga(a, dev):
         e1.record(stream)
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-    steps = a.steps if use_graph else -(-a.steps // period_len) * period_len
+    steps = a.steps
     assert torch.isfinite(out.float()).all(), 'non-finite output'
     n_launch = steps * layers
     us_wall, us_kernel = wall * 1e6 / n_launch, e0.elapsed_time(e1) * 1e3 / n_launch
@@ -259,11 +316,14 @@ def bench_gga(a, dev):
                    'value_heads': hv, 'key_heads': hk, 'd_k': dk, 'd_v': dv,
                    'state': f'per-head widths 2/4/6/8 bit + one fp16 pivot per layer, {pk.bits_per_value():.3f} bits '
                             f'per value with the window', 'window': f'FP8 pairs, m={m}', 'inputs': 'bf16',
-                   'launch': 'hip-graph' if use_graph else 'eager', 'bytes_per_slot': pk.nbytes,
+                   'launch': 'hip-graph' if use_graph else 'eager', 'steps_requested': requested[0],
+                   'warmup_requested': requested[1], 'steps_timed': steps, 'folds_timed': None,
+                   'bytes_per_slot': pk.nbytes,
                    'algorithmic_bytes_per_slot_step': round(alg / slots)},
         'hbm_gbs': round(achieved, 1),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(a.workload),
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': measured_traffic(a.workload),
+                     'traffic_source': 'profiles/hbm_traffic.json (rocprofv3 run of profile_step.py, not this run)',
                      'kernel_us': round(us_kernel, 3), 'algorithmic_bytes_per_launch': round(alg)},
     }
     if not a.no_cpu_baseline:
@@ -417,7 +477,10 @@ def main():
             for L in range(layers):
                 launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out, order)
 
-    use_graph = not a.no_graph and a.steps % m == 0 and a.warmup % m == 0 and a.steps > 0
+    requested = (a.steps, a.warmup)
+    a.steps = max(-(-a.steps // m), 1) * m                  # whole fold periods, so that any K times steps / m folds
+    a.warmup = -(-a.warmup // m) * m
+    use_graph = not a.no_graph
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         if use_graph:
@@ -451,6 +514,8 @@ def main():
     us_kernel = ev_ms * 1e3 / n_launch                      # average launch-to-launch duration on the stream
     alg_bytes = state_bytes_per_slot(bits, group, hv, dk, dv, m) * slots
     achieved = alg_bytes / (us_kernel * 1e-6) / 1e9
+    tot_bytes = total_bytes_per_slot(fam, bits, group, hv, hk, dk, dv, m) * slots
+    tot_gbs = tot_bytes / (us_kernel * 1e-6) / 1e9
     res = {
         'metric': 'us_per_layer_decode_step', 'value': round(us_wall, 3), 'unit': 'us',
         'n_gpus': 1, 'steps': a.steps, 'warmup': a.warmup, 'ms_per_step': round(wall * 1e3 / a.steps, 5),
@@ -458,16 +523,23 @@ def main():
         'config': {'workload': a.workload, 'family': fam, 'slots': slots, 'layers': layers, 'value_heads': hv,
                    'key_heads': hk, 'd_k': dk, 'd_v': dv, 'state': describe_state(bits, group),
                    'buffer': f'int8, m={m}', 'inputs': 'bf16', 'launch': 'hip-graph' if use_graph else 'eager',
+                   'steps_requested': requested[0], 'warmup_requested': requested[1], 'steps_timed': a.steps,
+                   'folds_timed': a.steps // m if not a.mixed_fill else None,
                    'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
                    'dispatch_order': 'folding rows first' if a.fold_first else 'natural',
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(a.workload),
-                     'kernel_us': round(us_kernel, 3), 'algorithmic_bytes_per_launch': round(alg_bytes)},
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': measured_traffic(a.workload),
+                     'traffic_source': 'profiles/hbm_traffic.json (rocprofv3 run of profile_step.py, not this run)',
+                     'kernel_us': round(us_kernel, 3), 'algorithmic_bytes_per_launch': round(alg_bytes),
+                     'total': {'bytes_per_launch': round(tot_bytes), 'achieved': round(tot_gbs, 1),
+                               'frac': round(tot_gbs / HBM_PEAK_GBS, 4),
+                               'counts': 'state + live buffer slots + append + counters + inputs + output'}},
     }
     if not a.no_cpu_baseline:
         res['cpu_baseline'] = cpu_baseline(a.workload, m, a.cpu_budget)
+        res['cpu_baseline_c1'] = cpu_baseline_c1()
     print(json.dumps(res))
 
 

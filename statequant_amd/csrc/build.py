@@ -128,7 +128,9 @@ def quad_variants(fam, c):
         wgs = min(160 * 1024 // lds, 32 // nw)
         if wgs < 1:
             continue
-        out.append((nb, gh, max(1, min(7, -(-wgs * nw // 4)))))
+        # register target: as many wavefronts per SIMD as LDS lets workgroups in, up to 6 (5 with the 16-token buffer);
+        # asked for 7, the int4 kernels spill into scratch memory inside the fold (measured: +60 % bytes written)
+        out.append((nb, gh, max(1, min(6 if mmax <= 8 else 5, -(-wgs * nw // 4)))))
     return out
 
 
@@ -311,11 +313,54 @@ def build(jobs=None, force=False, verbose=True):
     return LIB
 
 
+_REMARK = re.compile(r'remark: +(Function Name|VGPRs|AGPRs|SGPRs Spill|VGPRs Spill|ScratchSize \[bytes/lane\]|'
+                     r'Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]): +(\S+)')
+
+
+def resources(pattern='', jobs=None):
+    """Print one line per compiled kernel: what the compiler's -Rpass-analysis=kernel-resource-usage remarks state
+    for it (device pass only, nothing is linked).  VGPRs and AGPRs share one file of 512 registers per SIMD lane."""
+    jobs = jobs or min(16, os.cpu_count() or 4)
+    units = [u for u in generate() if not u.endswith(('dispatch.hip', 'sq_api.hip'))]
+
+    def one(src):
+        cmd = ['hipcc', *HIPCC_FLAGS, '--cuda-device-only', '-Rpass-analysis=kernel-resource-usage', '-c', src,
+               '-o', os.devnull]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        rows, cur = [], None
+        for key, val in _REMARK.findall(r.stderr):
+            if key == 'Function Name':
+                cur = {'name': val}
+                rows.append(cur)
+            elif cur is not None:
+                cur[key] = val
+        return rows
+
+    with cf.ThreadPoolExecutor(jobs) as ex:
+        rows = [r for unit in ex.map(one, units) for r in unit]
+    demangle = subprocess.run(['c++filt'], input='\n'.join(r['name'] for r in rows), capture_output=True, text=True)
+    names = demangle.stdout.split('\n') if demangle.returncode == 0 else [r['name'] for r in rows]
+    print('VGPR AGPR spill(V/S) scratch occupancy   LDS  kernel')
+    for r, n in sorted(zip(rows, names), key=lambda x: x[1]):
+        n = n.replace('sq::', '').replace('void ', '')
+        n = n[:n.index('>(') + 1] if '>(' in n else n
+        if pattern in n:
+            print(f"{r.get('VGPRs', '?'):>4} {r.get('AGPRs', '?'):>4} {r.get('VGPRs Spill', '?'):>5}/{r.get('SGPRs Spill', '?'):<3} "
+                  f"{r.get('ScratchSize [bytes/lane]', '?'):>6} {r.get('Occupancy [waves/SIMD]', '?'):>8} "
+                  f"{r.get('LDS Size [bytes/block]', '?'):>6}  {n}")
+
+
 if __name__ == '__main__':
     ap = argparse.ArgumentParser()
     ap.add_argument('-j', type=int, default=None)
     ap.add_argument('--force', action='store_true')
+    ap.add_argument('--resources', metavar='PATTERN', nargs='?', const='', default=None,
+                    help="instead of building, print the compiler's resource usage (registers, spills, LDS, "
+                         'occupancy) of every kernel whose name contains PATTERN')
     a = ap.parse_args()
+    if a.resources is not None:
+        resources(a.resources, a.j)
+        sys.exit(0)
     try:
         build(a.j, a.force)
     except RuntimeError as e:

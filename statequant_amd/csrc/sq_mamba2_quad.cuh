@@ -130,23 +130,27 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
         for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
-    // buffered values of this wavefront's rows, every slot: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
+    // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count, a
+    // scalar load issued ahead of everything above, is here by now
+    const uint32_t nfill = uint32_t(F.np & (m - 1));
+    const uint32_t nl = nfill > 0 ? nfill : 1u;
+    // buffered values of this wavefront's rows: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
 #pragma unroll
     for (int t = 0; t < Q::UT; ++t) {
         const uint32_t i = lane / Q::LU + Q::SU * t;
-        const uint32_t ic = i < um ? i : um - 1;
+        const uint32_t ic = i < nl ? i : nl - 1;
         F.uraw[t] = stream_raw4<T::QBUF>(UBp + (ic * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE);
     }
     // buffered keys, dealt over the workgroup: lane (slot = SPP (NW t + w) + lane / LPS, columns 4 (lane % LPS) ..)
 #pragma unroll
     for (int t = 0; t < Q::KT; ++t) {
         const uint32_t i = Q::SPP * (NW * t + w) + lane / Q::LPS;
-        const uint32_t ic = i < um ? i : um - 1;
+        const uint32_t ic = i < nl ? i : nl - 1;
         F.kraw[t] = stream_raw4<T::QBUF>(KBp + (ic * DK + 4 * (lane % Q::LPS)) * T::BE);
         F.kbs[t] = T::QBUF ? KBSp[ic] : uint16_t(0);
     }
     {   // per slot of this head, lane i: cumulative decay and value scale
-        const uint32_t li = uint32_t(lane) < um ? lane : 0;
+        const uint32_t li = uint32_t(lane) < nl ? lane : 0;
         F.gbl = GBh[li];
         F.ubs = T::QBUF ? UBSp[li] : uint16_t(0);
     }
