@@ -162,7 +162,11 @@ __global__ __launch_bounds__(WAVE) void read_kernel(const ReadParams p) {
     const uint32_t hk = h / uint32_t(p.gqa);
     float* out = p.out + (uint64_t(b) * p.s_out + uint64_t(h) * dv * DK);
     const int32_t slot = p.idx ? p.idx[b] : int32_t(b);
-    if (p.idx && slot <= 0) return;
+    if (p.idx && slot <= 0) {                                      // padding row: a zero state, nothing of a slot read
+        float4* o4 = reinterpret_cast<float4*>(out);
+        for (uint32_t e = l.lane; e < dv * DK / 4; e += WAVE) o4[e] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        return;
+    }
     const uint32_t seq = slot;
     const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (dv * T::ROW_BYTES));
     const uint16_t* SCh = field(p.st.SC, seq, p.st.sSC, AXV ? h * ((dv / GROUP) * DK) : h * (dv * T::NG));

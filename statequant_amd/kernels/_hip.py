@@ -189,32 +189,24 @@ def check(rc):
 def pack_into(lay, src, S, sS, SC, sSC, idx=None, GCUR=None, sGC=0, gcur_per_head=1, NPTR=None, sN=0):
     """``sq_pack_vk``: fp32 value-major ``src`` [rows, hv, dv, dk] (contiguous) -> codes ``S`` / scales ``SC`` (None
     for an unquantized state, which is cast) of the sequences ``idx`` (int32; None: sequence b), optionally emptying
-    their buffers.  Returns False when the library has
-    no instance for the format (the caller then packs with torch), raises on any other error."""
+    their buffers.  Raises when the library has no instance for the format, like every other error: GPU tensors never
+    take another path."""
     assert src.dtype == torch.float32 and src.is_contiguous()
     rows = src.shape[0]
     a = SqPackArgs(lay=lay, rows=rows, idx=ptr(idx), src=src.data_ptr(), s_src=src.stride(0) if rows else 0,
                    S=S.data_ptr(), sS=sS, SC=ptr(SC), sSC=sSC, GCUR=ptr(GCUR), sGC=sGC,
                    gcur_per_head=gcur_per_head, NPTR=ptr(NPTR), sN=sN)
-    rc = lib().sq_pack_vk(C.byref(a), current_stream(src.device))
-    if rc == E_UNSUPPORTED:
-        return False
-    check(rc)
-    return True
+    check(lib().sq_pack_vk(C.byref(a), current_stream(src.device)))
 
 
 def read_state(lay, T, strides, nptr_stride, idx, out, kda):
-    """``sq_read``: the current state of sequences ``idx`` (int32) into fp32 ``out`` [rows, hv, dv, dk] (contiguous).
-    Returns False when the library has no instance for the layout."""
+    """``sq_read``: the current state of sequences ``idx`` (int32) into fp32 ``out`` [rows, hv, dv, dk] (contiguous);
+    rows with ``idx <= 0`` come back as zeros.  Raises when the library has no instance for the layout."""
     assert out.dtype == torch.float32 and out.is_contiguous()
     rows = out.shape[0]
     a = SqReadArgs(st=make_state(T, strides, nptr_stride), lay=lay, kda=int(kda), rows=rows, idx=ptr(idx),
                    out=out.data_ptr(), s_out=out.stride(0) if rows else 0)
-    rc = lib().sq_read(C.byref(a), current_stream(out.device))
-    if rc == E_UNSUPPORTED:
-        return False
-    check(rc)
-    return True
+    check(lib().sq_read(C.byref(a), current_stream(out.device)))
 
 
 def fold_first(idx, nptr, m, out=None):
@@ -233,3 +225,13 @@ def require_gpu(t, what):
     if not t.is_cuda:
         raise RuntimeError(f'{what}: the packed decode step runs on the GPU only (HIP kernels, no fallback); '
                            f'got a tensor on {t.device}')
+
+
+def same_device(what, ref, **tensors):
+    """Raise unless ``ref`` is on a GPU and every given tensor (None: skipped) is on that same device.  The kernels
+    receive raw pointers: a host tensor among them would be a GPU memory fault, not a Python error, so every wrapper
+    calls this before it takes a pointer."""
+    require_gpu(ref, what)
+    for name, t in tensors.items():
+        if t is not None and t.device != ref.device:
+            raise RuntimeError(f'{what}: `{name}` is on {t.device}, the state on {ref.device}')

@@ -106,8 +106,8 @@ def pack_vk(x, fmt):
                          dtype=torch.float16)
         lay = _hip.SqLayout(bits=fmt.bits, axis_k=int(fmt.axis == 'k'), group=g, buffer_bits=8, m=1, hv=1, hk=1,
                             dk=dk, dv=dv)
-        if _hip.pack_into(lay, x.contiguous().view(n, 1, dv, dk), codes, codes[0].numel(), sc, sc[0].numel()):
-            return codes, sc
+        _hip.pack_into(lay, x.contiguous().view(n, 1, dv, dk), codes, codes[0].numel(), sc, sc[0].numel())
+        return codes, sc
     if fmt.axis == 'k':
         ng = -(-dk // g)
         xg = torch.nn.functional.pad(x, (0, ng * g - dk)).view(n, dv, ng, g)       # zero pad: same absmax
@@ -233,6 +233,7 @@ class PackedGDNState(LockstepState):
             assert q.shape[0] == self.B * HK and k.shape[0] == self.B * HK
         for t in (q, k, v, g, beta):
             assert t.is_contiguous()
+        _hip.same_device('PackedGDNState.step', self.O, q=q, k=k, v=v, g=g, beta=beta)
         sqk = (HK if per_key else HV) * self.DK
         a = _hip.SqGdnArgs(
             st=_hip.make_state(self._T, self._strides, HV), lay=self._lay, rows=self.B, idx=None,

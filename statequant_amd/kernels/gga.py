@@ -147,6 +147,9 @@ class GGAPacked:
         assert out.is_contiguous() and idx.dtype == torch.int32 and idx.is_contiguous()
         assert out.shape[0] >= B and tuple(out.shape[1:]) == (self.HV, self.DV)
         blob = views['blob']
+        ga, gb, A_log, dt_bias = gate if gate is not None else (None,) * 4
+        _hip.same_device('GGAPacked.step', blob, idx=idx, q=q, k=k, v=v, out=out, g=g, beta=beta, a=ga, b=gb,
+                         A_log=A_log, dt_bias=dt_bias)
         a = _hip.SqGgaArgs(sl=self._slots(blob, layer), rows=B, idx=idx.data_ptr(),
                            q=q.data_ptr(), s_q=q.stride(0), q_dtype=_hip.dtype_code(q),
                            k=k.data_ptr(), s_k=k.stride(0), k_dtype=_hip.dtype_code(k),
@@ -171,11 +174,11 @@ class GGAPacked:
     @torch.no_grad()
     def stored(self, views, idx, layer):
         """The stored states of slots idx, canonical fp32 [P, HV, d_k, d_v] (without the window)."""
-        idx32 = idx.to(torch.int32).contiguous()
+        blob = views['blob']
+        idx32 = idx.to(device=blob.device, dtype=torch.int32).contiguous()
         P = idx32.shape[0]
-        Y = torch.empty(P, self.HV, self.DK, self.DV, device=idx.device)
+        Y = torch.empty(P, self.HV, self.DK, self.DV, device=blob.device)
         if P:
-            blob = views['blob']
             sl = self._slots(blob, layer)
             _hip.check(_hip.lib().sq_gga_load(C.byref(sl), idx32.data_ptr(), P, Y.data_ptr(),
                                               _hip.current_stream(blob.device)))
@@ -184,9 +187,11 @@ class GGAPacked:
     @torch.no_grad()
     def window(self, views, idx):
         """The queued pairs of slots idx as reconstructed fp32 (P [n, m, HV, d_k], V [n, m, HV, d_v]) in ring order
-        from the oldest, and the counts n [n]; dead entries zeroed."""
+        from the oldest, and the counts n [n].  Dead entries are SELECTED away, never multiplied by zero: the store
+        kernel resets the two counters only, so on a page that was not zero-filled a dead entry may decode to NaN
+        (FP8 0x7F / 0xFF) or carry a non-finite scale."""
         m, HV, DK, DV = self.m, self.HV, self.DK, self.DV
-        rows = views['blob'].index_select(0, idx.long())
+        rows = views['blob'].index_select(0, idx.to(views['blob'].device).long())
         counters = rows[:, :8].contiguous().view(torch.int32)                  # n, ring position of the oldest
         count, oldest = counters[:, 0], counters[:, 1]
         win = rows[:, self.QOFF:self.QOFF + HV * self.QSZ].unflatten(1, (HV, self.QSZ))
@@ -205,7 +210,7 @@ class GGAPacked:
 
         def by_age(x):                                                          # [n, HV, m, d] -> [n, m, HV, d]
             picked = torch.stack([x[i, :, ring[i]] for i in range(x.shape[0])]) if x.shape[0] else x
-            return picked.transpose(1, 2) * alive
+            return torch.where(alive, picked.transpose(1, 2), torch.zeros((), device=x.device))
 
         return by_age(left), by_age(right), count
 
@@ -215,20 +220,22 @@ class GGAPacked:
         state = self.stored(views, idx, layer)                                 # [P, HV, d_k, d_v]
         if self.pw and idx.numel():
             left, right, _ = self.window(views, idx)
-            widths = self._plan(layer, idx.device)[1]
-            coded = (widths != 16).to(state.dtype).view(1, -1, 1, 1)           # pivots keep no window
-            state = state + coded * torch.einsum('pmhk,pmhv->phkv', left, right)
+            widths = self._plan(layer, state.device)[1]
+            coded = (widths != 16).view(1, 1, -1, 1)                           # pivots keep no window: whatever
+            left = torch.where(coded, left, torch.zeros((), device=left.device))      # their bytes hold is dropped
+            right = torch.where(coded, right, torch.zeros((), device=right.device))
+            state = state + torch.einsum('pmhk,pmhv->phkv', left, right)
         return state.mT
 
     @torch.no_grad()
     def write(self, views, idx, S, layer=None):
         """Fit + pack value-major states S [P, HV, d_v, d_k] into slots idx; empty the window."""
-        idx32 = idx.to(torch.int32).contiguous()
+        blob = views['blob']
+        idx32 = idx.to(device=blob.device, dtype=torch.int32).contiguous()
         P = idx32.shape[0]
         if P == 0:
             return
-        X = S.float().transpose(-1, -2).contiguous()
-        blob = views['blob']
+        X = S.to(device=blob.device, dtype=torch.float32).transpose(-1, -2).contiguous()
         sl = self._slots(blob, layer)
         _hip.check(_hip.lib().sq_gga_store(C.byref(sl), idx32.data_ptr(), P, X.data_ptr(),
                                            _hip.current_stream(blob.device)))

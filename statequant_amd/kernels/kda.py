@@ -67,7 +67,7 @@ def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_s
         assert t.stride(-1) == 1, 'unit inner stride'
     assert q.stride(-2) == st.DK and k.stride(-2) == st.DK and v.stride(-2) == st.DV and g.stride(-2) == st.DK
     assert beta.stride(-1) == 1 and out.stride(-1) == 1 and out.stride(-2) == st.DV
-    _hip.require_gpu(out, 'KDA step')
+    _hip.same_device('KDA step', T['S'], idx=idx, q=q, k=k, v=v, g=g, beta=beta, out=out, order=order)
     a = _hip.SqKdaArgs(
         st=_hip.make_state(T, strides, nptr_stride), lay=lay, rows=rows, idx=None if idx is None else idx.data_ptr(),
         q=q.data_ptr(), s_q=q.stride(0), q_dtype=_hip.dtype_code(q),

@@ -77,7 +77,8 @@ def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limi
     assert x.stride(-2) == st.DV and out.stride(-1) == 1 and out.stride(-2) == st.DV
     assert B.stride(-2) == st.DK and C.stride(-2) == st.DK
     assert A.is_contiguous() and (D is None or D.is_contiguous()) and (dt_bias is None or dt_bias.is_contiguous())
-    _hip.require_gpu(out, 'Mamba2 step')
+    _hip.same_device('Mamba2 step', T['S'], idx=idx, x=x, dt=dt, B=B, C=C, A=A, D=D, dt_bias=dt_bias, out=out,
+                     order=order)
     clamp = dt_limit is not None and tuple(dt_limit) != (0., float('inf'))
     lo, hi = (float(dt_limit[0]), float(dt_limit[1])) if clamp else (0., 0.)
     a = _hip.SqMamba2Args(

@@ -156,7 +156,7 @@ class SlotLayout:
         launch reading the slots' fill counters.  The counters of every layer of a model move together, so one order
         per decode step serves all layers.  Worth it when sequences joined the batch at different times; a batch that
         folds in lockstep gains nothing."""
-        _hip.require_gpu(idx, 'SlotLayout.fold_first')
+        _hip.same_device('SlotLayout.fold_first', views['NPTR'], idx=idx, out=out)
         return _hip.fold_first(idx, views['NPTR'], self.m, out)
 
     # -- decode -----------------------------------------------------------------------------------------------
@@ -182,7 +182,9 @@ class SlotLayout:
         assert q.stride(-2) == DK and k.stride(-2) == DK and v.stride(-2) == DV
         assert out.is_contiguous() and out.shape[0] >= B
         assert idx.dtype == torch.int32 and idx.is_contiguous()
-        _hip.require_gpu(out, 'SlotLayout.step')
+        ga, gb, A_log, dt_bias = gate if gate is not None else (None,) * 4
+        _hip.same_device('SlotLayout.step', views['S'], idx=idx, q=q, k=k, v=v, out=out, g=g, beta=beta, a=ga, b=gb,
+                         A_log=A_log, dt_bias=dt_bias, order=order)
         lay = self._layout_struct()
         T, strides, sN = slot_state(views)
         a = _hip.SqGdnArgs(
@@ -192,7 +194,6 @@ class SlotLayout:
             v=v.data_ptr(), s_v=v.stride(0), v_dtype=_hip.dtype_code(v), qk_per_key_head=1,
             out=out.data_ptr(), out_dtype=_hip.dtype_code(out), scale=float(scale), order=_order_ptr(order, B))
         if gate is not None:
-            ga, gb, A_log, dt_bias = gate
             assert ga.stride(-1) == 1 and gb.stride(-1) == 1 and A_log.is_contiguous() and dt_bias.is_contiguous()
             a.gate = 1
             a.a, a.s_a, a.a_dtype = ga.data_ptr(), ga.stride(0), _hip.dtype_code(ga)
@@ -207,7 +208,7 @@ class SlotLayout:
         _hip.check(_hip.lib().sq_gdn_step(ctypes.byref(a), _hip.current_stream(out.device)))
         return out
 
-    # -- prefill side: HIP kernels for the formats the step supports, else torch as in the reference -------------
+    # -- prefill side: HIP kernels for blobs on the GPU, the reference's torch formulation for CPU blobs ----------
     def _buffer(self, views, idx):
         """Dequantized buffer of slots idx: keys [P, HK, m, DK], values [P, HV, m, DV], fill counts [P]."""
         V = views
@@ -226,18 +227,22 @@ class SlotLayout:
         return unpack_vk(codes, sc, self.fmt, self.DK).view(P, self.HV, self.DV, self.DK)
 
     def _hip_format(self, views):
-        """States on the GPU go through the HIP pack / read kernels (a layout the library has no instance for falls
-        back to the reference's torch formulation below; CPU tensors always take it)."""
+        """States on the GPU go through the HIP pack / read kernels and nothing else (a layout the library has no
+        instance for raises, as in ``step``); the torch formulation below is for CPU tensors only."""
         return views['S'].is_cuda
 
     def _read_hip(self, views, idx, kda):
+        """``sq_read`` for a blob on the GPU (``idx`` may live anywhere, as in the reference's indexing; rows with
+        ``idx <= 0`` are padding and come back as zeros), None for a CPU blob."""
         if not self._hip_format(views) or idx.shape[0] == 0:
             return None
+        dev = views['S'].device
         P = idx.shape[0]
-        out = torch.empty(P, self.HV, self.DV, self.DK, device=idx.device, dtype=torch.float32)
+        out = torch.empty(P, self.HV, self.DV, self.DK, device=dev, dtype=torch.float32)
         T, strides, sN = slot_state(views)
-        ok = _hip.read_state(_hip.make_layout(self), T, strides, sN, idx.to(torch.int32).contiguous(), out, kda)
-        return out if ok else None
+        _hip.read_state(_hip.make_layout(self), T, strides, sN, idx.to(device=dev, dtype=torch.int32).contiguous(),
+                        out, kda)
+        return out
 
     @torch.no_grad()
     def read(self, views, idx):
@@ -263,18 +268,22 @@ class SlotLayout:
     @torch.no_grad()
     def write(self, views, idx, S):
         """Store states S [P, HV, d_v, d_k] (value-major) packed into slots ``idx`` and empty their buffers
-        (n = 0, running decay 0) (slots.py:236-252)."""
+        (n = 0, running decay 0) (slots.py:236-252).  On the GPU rows with ``idx <= 0`` are padding and store nothing
+        (slot 0 is the engine's null slot); the CPU formulation indexes like the reference."""
         P = idx.shape[0]
         V = views
-        if self._hip_format(views) and P:
-            src = S.reshape(P, self.HV, self.DV, self.DK).float().contiguous()
+        if self._hip_format(views):
+            if P == 0:
+                return
+            dev = V['S'].device
+            src = S.reshape(P, self.HV, self.DV, self.DK).to(device=dev, dtype=torch.float32).contiguous()
             gc = V['GCUR']
             sc = V.get('SC')
-            if _hip.pack_into(_hip.make_layout(self), src, V['S'], V['S'].stride(0), sc,
-                              sc.stride(0) if sc is not None else 0,
-                              idx=idx.to(torch.int32).contiguous(), GCUR=gc, sGC=gc.stride(0),
-                              gcur_per_head=gc[0].numel() // self.HV, NPTR=V['NPTR'], sN=V['NPTR'].stride(0)):
-                return
+            _hip.pack_into(_hip.make_layout(self), src, V['S'], V['S'].stride(0), sc,
+                           sc.stride(0) if sc is not None else 0,
+                           idx=idx.to(device=dev, dtype=torch.int32).contiguous(), GCUR=gc, sGC=gc.stride(0),
+                           gcur_per_head=gc[0].numel() // self.HV, NPTR=V['NPTR'], sN=V['NPTR'].stride(0))
+            return
         idx = idx.long()
         if self.fmt is None and self.state_dtype == torch.float32:
             V['S'][idx] = S.reshape(P, *V['S'].shape[1:]).float()

@@ -279,17 +279,22 @@ def golden_gga():
     save('gga.pt', out)
 
 
+CASES = {
+    'pack.pt': golden_pack,
+    # config 1 whole (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start): 64 steps, eight folds
+    'gdn_c1.pt': lambda: run_gdn('gdn_c1.pt', (8, 'k', 64), 4, 4, 2, 64, 64, 8, 16, 64, seed=1, S0_scale=0.0),
+    'gdn_int4.pt': lambda: run_gdn('gdn_int4.pt', (4, 'k', 32), 2, 4, 2, 64, 64, 4, 8, 14, seed=2, v_head_scale=True),
+    'gdn_int8_m1.pt': lambda: run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 64, 1, 8, 4, seed=3, per_key=False),
+    'gdn_int4v.pt': lambda: run_gdn('gdn_int4v.pt', (4, 'v', 32), 2, 4, 2, 64, 64, 4, 8, 10, seed=8),   # value-axis groups
+    'gdn_bf16.pt': lambda: run_gdn('gdn_bf16.pt', 'bf16', 2, 4, 2, 64, 64, 4, 8, 10, seed=9),           # unquantized state
+    'kda_int4.pt': lambda: run_kda('kda_int4.pt', (4, 'k', 32), 2, 3, 64, 64, 4, 8, 10, seed=4),
+    'kda_int8_bf16buf.pt': lambda: run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 64, 2, 16, 6, seed=5),
+    'm2_int8.pt': lambda: run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 64, 4, 8, 10, seed=6),
+    'm2_int4_bf16buf.pt': lambda: run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 128, 64, 2, 16, 6, seed=7),
+    'slots.pt': golden_slots,
+    'gga.pt': golden_gga,
+}
+
 if __name__ == '__main__':
-    golden_pack()
-    # config-1 shape (B4 / HV4 / HK2 / d64, int8 per-row scale, bf16 buffer, zero start) in a 17-step excerpt (two folds)
-    run_gdn('gdn_c1.pt', (8, 'k', 64), 4, 4, 2, 64, 64, 8, 16, 17, seed=1, S0_scale=0.0)
-    run_gdn('gdn_int4.pt', (4, 'k', 32), 2, 4, 2, 64, 64, 4, 8, 14, seed=2, v_head_scale=True)
-    run_gdn('gdn_int8_m1.pt', (8, 'k', 32), 1, 2, 1, 64, 64, 1, 8, 4, seed=3, per_key=False)
-    run_gdn('gdn_int4v.pt', (4, 'v', 32), 2, 4, 2, 64, 64, 4, 8, 10, seed=8)      # value-axis scale groups
-    run_gdn('gdn_bf16.pt', 'bf16', 2, 4, 2, 64, 64, 4, 8, 10, seed=9)             # the unquantized bf16 state
-    run_kda('kda_int4.pt', (4, 'k', 32), 2, 3, 64, 64, 4, 8, 10, seed=4)
-    run_kda('kda_int8_bf16buf.pt', (8, 'k', 64), 1, 2, 64, 64, 2, 16, 6, seed=5)
-    run_m2('m2_int8.pt', (8, 'k', 64), 2, 4, 2, 64, 64, 4, 8, 10, seed=6)
-    run_m2('m2_int4_bf16buf.pt', (4, 'k', 32), 1, 4, 1, 128, 64, 2, 16, 6, seed=7)
-    golden_slots()
-    golden_gga()
+    for case in sys.argv[1:] or CASES:          # python tests/golden/make_golden.py [file.pt ...]: those, else all
+        CASES[case]()

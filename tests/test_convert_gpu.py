@@ -132,3 +132,62 @@ def test_mamba2_read_matches_oracle(fmt):
     got = lay.read(views, slots.to(DEV)).cpu()
     want = OS.read(OS.views(table, dev.cpu()), slots, fmt, H, G, DK, DV, m)
     assert torch.allclose(got, want, rtol=1e-5, atol=1e-6 * want.abs().max().item())
+
+
+def test_padding_rows_in_read_and_write_and_a_host_index():
+    """`read` / `write` on a GPU blob: the slot indices may live on the host (the reference indexes with whatever
+    tensor it is given); rows with ``idx <= 0`` are padding -- `write` stores nothing for them, `read` returns zeros
+    (not uninitialised memory)."""
+    HV, HK, D, m = 4, 2, 128, 8
+    lay = SlotLayout(quantizer((8, 'k', 64)), HV, HK, D, D, m=m, buffer_bits=8)
+    gen = torch.Generator().manual_seed(7)
+    blob = torch.randint(0, 256, (6, lay.nbytes), dtype=torch.uint8, generator=gen).to(DEV)
+    before = blob.clone()
+    views = lay.views(blob)
+    idx = torch.tensor([3, 0, 5, -1])                                      # on the host
+    S = torch.randn(4, HV, D, D, generator=gen)
+    lay.write(views, idx, S)                                               # S on the host as well
+    untouched = torch.tensor([0, 1, 2, 4])
+    assert torch.equal(blob[untouched.to(DEV)], before[untouched.to(DEV)])
+    got = lay.read(views, idx)
+    assert got.is_cuda
+    twin = lay.views(before.clone())
+    lay.write(twin, idx[[0, 2]].to(DEV), S[[0, 2]].to(DEV))
+    want = lay.read(twin, idx[[0, 2]].to(DEV))
+    assert torch.equal(got[[0, 2]], want)
+    assert torch.equal(got[[1, 3]], torch.zeros(2, HV, D, D, device=DEV))
+    for _ in range(3):                                                     # fresh allocations: still zeros
+        assert torch.equal(lay.read(views, idx)[[1, 3]], torch.zeros(2, HV, D, D, device=DEV))
+
+
+def test_step_refuses_a_host_operand():
+    """`step` takes raw pointers, so an operand that is not on the state's device is refused in Python."""
+    HV, HK, D = 4, 2, 128
+    lay = SlotLayout(quantizer((8, 'k', 128)), HV, HK, D, D, m=4)
+    views = lay.views(lay.alloc(3, DEV))
+    q, k, v, g, beta = (x.to(DEV) for x in gdn_token(torch.Generator().manual_seed(1), 2, HV, HK, D, D))
+    out = torch.zeros(2, HV, D, device=DEV)
+    with pytest.raises(RuntimeError, match='`idx` is on cpu'):
+        lay.step(views, torch.tensor([1, 2], dtype=torch.int32), q, k, v, out, 1.0, g=g, beta=beta)
+    with pytest.raises(RuntimeError, match='`beta` is on cpu'):
+        lay.step(views, torch.tensor([1, 2], dtype=torch.int32, device=DEV), q, k, v, out, 1.0, g=g, beta=beta.cpu())
+    assert torch.equal(views['NPTR'], torch.zeros_like(views['NPTR']))
+
+
+def test_unsupported_layout_raises_instead_of_falling_back(monkeypatch):
+    """A GPU blob never takes the torch formulation: `read` / `write` / `pack_vk` either run the HIP kernels or
+    raise.  The torch helpers are made to fail here, and every parametrised format above still passes through
+    `_hip.pack_into` / `_hip.read_state`."""
+    import statequant_amd.kernels.slots as SL
+    monkeypatch.setattr(SL, 'pack_vk', lambda *a, **k: (_ for _ in ()).throw(AssertionError('torch path taken')))
+    monkeypatch.setattr(SL.SlotLayout, '_stored', lambda *a, **k: (_ for _ in ()).throw(AssertionError('torch path taken')))
+    for fmt in [(8, 'k', 128), (4, 'k', 32), (4, 'v', 32), (8, 'v', 16), 'bf16', 'fp32']:
+        lay = SlotLayout(quantizer(fmt), 4, 2, 128, 128, m=8)
+        views = lay.views(lay.alloc(3, DEV))
+        idx = torch.tensor([1, 2], device=DEV)
+        lay.write(views, idx, torch.randn(2, 4, 128, 128, device=DEV))
+        assert torch.isfinite(lay.read(views, idx)).all()
+    lay = SlotLayout(quantizer((8, 'k', 128)), 4, 2, 128, 128, m=32)       # the read kernel stops at m = 16
+    views = lay.views(lay.alloc(3, DEV))
+    with pytest.raises(RuntimeError, match='libsqhip'):
+        lay.read(views, torch.tensor([1], device=DEV))

@@ -1,0 +1,158 @@
+"""The Mamba2 and KDA steps at the benchmark configurations' full sizes, the ragged KDA variant with padding rows, and
+the PACE-4 Gated DeltaNet configuration (d 128, int4 groups of 32, values scaled per head).
+
+Full sizes are far beyond what the oracle steps in seconds, so -- as tests/test_scale_gpu.py does for the headline --
+a run is checked through (i) a subset of its rows against the oracle, (ii) a size-independent property: batch rows r
+and r + rows / 2 get the same state and the same inputs, so their slots must end byte-identical and their outputs equal
+whichever tile, compute unit or XCD processed them, and (iii) the counters of every slot.  Mirrors the reference's
+slot-step tests (tests/test_mamba2.py:273-300, tests/test_kda_kernels.py:238-265 there).
+"""
+import pytest
+import torch
+
+import statequant_amd as sq
+from oracle import states as ST
+from statequant_amd.kernels import KDASlotLayout, Mamba2SlotLayout
+from tests._util import unpack_nib
+from tests.test_gdn_gpu import check as check_gdn, run_decode as run_gdn
+from tests.test_kda_gpu import kda_token
+from tests.test_mamba2_gpu import m2_token, params
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def _codes_close(views, idx, rows, ref, bits):
+    codes = views['S'][idx[rows].long()].cpu().reshape(ref.codes.shape)
+    d = (unpack_nib(codes, bits).int() - unpack_nib(ref.codes, bits).int()).abs()
+    assert d.max().item() <= 1 and (d != 0).float().mean().item() < 1e-3, ((d != 0).float().mean().item(), d.max())
+
+
+def _twins_equal(views, idx, half, live=None, written=2):
+    a_idx, b_idx = idx[:half].long(), idx[half:].long()
+    if live is not None:
+        a_idx, b_idx = a_idx[live], b_idx[live]
+    for f in ('S', 'SC', 'GCUR', 'NPTR'):
+        assert torch.equal(views[f][a_idx], views[f][b_idx]), f
+    for f in ('UB', 'KB', 'GB', 'UBS', 'KBS'):                  # the buffer slots written since the fold
+        assert torch.equal(views[f][a_idx][:, :, :written], views[f][b_idx][:, :, :written]), f
+
+
+def test_mamba2_full_size_subset_and_twin_rows():
+    """128 heads / 8 groups, head_dim 64, d_state 128, 128 slots, int8 state with one scale per (head, row)."""
+    H, G, DK, DV, m, slots = 128, 8, 128, 64, 8, 128
+    fmt = (8, 'k', 128)
+    lay = Mamba2SlotLayout(sq.Quantizer(*fmt), H, G, DK, DV, m=m, buffer_bits=8)
+    views = lay.views(lay.alloc(slots + 1, DEV))
+    gen = torch.Generator().manual_seed(11)
+    half = slots // 2
+    idx = (torch.randperm(slots, generator=gen) + 1).to(torch.int32).to(DEV)
+    S_half = torch.randn(half, H, DV, DK, generator=gen) * 0.5
+    lay.write(views, idx[:half].long(), S_half.to(DEV))
+    lay.write(views, idx[half:].long(), S_half.to(DEV))
+    A, D, dtb = params(gen, H)
+    rows = [0, 29, 63]
+    ref = ST.Mamba2Oracle(S_half[rows].reshape(-1, DV, DK), fmt, m=m, hv=H, hk=G, buffer_bits=8)
+    two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
+    worst = 0.0
+    for t in range(m + 2):                                  # through one fold and two tokens beyond
+        x, dt, Bm, C = m2_token(gen, half, H, G, DK, DV)
+        out = torch.full((slots, H, DV), 7.0, device=DEV)
+        lay.step(views, idx, two(x), two(dt), two(Bm), two(C), out, A.to(DEV), D.to(DEV), dtb.to(DEV))
+        got = out.cpu()
+        assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
+        want = ref.step(x[rows], dt[rows], Bm[rows], C[rows], A, D, dtb, True, (0., float('inf'))).view(len(rows), H, DV)
+        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        assert torch.equal(views['NPTR'][idx.long(), :H].cpu(), torch.full((slots, H), (t + 1) % m, dtype=torch.int32))
+    assert worst < 5e-3, worst                 # no re-sync with the oracle here: a flipped buffer entry persists
+    _twins_equal(views, idx, half)
+    _codes_close(views, idx, rows, ref, 8)
+
+
+def test_kda_full_size_subset_and_twin_rows():
+    """32 heads, d_k = d_v = 128, 256 slots, int4 state in groups of 32."""
+    H, D, m, slots = 32, 128, 8, 256
+    fmt = (4, 'k', 32)
+    lay = KDASlotLayout(sq.Quantizer(*fmt), H, D, D, m=m, buffer_bits=8)
+    views = lay.views(lay.alloc(slots + 1, DEV))
+    gen = torch.Generator().manual_seed(12)
+    half = slots // 2
+    idx = (torch.randperm(slots, generator=gen) + 1).to(torch.int32).to(DEV)
+    S_half = torch.randn(half, H, D, D, generator=gen) * 0.5
+    lay.write(views, idx[:half].long(), S_half.to(DEV))
+    lay.write(views, idx[half:].long(), S_half.to(DEV))
+    rows = [0, 57, 127]
+    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8)
+    two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
+    flat = lambda x: x[rows].reshape(len(rows) * H, *x.shape[2:])          # noqa: E731
+    worst = 0.0
+    for t in range(m + 2):
+        q, k, v, g, beta = kda_token(gen, half, H, D, D)
+        out = torch.full((slots, H, D), 7.0, device=DEV)
+        lay.step(views, idx, two(q), two(k), two(v), two(g), two(beta), out)
+        got = out.cpu()
+        assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
+        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta)).view(len(rows), H, D)
+        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        assert torch.equal(views['NPTR'][idx.long(), :H].cpu(), torch.full((slots, H), (t + 1) % m, dtype=torch.int32))
+    assert worst < 5e-3, worst
+    _twins_equal(views, idx, half)
+    _codes_close(views, idx, rows, ref, 4)
+
+
+def test_kda_ragged_variant_with_padding_rows():
+    """20 heads, d_k = d_v = 96 (neither a power of two), 256 batch rows of which about 40 % are padding (slot index
+    0 or -1): padding rows give zeros and touch nothing, live rows behave as in the dense run."""
+    H, D, m, nrows = 20, 96, 8, 256
+    fmt = (4, 'k', 32)
+    lay = KDASlotLayout(sq.Quantizer(*fmt), H, D, D, m=m, buffer_bits=8)
+    blob = lay.alloc(nrows + 1, DEV)
+    views = lay.views(blob)
+    gen = torch.Generator().manual_seed(13)
+    half = nrows // 2
+    slot = torch.randperm(nrows, generator=gen) + 1
+    dead = torch.rand(half, generator=gen) < 0.4                            # the same rows in both halves
+    dead[[0, 57]] = False                                                   # rows checked against the oracle stay live
+    pad = torch.where(torch.rand(half, generator=gen) < 0.5, 0, -1)
+    slot[:half][dead], slot[half:][dead] = pad[dead], pad[dead]
+    idx = slot.to(torch.int32).to(DEV)
+    live = ~dead
+    assert 0.3 < dead.float().mean().item() < 0.5
+    S_half = torch.randn(half, H, D, D, generator=gen) * 0.5
+    lay.write(views, idx[:half][live].long(), S_half[live].to(DEV))
+    lay.write(views, idx[half:][live].long(), S_half[live].to(DEV))
+    untouched = torch.ones(nrows + 1, dtype=torch.bool)
+    untouched[slot[slot > 0]] = False                                       # slot 0 and the slots no row points at
+    before = blob[untouched.to(DEV)].clone()
+    rows = [0, 57]
+    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8)
+    two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
+    flat = lambda x: x[rows].reshape(len(rows) * H, *x.shape[2:])          # noqa: E731
+    worst = 0.0
+    for t in range(m + 2):
+        q, k, v, g, beta = kda_token(gen, half, H, D, D)
+        out = torch.full((nrows, H, D), 7.0, device=DEV)
+        lay.step(views, idx, two(q), two(k), two(v), two(g), two(beta), out)
+        got = out.cpu()
+        assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
+        assert torch.equal(got[:half][dead], torch.zeros(int(dead.sum()), H, D)), 'padding rows must give zeros'
+        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta)).view(len(rows), H, D)
+        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        n_live = views['NPTR'][idx[:half][live].long(), :H].cpu()
+        assert torch.equal(n_live, torch.full((int(live.sum()), H), (t + 1) % m, dtype=torch.int32))
+    assert worst < 5e-3, worst
+    assert torch.equal(blob[untouched.to(DEV)], before), 'a padding row wrote to a slot'
+    _twins_equal(views, idx, half, live=live.to(DEV))
+    _codes_close(views, idx, rows, ref, 4)
+
+
+@pytest.mark.parametrize('m,bb', [(8, 8), (8, 16)])
+def test_gdn_pace4_d128_values_scaled_per_head(m, bb):
+    """The PACE-4 configuration's numerics: d 128, int4 groups of 32, re-encode every 8 tokens, v scaled by a
+    per-head log-uniform factor in [0.1, 10] (outlier channels), against the oracle step by step."""
+    HV, T = 4, 5 * m
+    vs = torch.exp(torch.empty(HV).uniform_(-2.302585, 2.302585, generator=torch.Generator().manual_seed(21)))
+    assert vs.max() / vs.min() > 3
+
+    tal = run_gdn((4, 'k', 32), m, bb, B=3, HV=HV, HK=2, D=128, T=T, seed=22, v_scale=vs)
+    check_gdn(tal, f'gdn pace4 d128 per-head v scale, buf{bb}', T, m)

@@ -23,7 +23,7 @@ VALUE_AXIS = {'int8-v-g32': (8, 'v', 32), 'int4-v-g32': (4, 'v', 32)}
 
 
 def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.float32, S0_scale=0.5, DV=None,
-               shape_state=None, shape_token=None):
+               shape_state=None, shape_token=None, v_scale=None):
     DV = DV or D
     gen = torch.Generator().manual_seed(seed)
     S0 = torch.randn(B * HV, DV, D, generator=gen) * S0_scale                    # value-major
@@ -36,7 +36,7 @@ def run_decode(fmt, m, bb, B=2, HV=4, HK=2, D=128, T=40, seed=1, dtype=torch.flo
     tal = Tally()
     scale = D ** -0.5
     for t in range(T):
-        q, k, v, g, beta = gdn_token(gen, B, HV, HK, D, DV, dtype)
+        q, k, v, g, beta = gdn_token(gen, B, HV, HK, D, DV, dtype, v_scale=v_scale)
         if shape_token is not None:
             shape_token(q, k, v)
         slot = ker.n

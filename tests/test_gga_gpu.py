@@ -335,3 +335,29 @@ def test_random_configurations(cfg):
             assert off.float().mean().item() < (3e-2 if cfg['bf16'] else 2e-3), t
             assert torch.equal(V.cpu() * nonp, ora.V[li] * nonp), t
     assert not Vp['blob'][0].any()
+
+
+def test_write_read_on_a_page_that_was_never_zeroed():
+    """`write` then `read` on a blob pre-filled with 0xFF and with random bytes: the store kernel resets only the
+    window's counters, so the dead window entries keep decoding to NaN -- and must not reach the logical state."""
+    HV, HK, D, layer = 8, 4, 128, 0
+    pk = GGAPacked(plan(HV, D), HV, HK, D, D, pw=True).prepare(DEV)
+    g = torch.Generator().manual_seed(3)
+    S = (torch.randn(2, HV, D, D, generator=g) * 0.3).to(DEV)
+    idx = torch.tensor([2, 1], dtype=torch.int32, device=DEV)
+    clean = pk.views(pk.alloc(4, DEV))
+    pk.write(clean, idx, S, layer=layer)
+    want = pk.read(clean, idx, layer=layer)
+    for fill in (0xFF, None):
+        blob = pk.alloc(4, DEV)
+        if fill is None:
+            blob.copy_(torch.randint(0, 256, blob.shape, dtype=torch.uint8, generator=g).to(DEV))
+        else:
+            blob.fill_(fill)
+        V = pk.views(blob)
+        pk.write(V, idx, S, layer=layer)
+        got = pk.read(V, idx, layer=layer)
+        assert torch.isfinite(got).all(), fill
+        assert torch.equal(got, want), fill
+        left, right, count = pk.window(V, idx)
+        assert count.tolist() == [0, 0] and not left.any() and not right.any()

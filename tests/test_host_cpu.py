@@ -278,3 +278,66 @@ def test_unsupported_dims_refused_and_olmo_bytes():
     assert b['KB'] == 30 * 8 * 96 and b['UB'] == 30 * 8 * 192
     from statequant_amd.kernels import Mamba2SlotLayout
     assert Mamba2SlotLayout('bf16', 96, 8, 128, 80, m=8, buffer_bits=8).breakdown()['S'] == 96 * 80 * 128 * 2
+
+
+def test_host_tensors_are_refused_before_any_launch():
+    """Every wrapper that hands raw pointers to the library checks devices first: with CPU tensors the call ends in a
+    RuntimeError raised in Python, not in a kernel dereferencing a host pointer."""
+    from statequant_amd.kernels.gga import GGAPacked, GGAPlan
+    B, HV, HK, D, m = 2, 4, 2, 128, 4
+    idx = torch.tensor([1, 2], dtype=torch.int32)
+    q, k, v = torch.zeros(B, HK, D), torch.zeros(B, HK, D), torch.zeros(B, HV, D)
+    out = torch.zeros(B, HV, D)
+    lay = SlotLayout(sq.Quantizer(8, 'k', 128), HV, HK, D, D, m=m)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        lay.step(lay.views(lay.alloc(3, 'cpu')), idx, q, k, v, out, 1.0, g=torch.zeros(B, HV), beta=torch.zeros(B, HV))
+    with pytest.raises(RuntimeError, match='GPU only'):
+        lay.fold_first(lay.views(lay.alloc(3, 'cpu')), idx)
+    kl = KDASlotLayout(sq.Quantizer(4, 'k', 32), HV, D, D, m=m)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        kl.step(kl.views(kl.alloc(3, 'cpu')), idx, torch.zeros(B, HV, D), torch.zeros(B, HV, D), v,
+                torch.zeros(B, HV, D), torch.zeros(B, HV), out)
+    ml = Mamba2SlotLayout(sq.Quantizer(8, 'k', 128), HV, HK, D, 64, m=m)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        ml.step(ml.views(ml.alloc(3, 'cpu')), idx, torch.zeros(B, HV, 64), torch.zeros(B, HV), q, k,
+                torch.zeros(B, HV, 64), torch.zeros(HV))
+    pk = GGAPacked(GGAPlan({0: (torch.tensor([4] * HV), torch.ones(HV, D))}), HV, HK, D, D, pw=True)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        pk.write(pk.views(pk.alloc(3, 'cpu')), idx, torch.zeros(B, HV, D, D), layer=0)
+    # the helper itself: a state on one device and an operand on another
+    class On:                                              # stands in for tensors on two GPUs
+        def __init__(self, d):
+            self.is_cuda, self.device = True, d
+    with pytest.raises(RuntimeError, match='`idx` is on cpu'):
+        _hip.same_device('step', On('cuda:0'), q=On('cuda:0'), idx=torch.zeros(1), beta=None)
+    _hip.same_device('step', On('cuda:0'), q=On('cuda:0'), beta=None)
+
+
+def test_gga_window_selects_dead_entries_away():
+    """`GGAPacked.window` on a slot whose page was never zero-filled: dead ring entries decode to NaN (FP8 0xFF) with
+    NaN scales and must come back as zeros, as the reference's `where(live, ..., 0)` gives them
+    (vllm_gga.py, window()); live entries are untouched by the garbage around them."""
+    from statequant_amd.kernels.gga import GGAPacked, GGAPlan
+    HV, HK, D, m = 4, 2, 64, 4
+    pk = GGAPacked(GGAPlan({0: (torch.tensor([4, 8, 16, 2]), torch.ones(HV, D))}), HV, HK, D, D, pw=True, m=m)
+    blob = torch.full((3, pk.alloc(1, 'cpu').shape[1]), 0xFF, dtype=torch.uint8)
+    views = pk.views(blob)
+    idx = torch.tensor([1, 2])
+    blob[:, :8] = 0                                        # counters: empty windows
+    left, right, count = pk.window(views, idx)
+    assert count.tolist() == [0, 0]
+    assert torch.equal(left, torch.zeros_like(left)) and torch.equal(right, torch.zeros_like(right))
+    # two live entries in slot 2 (ring positions 3 and 0), the other two entries garbage
+    blob[2, :8] = torch.tensor([2, 3], dtype=torch.int32).view(torch.uint8)
+    win = blob[2, pk.QOFF:pk.QOFF + HV * pk.QSZ].view(HV, pk.QSZ)
+    one = torch.tensor([1.0], dtype=torch.float32).to(torch.float8_e4m3fn).view(torch.uint8).item()
+    for pos in (3, 0):
+        win[:, pos * D:(pos + 1) * D] = one                                           # left codes: all 1.0
+        win[:, m * D + pos * D:m * D + (pos + 1) * D] = one                           # right codes
+    sc = win[:, m * 2 * D:].view(torch.float32).view(HV, 2, m)
+    sc[:, :, 3], sc[:, :, 0] = 0.5, 2.0
+    left, right, count = pk.window(views, idx)
+    assert count.tolist() == [0, 2]
+    assert torch.isfinite(left).all() and torch.isfinite(right).all()
+    assert torch.equal(left[1, 0], torch.full((HV, D), 0.5)) and torch.equal(left[1, 1], torch.full((HV, D), 2.0))
+    assert torch.equal(left[1, 2:], torch.zeros(2, HV, D)) and torch.equal(left[0], torch.zeros(m, HV, D))
