@@ -282,6 +282,7 @@ def bench_gga(a, dev):
     a.steps = max(-(-a.steps // period_len), 1) * period_len          # whole graphs of period_len steps
     a.warmup = -(-a.warmup // period_len) * period_len
     use_graph = not a.no_graph
+    torch.cuda.synchronize()                                # states and inputs were made on the default stream
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         period()
@@ -481,6 +482,7 @@ def main():
     a.steps = max(-(-a.steps // m), 1) * m                  # whole fold periods, so that any K times steps / m folds
     a.warmup = -(-a.warmup // m) * m
     use_graph = not a.no_graph
+    torch.cuda.synchronize()                                # states and inputs were made on the default stream
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         if use_graph:

@@ -28,7 +28,7 @@ import tempfile
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 LAYERS, M = 24, 8                       # bench.py's layer blobs and fold period
-STEP_KERNELS = ('step_kernel', 'quad_kernel')
+STEP_KERNELS = ('step_kernel', 'quad_kernel', 'pack_kernel', 'pack_v_kernel', 'pack_f_kernel', 'read_kernel')
 SHADER_SETS = {
     'issue': ['SQ_WAVES', 'SQ_INSTS_VALU', 'SQ_INSTS_SALU', 'SQ_INSTS_LDS', 'SQ_INSTS_VMEM_RD', 'SQ_INSTS_VMEM_WR',
               'SQ_INSTS_SMEM', 'SQ_INSTS_MFMA'],
@@ -82,18 +82,21 @@ def main():
     ap.add_argument('--workload', default='gdn-int8-g128')
     ap.add_argument('--out', default=os.path.join(ROOT, 'profiles'))
     ap.add_argument('--sets', default='trace,hbm,shader')
-    ap.add_argument('--bench-args', default='', help='extra bench.py arguments, e.g. "--mixed-fill"')
+    ap.add_argument('--bench-args', default='', help='extra bench.py arguments, given as --bench-args=--mixed-fill')
     a = ap.parse_args()
     sets = a.sets.split(',')
     os.makedirs(a.out, exist_ok=True)
     work = tempfile.mkdtemp(prefix='profile_step_', dir='/tmp')
     bargs = ['--workload', a.workload, '--no-cpu-baseline', '--steps', str(2 * M), '--warmup', str(2 * M),
              *a.bench_args.split()]
-    is_step = lambda n: any(s in n for s in STEP_KERNELS)          # noqa: E731
+    names = STEP_KERNELS[:2]
+    if '--op' in a.bench_args:                               # the prefill-side kernels instead
+        names = ('read_kernel',) if 'read' in a.bench_args else STEP_KERNELS[2:5]
+    is_step = lambda n: any(s in n for s in names)         # noqa: E731
     lines = [f'rocprofv3 profile of the decode-step kernel, bench.py workload {a.workload}'
              + (f' ({a.bench_args})' if a.bench_args else ''),
              f'made by: python profile_step.py --workload {a.workload} --sets {a.sets}'
-             + (f' --bench-args "{a.bench_args}"' if a.bench_args else ''),
+             + (f' --bench-args={a.bench_args}' if a.bench_args else ''),
              'every pass below is a run of its own, from /tmp with TMPDIR=/tmp; <dir> is a scratch directory', '']
     kernel = ''
 
@@ -147,7 +150,8 @@ def main():
                   f"  fold step   read {per['FETCH_SIZE']['fold']:,.0f}  written {per['WRITE_SIZE']['fold']:,.0f}",
                   f'  average over a fold period of {M} steps: {traffic:,.0f} bytes per launch', '']
         path = os.path.join(a.out, 'hbm_traffic.json')
-        table = json.load(open(path)) if os.path.exists(path) else {}
+        kept = path if os.path.exists(path) else os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+        table = json.load(open(kept)) if os.path.exists(kept) else {}          # other workloads' rows stay
         table[a.workload + (' ' + a.bench_args if a.bench_args else '')] = {
             'traffic': round(traffic), 'read_plain': round(per['FETCH_SIZE']['plain']),
             'read_fold': round(per['FETCH_SIZE']['fold']), 'written_plain': round(per['WRITE_SIZE']['plain']),
