@@ -2,9 +2,10 @@
 
     python profile_step.py --workload gdn-int8-g128 [--out profiles] [--sets trace,hbm,shader]
 
-Runs ``bench.py --workload W --no-cpu-baseline --steps 16 --warmup 16`` (two fold periods of m = 8 after two of
-warm-up; 24 launches per step) under rocprofv3, once per pass -- the kernel trace, then one run per counter set,
-because the profiler does not split counters over passes -- from /tmp with TMPDIR=/tmp, and the same passes over
+Runs ``bench.py --workload W --no-cpu-baseline`` under rocprofv3, once per pass, from /tmp with TMPDIR=/tmp: the
+kernel trace with bench.py's own step counts (the command of the bench line, so the two averages can be compared),
+then one run per counter set (the profiler does not split counters over passes) with ``--steps 16 --warmup 16`` (two
+fold periods of m = 8 after two of warm-up; counter collection serialises the launches), and the same passes over
 ``bench.py --calibrate-copy`` for the two HBM counters (a device copy of known size: what FETCH_SIZE / WRITE_SIZE read
 for it gives the factor their readings are scaled by).  Writes
 
@@ -82,13 +83,18 @@ def main():
     ap.add_argument('--workload', default='gdn-int8-g128')
     ap.add_argument('--out', default=os.path.join(ROOT, 'profiles'))
     ap.add_argument('--sets', default='trace,hbm,shader')
+    ap.add_argument('--trace-steps', default='', metavar='K,W',
+                    help="steps and warm-up of the trace pass instead of bench.py's own (e.g. 16,16)")
     ap.add_argument('--bench-args', default='', help='extra bench.py arguments, given as --bench-args=--mixed-fill')
     a = ap.parse_args()
     sets = a.sets.split(',')
     os.makedirs(a.out, exist_ok=True)
     work = tempfile.mkdtemp(prefix='profile_step_', dir='/tmp')
-    bargs = ['--workload', a.workload, '--no-cpu-baseline', '--steps', str(2 * M), '--warmup', str(2 * M),
-             *a.bench_args.split()]
+    targs = ['--workload', a.workload, '--no-cpu-baseline', *a.bench_args.split()]     # the trace: bench.py's own K, W
+    bargs = [*targs, '--steps', str(2 * M), '--warmup', str(2 * M)]                   # counters: two fold periods
+    if a.trace_steps:
+        k, w = a.trace_steps.split(',')
+        targs = [*targs, '--steps', k, '--warmup', w]
     names = STEP_KERNELS[:2]
     if '--op' in a.bench_args:                               # the prefill-side kernels instead
         names = ('read_kernel',) if 'read' in a.bench_args else STEP_KERNELS[2:5]
@@ -96,12 +102,13 @@ def main():
     lines = [f'rocprofv3 profile of the decode-step kernel, bench.py workload {a.workload}'
              + (f' ({a.bench_args})' if a.bench_args else ''),
              f'made by: python profile_step.py --workload {a.workload} --sets {a.sets}'
+             + (f' --trace-steps {a.trace_steps}' if a.trace_steps else '')
              + (f' --bench-args={a.bench_args}' if a.bench_args else ''),
              'every pass below is a run of its own, from /tmp with TMPDIR=/tmp; <dir> is a scratch directory', '']
     kernel = ''
 
     if 'trace' in sets:
-        cmd, d = rocprof(['--kernel-trace', '--stats'], bargs, work)
+        cmd, d = rocprof(['--kernel-trace', '--stats'], targs, work, timeout=600)
         rows = [r for r in read_csv(d, 'kernel_trace.csv') if is_step(r['Kernel_Name'])]
         rows.sort(key=lambda r: int(r['Start_Timestamp']))
         dur = [(int(r['End_Timestamp']) - int(r['Start_Timestamp'])) / 1e3 for r in rows]
