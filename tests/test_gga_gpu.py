@@ -8,7 +8,8 @@ of the fit's reductions differs from the oracle, which can move a row / column f
 threshold: outputs 1e-5 relative; < 2e-3 of the stored values off by more than 1e-3 of the largest; < 1e-3 of the
 window's left factors off; right factors, counters and fp16 pivots exact.  (The reference's bound on values that
 differ at all after a fit, 1e-3, is quoted on 512 heads; on the 24 small heads here one moved row factor is more than
-that, so the fit test counts heads instead.)
+that, so the fit test counts heads instead: at most one of 24, and the factor test shows each difference to be one
+fp16 step of a factor whose unrounded value sits on the rounding threshold.)
 """
 import numpy as np
 import pytest
@@ -58,9 +59,13 @@ def test_pack_unpack_equals_fit(D, layer):
     # A row factor on an fp16 rounding threshold re-codes its whole row (d of 24 d^2 values here; the same sums taken
     # in float64 on the CPU move the same few factors), so: few heads differ at all, and those by a rounding step.
     heads_off = sum(not torch.equal(got[bi, h], want[bi, h]) for bi in range(B) for h in range(HV))
-    assert heads_off <= 3, heads_off
-    assert (got != want).float().mean().item() < 5e-3
-    assert ((got - want).norm() / want.norm()).item() < 1e-3
+    print(f'\n[gga store d={D} layer {layer}] heads off {heads_off}, values off {(got != want).float().mean().item():.2e}, '
+          f'rel norm {((got - want).norm() / want.norm()).item():.2e}')
+    # measured on these seeds: 0 or 1 of the 24 heads off (one row or column factor on an fp16 rounding threshold, see
+    # test_fit_factors_differ_from_the_oracle_only_on_rounding_thresholds), at most 3.2e-3 of the values, 6e-5 in norm
+    assert heads_off <= 1, heads_off
+    assert (got != want).float().mean().item() < 4e-3
+    assert ((got - want).norm() / want.norm()).item() < 1e-4
     piv = bits == 16
     assert torch.equal(got[:, piv], S[:, piv].half().float())
     assert torch.equal(pk.read(Vp, idx.to(DEV), layer=layer).cpu(), got.transpose(-1, -2))     # empty window
@@ -83,7 +88,7 @@ def test_pack_unpack_equals_fit(D, layer):
             if torch.equal(got[bi, h], want[bi, h]):
                 assert np.array_equal(have, raw), (slot, h, b)
                 same += 1
-    assert same >= 0.8 * B * HV, same
+    assert same >= B * HV - 1, same
     assert not blob[[0, 1, 3]].any()                                             # other slots untouched
 
 
@@ -361,3 +366,85 @@ def test_write_read_on_a_page_that_was_never_zeroed():
         assert torch.equal(got, want), fill
         left, right, count = pk.window(V, idx)
         assert count.tolist() == [0, 0] and not left.any() and not right.any()
+
+
+def _f16_steps_apart(a, b):
+    """How many fp16 values lie between two fp16 arrays' entries (0: equal, 1: neighbours)."""
+    ia, ib = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+    return np.abs(ia - ib)                                   # factors are positive: the bit pattern orders like the value
+
+
+@pytest.mark.parametrize('D', [128, 64])
+def test_fit_factors_differ_from_the_oracle_only_on_rounding_thresholds(D):
+    """Where the stored fit differs from the oracle's, why: a row factor r = fp16(sqrt(mean|x| / w)) or a column factor
+    c = fp16(num / den) comes from an fp32 sum whose order is the kernel's, not torch's.  Every stored factor is read
+    back from the slot's bytes and compared: a factor that differs is the NEIGHBOURING fp16 number, and the float64
+    value of what is being rounded lies within 2^-17 (rows: a mean of d_v magnitudes under a square root) or 2^-15
+    (columns: a ratio of two sums over d_k) of the midpoint between the two -- 0.03 / 0.13 of half an fp16 step, i.e. both
+    roundings are answers an fp32 sum in some order gives.  Heads all of whose factors agree are byte-identical."""
+    B, HV, HK, layers = 8, 8, 4, 2
+    q = plan(HV, D)
+    pk = GGAPacked(q, HV, HK, D, D, pw=True)
+    g = torch.Generator().manual_seed(19)
+    idx = (torch.randperm(B, generator=g) + 1).to(torch.int32)
+    rows_seen = rows_off = cols_seen = cols_off = heads = heads_exact = 0
+    for layer in range(layers):
+        Vp = pk.views(pk.alloc(B + 1, DEV))
+        S = torch.randn(B, HV, D, D, generator=g) * torch.logspace(-3, 0, D)      # canonical [B, HV, d_k, d_v]
+        pk.write(Vp, idx.to(DEV), S.transpose(-1, -2).to(DEV), layer=layer)
+        bits, w = q.plan[layer]
+        rf, c, z, _ = G.fit_parts(S, bits, w)
+        blob = Vp['blob'].cpu().numpy()
+        offs = pk.tables[layer][0]
+        x64, w64 = S.double(), w.double()
+        for bi, slot in enumerate(idx.tolist()):
+            for h in range(HV):
+                b = int(bits[h])
+                if b == 16:
+                    continue
+                heads += 1
+                raw = blob[slot, offs[h]:offs[h] + G.head_bytes(b, D, D)]
+                ncode = D * D * b // 8
+                per_row = D // 32 if b == 2 else 1
+                r_got = raw[ncode:ncode + 2 * D * per_row].view(np.float16).reshape(D, per_row)
+                c_got = raw[ncode + 2 * D * per_row:].view(np.float16)
+                r_want = (rf[bi, h, :, ::32] if b == 2 else rf[bi, h, :, :1]).numpy().astype(np.float16)
+                c_want = c[bi, h, 0].numpy().astype(np.float16)
+                # rows
+                dr = _f16_steps_apart(r_got, r_want)
+                rows_seen += dr.size
+                rows_off += int((dr != 0).sum())
+                assert dr.max() <= 1, (layer, slot, h, int(dr.max()))
+                mags = x64[bi, h].abs().reshape(D, per_row, -1).mean(-1).clamp_min(1e-20)
+                exact = (mags / w64[h][:, None]).sqrt().numpy()
+                for k_, j in zip(*np.nonzero(dr)):
+                    mid = (float(r_got[k_, j]) + float(r_want[k_, j])) / 2
+                    assert abs(exact[k_, j] - mid) <= 2.0 ** -17 * mid, (layer, slot, h, k_, exact[k_, j], mid)
+                if dr.any():
+                    continue                               # another row factor re-codes its row: columns follow suit
+                # columns: the refit c = num / den from the oracle's own codes (same rows, so same codes)
+                dc = _f16_steps_apart(c_got, c_want)
+                cols_seen += dc.size
+                cols_off += int((dc != 0).sum())
+                assert dc.max() <= 1, (layer, slot, h, int(dc.max()))
+                if dc.any():
+                    qmax = 3.0 if b == 2 else 2.0 ** (min(b, 8) - 1) - 1
+                    y0 = S[bi, h] / rf[bi, h]
+                    c0 = G.half_clamp((y0.abs() / qmax).amax(0, keepdim=True))
+                    y = y0 / c0
+                    z0 = torch.round(y).clamp(-qmax, qmax)
+                    if b == 2:
+                        z0 = torch.where(y >= 0, 1., -1.) * torch.where(y.abs() >= 2, 3., 1.)
+                    vv = rf[bi, h].double() * z0.double()
+                    ww = w64[h].square()[:, None]
+                    ratio = ((ww * vv * x64[bi, h]).sum(0) / (ww * vv.square()).sum(0)).numpy()
+                    for j in np.nonzero(dc)[0]:
+                        mid = (float(c_got[j]) + float(c_want[j])) / 2
+                        assert abs(ratio[j] - mid) <= 2.0 ** -15 * abs(mid), (layer, slot, h, j, ratio[j], mid)
+                else:
+                    want_raw = G.pack_head(r_want[:, 0] if b != 2 else r_want, c[bi, h, 0], z[bi, h], b)
+                    assert np.array_equal(raw, want_raw), (layer, slot, h)
+                    heads_exact += 1
+    print(f'\n[gga fit, d={D}] row factors one fp16 step off: {rows_off} of {rows_seen}; column factors (heads with all '
+          f'rows equal): {cols_off} of {cols_seen}; heads byte-identical to the oracle: {heads_exact} of {heads}')
+    assert rows_off <= 2e-3 * rows_seen and cols_off <= 2e-3 * cols_seen, (rows_off, rows_seen, cols_off, cols_seen)
