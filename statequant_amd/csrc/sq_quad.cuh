@@ -364,7 +364,29 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     const float sm = COLVEC ? s : s * cmul;
     const float off = -128.0f * sm;
     v4f acc[NT];
-    if constexpr (T::BITS == 8) {
+    // int8 with one scale group per row: the whole half block is folded in units of the row's old scale x decay
+    // (S / sm = code + sum_i (du_i / sm) kx_i), so the codes need neither conversion nor multiplication on the vector
+    // ALU -- they enter the accumulators through the matrix core: each byte, biased to unsigned, becomes the fp16
+    // number 1024 + byte by a byte permute (exponent byte 0x64 on top), and one v_mfma_f32_16x16x16_f16 against the
+    // 16 x 16 identity hands every lane its own four numbers back as fp32 on top of the constant -1152 (exact).
+    constexpr bool UNITS = T::BITS == 8 && T::NG == 1 && !COLVEC;
+    float unit = 1.0f;                                       // what one accumulator unit is worth
+    if constexpr (UNITS) {
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        unit = fmaxf(sm, 1e-30f);                            // a vanished old state: its term is below any scale
+        v4h ident;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ident[j] = (n == 4 * q + j) ? _Float16(1.0f) : _Float16(0.0f);
+        const v4f bias = {-1152.0f, -1152.0f, -1152.0f, -1152.0f};
+#pragma unroll
+        for (int d = 0; d < NW32; ++d) {
+            const uint32_t u = w[d] ^ 0x80808080u;
+            v2u h2;
+            h2.x = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);      // halves 1024 + byte 0, 1024 + byte 1
+            h2.y = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);      // bytes 2, 3
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(ident, __builtin_bit_cast(v4h, h2), bias, 0, 0, 0);
+        }
+    } else if constexpr (T::BITS == 8) {
 #pragma unroll
         for (int d = 0; d < NW32; ++d) {
             const uint32_t u = w[d] ^ 0x80808080u;
@@ -390,11 +412,17 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
         }
     }
     // the m rank-1 updates: first operand = keys (result row i = 4 q' + b <-> column q' CL + 4 ct + b), second = values
+    float bv[MT4];
+    {
+        const float runit = UNITS ? 1.0f / unit : 1.0f;
+#pragma unroll
+        for (int t = 0; t < MT4; ++t) bv[t] = UNITS ? bop[t] * runit : bop[t];
+    }
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct)
 #pragma unroll
         for (int t = 0; t < MT4; ++t)
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop[ct][t], bop[t], acc[ct], 0, 0, 0);
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop[ct][t], bv[t], acc[ct], 0, 0, 0);
     // absmax of the lane's columns (three-operand maxima), then of its scale group
     float mx = 0.0f;
 #pragma unroll
@@ -404,8 +432,8 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     }
     if constexpr (LPG >= 2) { const Pair pm = pair16(mx); mx = fmaxf(pm.lo, pm.hi); }
     if constexpr (LPG >= 4) { const Pair pm = pair32(mx); mx = fmaxf(pm.lo, pm.hi); }
-    const float sc = fp16_scale(mx, T::QMAX);
-    const float rs = 1.0f / sc;
+    const float sc = fp16_scale(UNITS ? mx * unit : mx, T::QMAX);
+    const float rs = UNITS ? unit * (1.0f / sc) : 1.0f / sc;
     if (q % LPG == 0) *sc_out = f32_to_f16(sc);
     // new codes, back into the LDS image.  A scale in fp16's normal range cannot push a quotient past qmax + 1/2, so
     // the clamp is only compiled into the path taken when some lane's scale is subnormal (or at its floor).
