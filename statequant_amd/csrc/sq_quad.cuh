@@ -1,6 +1,7 @@
 // The state tile of one (sequence, value head) shared by the wavefronts of one workgroup: every wavefront owns NB of
-// the tile's 32-row blocks.  Shared by the Gated DeltaNet, KDA and Mamba2 step kernels for int4 / int8 codes with
-// key-axis scale groups and a power-of-two row size.
+// the tile's 32-row blocks.  Shared by the Gated DeltaNet and Mamba2 workgroup-per-key-head step kernels (int4 / int8
+// codes with key-axis scale groups and a power-of-two row size); the fold also carries the per-column factors a
+// per-channel decay needs (COLVEC).
 //
 // What this buys over one wavefront per tile (sq_tile.cuh, kept for the other formats):
 //   * a tile's life is a quarter as long, so the launch's ramp-up and tail shrink and the dispatcher balances the
@@ -26,19 +27,6 @@
 #include "sq_params.h"
 
 namespace sq {
-
-// Compute units of the current device (queried once per process and device; 256 on an MI355X).
-inline int quad_compute_units() {
-    static int cached[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (!cached[dev]) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
 
 // LDS-only release / acquire around a workgroup barrier: the state codes still in flight from global memory (plain
 // register loads) are not waited for.
