@@ -74,6 +74,8 @@ GGA_SHAPES = [(128, 128), (64, 64)]                  # (d_k, d_v) of the mixed-w
 PARAMS = {'gdn': 'GdnParams', 'kda': 'KdaParams', 'mamba2': 'Mamba2Params'}
 # families with a workgroup-per-key-head kernel (sq_<family>_quad.cuh) -> value heads per workgroup that are built
 QUAD_FAMILIES = {'gdn': (2, 1), 'mamba2': (4, 2, 1)}
+# ... and their compile-time specialisations, most specific first (0: everything read from the arguments)
+QUAD_SPECS = {'gdn': (1, 2, 0), 'mamba2': (1, 0)}
 CHUNK = 6                                            # instances per translation unit
 
 
@@ -92,6 +94,13 @@ QUAD_OK = {'gdn': [
     '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
     '    };',
     '    return ok(p.q, p.s_q, p.q_dt) && ok(p.k, p.s_k, p.k_dt);',
+    '}',
+    '// which compiled-in serving case the call is (SPEC of gdn_quad_kernel), 0: none',
+    'static int gdn_quad_spec(const GdnParams& p) {',
+    '    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;',
+    '    if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;',
+    '    if (!p.gate) return (p.a_dt == 0 && p.bt_dt == 0) ? 1 : 0;',
+    '    return (p.a_dt == 1 && p.bt_dt == 1 && p.A_log_dt == 0 && p.dt_bias_dt == 0) ? 2 : 0;',
     '}'],
     'mamba2': [
     '// B, C rows that 16-byte vector loads can address',
@@ -100,6 +109,11 @@ QUAD_OK = {'gdn': [
     '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
     '    };',
     '    return ok(p.B, p.s_B, p.B_dt) && ok(p.C, p.s_C, p.C_dt);',
+    '}',
+    'static int mamba2_quad_spec(const Mamba2Params& p) {',
+    '    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;',
+    '    if (p.x_dt != 1 || p.B_dt != 1 || p.C_dt != 1 || p.out_dt != 1) return 0;',
+    '    return (p.dt_dt == 0 && p.A_dt == 0 && p.D_dt == 0 && p.dt_bias_dt == 0) ? 1 : 0;',
     '}']}
 
 
@@ -130,13 +144,16 @@ def quad_variants(fam, c):
             continue
         # register target: as many wavefronts per SIMD as LDS lets workgroups in, up to 6 (5 with the 16-token buffer);
         # asked for 7, the int4 kernels spill into scratch memory inside the fold (measured: +60 % bytes written)
-        out.append((nb, gh, max(1, min(6 if mmax <= 8 else 5, -(-wgs * nw // 4)))))
+        wpe = max(1, min(6 if mmax <= 8 else 5, -(-wgs * nw // 4)))
+        # the serving cases compiled in (SPEC of the kernels) for the default buffer: int8, 8 tokens
+        for spec in QUAD_SPECS[fam] if (qbuf and mmax == 8) else (0,):
+            out.append((nb, gh, wpe, spec))
     return out
 
 
 def _quad_name(fam, c, v):
-    nb, gh, wpe = v
-    return f'launch_{fam}_quad<{_tile(c)}, {nb}, {gh}, {wpe}>'
+    nb, gh, wpe, spec = v
+    return f'launch_{fam}_quad<{_tile(c)}, {nb}, {gh}, {wpe}, {spec}>'
 
 
 def _write_if_changed(path, text):
@@ -196,19 +213,21 @@ def generate():
         P = PARAMS[fam]
         d.append(f'template <class T> int launch_{fam}(const {P}&, hipStream_t);')
         if fam in QUAD_FAMILIES:
-            d.append(f'template <class T, int NB, int GH, int WPE> int launch_{fam}_quad(const {P}&, hipStream_t);')
+            d.append(f'template <class T, int NB, int GH, int WPE, int SPEC> int launch_{fam}_quad(const {P}&, hipStream_t);')
             d += QUAD_OK[fam]
         d.append(f'int dispatch_{fam}(const {P}& p, hipStream_t stream, bool run) {{')
         if fam in QUAD_FAMILIES:
             d.append(f'    const bool quad = !getenv("SQ_NO_QUAD") && (!run || {fam}_quad_ok(p));')
             d.append('    const int ghmax = getenv("SQ_GHMAX") ? atoi(getenv("SQ_GHMAX")) : 64;')
+            d.append(f'    const int spec = (run && !getenv("SQ_NO_SPEC")) ? {fam}_quad_spec(p) : 0;')
         # smallest sufficient buffer bound first
         for c in sorted(rows, key=lambda c: c[5]):
             bits, dk, dv, group, qbuf, mmax, axv = c
             cond = (f'p.bits == {bits} && p.dk == {dk} && p.dv == {dv} && p.group == {group} && p.axv == {axv} '
                     f'&& p.qbuf == {qbuf} && p.m <= {mmax}')
             for v in quad_variants(fam, c):
-                d.append(f'    if (quad && p.gqa % {v[1]} == 0 && {v[1]} <= ghmax && {cond}) return run ? {_quad_name(fam, c, v)}(p, stream) : 0;')
+                want = f'spec == {v[3]} && ' if v[3] else ''             # the general instance takes whatever is left
+                d.append(f'    if (quad && {want}p.gqa % {v[1]} == 0 && {v[1]} <= ghmax && {cond}) return run ? {_quad_name(fam, c, v)}(p, stream) : 0;')
             d.append(f'    if ({cond}) return run ? launch_{fam}<{_tile(c)}>(p, stream) : 0;')
         d.append('    return -1;\n}')
     d.append('template <int BITS, int DK, int GROUP, bool AXV> int launch_pack(const PackParams&, hipStream_t);')

@@ -26,10 +26,16 @@ struct Mamba2Loads {
     uint32_t xr[Q::NE], xr2[Q::NE], g0, g1, g2, g3, vr;
 };
 
-template <class T, int NB, int GH, int WPE>
+// SPEC = 1 compiles the serving case in (as in the Gated DeltaNet kernel): bf16 x / B / C / out, fp32 dt, A, D and
+// dt_bias, no dispatch order, head counts that are powers of two.  SPEC = 0 reads all of it from the arguments.
+template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
 void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd, int hv,
                         int hv_shift, const Mamba2Params p) {
+    constexpr bool FIX = SPEC > 0;
+    const int x_dt = FIX ? int(BF16) : p.x_dt, B_dt = FIX ? int(BF16) : p.B_dt, C_dt = FIX ? int(BF16) : p.C_dt;
+    const int out_dt = FIX ? int(BF16) : p.out_dt, dt_dt = FIX ? int(F32) : p.dt_dt, A_dt = FIX ? int(F32) : p.A_dt;
+    const int D_dt = FIX ? int(F32) : p.D_dt, dt_bias_dt = FIX ? int(F32) : p.dt_bias_dt;
     using Q = Quad<T, NB, GH>;
     using L = QuadLds<T, NB, GH, 2, 1>;
     constexpr int DK = T::DK, DV = T::DV, NW = Q::NW, NWH = Q::NWH, MM = T::MMAX, NE = Q::NE, NG = T::NG;
@@ -62,9 +68,9 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     {
         const int wg = blockIdx.x;
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
-        b = hv_shift >= 0 ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
+        b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
         grp = item - b * ngrp;
-        if (order) {
+        if (!FIX && order) {
             int pos = b;
             if (rows_per_xcd) {
                 const int x = pos / rows_per_xcd;
@@ -75,7 +81,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         slot = idx ? idx[b] : b;
     }
     const uint32_t h = grp * GH + hl;
-    const uint32_t hk = p.gqa_shift >= 0 ? h >> p.gqa_shift : h / uint32_t(p.gqa);
+    const uint32_t hk = (FIX || p.gqa_shift >= 0) ? h >> p.gqa_shift : h / uint32_t(p.gqa);
 
     const int lane = lane0;
     const int n32 = lane & 31, kb = lane >> 5;
@@ -87,25 +93,25 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     Mamba2Loads<T, Q> F;
     if constexpr (RQ == RK) {                                     // a single wavefront carries both vectors
         if (w == RQ) {
-            load_vec<NE>(advance(p.C, p.C_dt, uint64_t(uint32_t(b)) * p.s_C + hk * DK), p.C_dt, lane, F.xr);
-            load_vec<NE>(advance(p.B, p.B_dt, uint64_t(uint32_t(b)) * p.s_B + hk * DK), p.B_dt, lane, F.xr2);
+            load_vec<NE>(advance(p.C, C_dt, uint64_t(uint32_t(b)) * p.s_C + hk * DK), C_dt, lane, F.xr);
+            load_vec<NE>(advance(p.B, B_dt, uint64_t(uint32_t(b)) * p.s_B + hk * DK), B_dt, lane, F.xr2);
         }
     } else if (w == RQ || w == RK) {
         const bool isq = w == RQ;
-        const void* base = isq ? advance(p.C, p.C_dt, uint64_t(uint32_t(b)) * p.s_C + hk * DK)
-                               : advance(p.B, p.B_dt, uint64_t(uint32_t(b)) * p.s_B + hk * DK);
-        load_vec<NE>(base, isq ? p.C_dt : p.B_dt, lane, F.xr);
+        const void* base = isq ? advance(p.C, C_dt, uint64_t(uint32_t(b)) * p.s_C + hk * DK)
+                               : advance(p.B, B_dt, uint64_t(uint32_t(b)) * p.s_B + hk * DK);
+        load_vec<NE>(base, isq ? C_dt : B_dt, lane, F.xr);
     }
     if (wh == 0) {
-        F.g0 = load_raw_uniform(p.dt, p.dt_dt, uint64_t(uint32_t(b)) * p.s_dt + h);
-        F.g1 = load_raw_uniform(p.A, p.A_dt, h);
-        F.g2 = load_raw_uniform(p.dt_bias, p.dt_bias_dt, h);      // absent: the C ABI points them at A, so the loads
-        F.g3 = load_raw_uniform(p.D, p.D_dt, h);                  // need no branch
+        F.g0 = load_raw_uniform(p.dt, dt_dt, uint64_t(uint32_t(b)) * p.s_dt + h);
+        F.g1 = load_raw_uniform(p.A, A_dt, h);
+        F.g2 = load_raw_uniform(p.dt_bias, dt_bias_dt, h);      // absent: the C ABI points them at A, so the loads
+        F.g3 = load_raw_uniform(p.D, D_dt, h);                  // need no branch
     }
-    F.vr = load_raw(advance(p.x, p.x_dt, uint64_t(uint32_t(b)) * p.s_x + h * DV), p.x_dt, uint32_t(row));
-    void* const outp = advance(p.out, p.out_dt, uint64_t(uint32_t(b)) * p.s_out + h * DV);
+    F.vr = load_raw(advance(p.x, x_dt, uint64_t(uint32_t(b)) * p.s_x + h * DV), x_dt, uint32_t(row));
+    void* const outp = advance(p.out, out_dt, uint64_t(uint32_t(b)) * p.s_out + h * DV);
     if (idx && slot <= 0) {                              // padding row: zero output, touch nothing else
-        for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(outp, p.out_dt, r, 0.0f);
+        for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(outp, out_dt, r, 0.0f);
         return;
     }
     // ... and the slot's side
@@ -171,25 +177,25 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     };
     if constexpr (RQ == RK) {
         if (w == RQ) {
-            role_vector(F.xr, p.C_dt, 0);
-            role_vector(F.xr2, p.B_dt, 1);
+            role_vector(F.xr, C_dt, 0);
+            role_vector(F.xr2, B_dt, 1);
         }
     } else {
-        if (w == RQ) role_vector(F.xr, p.C_dt, 0);
-        if (w == RK) role_vector(F.xr, p.B_dt, 1);
+        if (w == RQ) role_vector(F.xr, C_dt, 0);
+        if (w == RK) role_vector(F.xr, B_dt, 1);
     }
     if (wh == 0) {                                       // this head's step size and decays
-        float dt = raw_to_f(F.g0, p.dt_dt);
-        if (p.has_dt_bias) dt = dt + raw_to_f(F.g2, p.dt_bias_dt);
+        float dt = raw_to_f(F.g0, dt_dt);
+        if (p.has_dt_bias) dt = dt + raw_to_f(F.g2, dt_bias_dt);
         if (p.dt_softplus) dt = dt <= 20.0f ? logf(1.0f + expf(dt)) : dt;
         if (p.dt_clamp) dt = fminf(fmaxf(dt, p.dt_min), p.dt_max);
-        const float g = raw_to_f(F.g1, p.A_dt) * dt;     // rounded on its own (no contraction into gcur + g)
+        const float g = raw_to_f(F.g1, A_dt) * dt;     // rounded on its own (no contraction into gcur + g)
         if (lane == 0) {
             lds_scal[0] = dt;
             lds_scal[1] = expf(F.gcur);
             lds_scal[2] = expf(g);
             lds_scal[3] = F.gcur + g;
-            lds_scal[4] = p.has_D ? raw_to_f(F.g3, p.D_dt) : 0.0f;
+            lds_scal[4] = p.has_D ? raw_to_f(F.g3, D_dt) : 0.0f;
         }
     }
     // ---- the loads land: LDS images of the row blocks, scales, raw buffer pieces ----
@@ -349,11 +355,11 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         const float u_i = T::QBUF ? uv[i] : (i < n ? uv[i] : 0.0f);
         accq = __builtin_fmaf(u_i, lane_bcast(cq, i), accq);
     }
-    const float xt = raw_to_f(vr, p.x_dt);
+    const float xt = raw_to_f(vr, x_dt);
     const float u = dt * xt;
     float y = __builtin_fmaf(bc, u, a * accq);
     if (p.has_D) y = __builtin_fmaf(dd, xt, y);
-    if (NB == 2 || kb == 0) store_f(outp, p.out_dt, row, y);
+    if (NB == 2 || kb == 0) store_f(outp, out_dt, row, y);
 
     // ---- append ----
     float us = 1.0f;
@@ -428,12 +434,12 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     }
 }
 
-template <class T, int NB, int GH, int WPE>
+template <class T, int NB, int GH, int WPE, int SPEC>
 int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     Mamba2Params p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     if (p.per_xcd == 0) p.rows_per_xcd = 0;
-    hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
+    hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
                        0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
     return int(hipGetLastError());
 }

@@ -156,3 +156,73 @@ def test_gdn_pace4_d128_values_scaled_per_head(m, bb):
 
     tal = run_gdn((4, 'k', 32), m, bb, B=3, HV=HV, HK=2, D=128, T=T, seed=22, v_scale=vs)
     check_gdn(tal, f'gdn pace4 d128 per-head v scale, buf{bb}', T, m)
+
+
+def _stepped_twice(step, blobs):
+    """Run `step(views_index)` on blob 0 with the compiled-in serving case allowed and on blob 1 with it switched off
+    (`SQ_NO_SPEC`: the general instance, which reads dtypes and options from the arguments)."""
+    import os
+    a = step(0)
+    os.environ['SQ_NO_SPEC'] = '1'
+    try:
+        b = step(1)
+    finally:
+        del os.environ['SQ_NO_SPEC']
+    assert torch.equal(a, b)
+    assert torch.equal(blobs[0], blobs[1])
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32), (4, 'k', 64)])
+@pytest.mark.parametrize('gated', [False, True])
+def test_gdn_serving_case_instances_match_the_general_one(fmt, gated):
+    """bf16 q / k / v / out with fp32 g, beta -- or the gate formed in the kernel from bf16 a, b and fp32 A_log, dt_bias
+    -- take kernel instances with those choices compiled in; they must leave exactly the bytes and outputs of the
+    general instance (two fold periods, a padding row, slots out of step)."""
+    from statequant_amd.kernels import SlotLayout
+    HV, HK, D, m, rows = 8, 4, 128, 8, 5
+    lay = SlotLayout(sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
+    gen = torch.Generator().manual_seed(31)
+    blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
+    views = [lay.views(b) for b in blobs]
+    idx = torch.tensor([4, 0, 2, 5, 1], dtype=torch.int32, device=DEV)
+    live = idx > 0
+    S0 = (torch.randn(rows, HV, D, D, generator=gen) * 0.4).to(DEV)
+    for v in views:
+        lay.write(v, idx[live].long(), S0[live])
+        v['NPTR'][idx[live].long()] = torch.tensor([0, 3, 6, 7], dtype=torch.int32, device=DEV)[:, None]
+    A_log, dtb = (torch.randn(HV, generator=gen) * 0.3).to(DEV), (torch.randn(HV, generator=gen) * 0.3).to(DEV)
+    r = lambda *s: torch.randn(*s, generator=gen).to(DEV)          # noqa: E731
+    for t in range(2 * m + 1):
+        q, k, v = r(rows, HK, D).bfloat16(), r(rows, HK, D).bfloat16(), r(rows, HV, D).bfloat16()
+        if gated:
+            kw = dict(gate=((r(rows, HV) * 0.5 - 2).bfloat16(), r(rows, HV).bfloat16(), A_log, dtb))
+        else:
+            kw = dict(g=-torch.nn.functional.softplus(r(rows, HV)), beta=torch.sigmoid(r(rows, HV)))
+
+        def step(i):
+            out = torch.full((rows, HV, D), 7.0, device=DEV, dtype=torch.bfloat16)
+            return lay.step(views[i], idx, q, k, v, out, D ** -0.5, **kw).clone()
+        _stepped_twice(step, blobs)
+
+
+def test_mamba2_serving_case_instance_matches_the_general_one():
+    H, G, DK, DV, m, rows = 16, 2, 128, 64, 8, 5
+    lay = Mamba2SlotLayout(sq.Quantizer(8, 'k', 128), H, G, DK, DV, m=m, buffer_bits=8)
+    gen = torch.Generator().manual_seed(32)
+    blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
+    views = [lay.views(b) for b in blobs]
+    idx = torch.tensor([4, 0, 2, 5, 1], dtype=torch.int32, device=DEV)
+    live = idx > 0
+    S0 = (torch.randn(rows, H, DV, DK, generator=gen) * 0.4).to(DEV)
+    for v in views:
+        lay.write(v, idx[live].long(), S0[live])
+        v['NPTR'][idx[live].long()] = torch.tensor([0, 3, 6, 7], dtype=torch.int32, device=DEV)[:, None]
+    A, D_, dtb = (t.to(DEV) for t in params(gen, H))
+    for t in range(2 * m + 1):
+        x, dt, Bm, C = m2_token(gen, rows, H, G, DK, DV)
+        x, Bm, C, dt = x.bfloat16().to(DEV), Bm.bfloat16().to(DEV), C.bfloat16().to(DEV), dt.to(DEV)
+
+        def step(i):
+            out = torch.full((rows, H, DV), 7.0, device=DEV, dtype=torch.bfloat16)
+            return lay.step(views[i], idx, x, dt, Bm, C, out, A, D_, dtb).clone()
+        _stepped_twice(step, blobs)
