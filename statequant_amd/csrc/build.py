@@ -74,8 +74,22 @@ GGA_SHAPES = [(128, 128), (64, 64)]                  # (d_k, d_v) of the mixed-w
 PARAMS = {'gdn': 'GdnParams', 'kda': 'KdaParams', 'mamba2': 'Mamba2Params'}
 # families with a workgroup-per-key-head kernel (sq_<family>_quad.cuh) -> value heads per workgroup that are built
 QUAD_FAMILIES = {'gdn': (2, 1), 'mamba2': (4, 2, 1)}
-# ... and their compile-time specialisations, most specific first (0: everything read from the arguments)
-QUAD_SPECS = {'gdn': (1, 2, 0), 'mamba2': (1, 0)}
+# compile-time specialisations of the step kernels (SPEC, sq_params.h), most specific first; 0: everything read from
+# the arguments.  Built for the default buffer (int8, 8 tokens) only.
+SPECS = {'gdn': (1, 2, 0), 'kda': (1, 0), 'mamba2': (1, 0)}
+
+
+def specs_of(fam, c, quad):
+    """SPEC values an instance is built for: the workgroup-per-key-head kernels for every case they serve, the
+    one-wavefront kernels for the cases that have no such kernel."""
+    bits, dk, dv, group, qbuf, mmax, axv = c
+    if not (qbuf and mmax == 8) or (not quad and quad_variants(fam, c)):
+        return (0,)
+    if not quad and fam != 'kda':
+        # measured on the one-wavefront kernels: KDA int4 g32 40.0 -> 38.9 us, GDN value-axis int4 36.3 -> 35.1, but
+        # value-axis int8 45.2 -> 48.4 and Mamba2 d_state 256 41.9 -> 48.1 (their register allocation tips over)
+        return (0,)
+    return SPECS[fam]
 CHUNK = 6                                            # instances per translation unit
 
 
@@ -94,13 +108,6 @@ QUAD_OK = {'gdn': [
     '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
     '    };',
     '    return ok(p.q, p.s_q, p.q_dt) && ok(p.k, p.s_k, p.k_dt);',
-    '}',
-    '// which compiled-in serving case the call is (SPEC of gdn_quad_kernel), 0: none',
-    'static int gdn_quad_spec(const GdnParams& p) {',
-    '    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;',
-    '    if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;',
-    '    if (!p.gate) return (p.a_dt == 0 && p.bt_dt == 0) ? 1 : 0;',
-    '    return (p.a_dt == 1 && p.bt_dt == 1 && p.A_log_dt == 0 && p.dt_bias_dt == 0) ? 2 : 0;',
     '}'],
     'mamba2': [
     '// B, C rows that 16-byte vector loads can address',
@@ -109,11 +116,6 @@ QUAD_OK = {'gdn': [
     '        return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && (uint64_t(stride) * (dt == 0 ? 4 : 2)) % 16 == 0;',
     '    };',
     '    return ok(p.B, p.s_B, p.B_dt) && ok(p.C, p.s_C, p.C_dt);',
-    '}',
-    'static int mamba2_quad_spec(const Mamba2Params& p) {',
-    '    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;',
-    '    if (p.x_dt != 1 || p.B_dt != 1 || p.C_dt != 1 || p.out_dt != 1) return 0;',
-    '    return (p.dt_dt == 0 && p.A_dt == 0 && p.D_dt == 0 && p.dt_bias_dt == 0) ? 1 : 0;',
     '}']}
 
 
@@ -146,7 +148,7 @@ def quad_variants(fam, c):
         # asked for 7, the int4 kernels spill into scratch memory inside the fold (measured: +60 % bytes written)
         wpe = max(1, min(6 if mmax <= 8 else 5, -(-wgs * nw // 4)))
         # the serving cases compiled in (SPEC of the kernels) for the default buffer: int8, 8 tokens
-        for spec in QUAD_SPECS[fam] if (qbuf and mmax == 8) else (0,):
+        for spec in SPECS[fam] if (qbuf and mmax == 8) else (0,):
             out.append((nb, gh, wpe, spec))
     return out
 
@@ -168,9 +170,10 @@ def generate():
     os.makedirs(OUT, exist_ok=True)
     units = []
     for fam, rows in CASES.items():
-        for k in range(0, len(rows), CHUNK):
-            body = ''.join(f'template int launch_{fam}<{_tile(c)}>(const {PARAMS[fam]}&, hipStream_t);\n'
-                           for c in rows[k:k + CHUNK])
+        insts = [(c, sp) for c in rows for sp in specs_of(fam, c, False)]
+        for k in range(0, len(insts), CHUNK):
+            body = ''.join(f'template int launch_{fam}<{_tile(c)}, {sp}>(const {PARAMS[fam]}&, hipStream_t);\n'
+                           for c, sp in insts[k:k + CHUNK])
             path = os.path.join(OUT, f'inst_{fam}_{k // CHUNK:02d}.hip')
             _write_if_changed(path, f'// generated by build.py\n#include "../sq_{fam}.cuh"\nnamespace sq {{\n{body}}}\n')
             units.append(path)
@@ -211,15 +214,15 @@ def generate():
          '}']
     for fam, rows in CASES.items():
         P = PARAMS[fam]
-        d.append(f'template <class T> int launch_{fam}(const {P}&, hipStream_t);')
+        d.append(f'template <class T, int SPEC> int launch_{fam}(const {P}&, hipStream_t);')
         if fam in QUAD_FAMILIES:
             d.append(f'template <class T, int NB, int GH, int WPE, int SPEC> int launch_{fam}_quad(const {P}&, hipStream_t);')
             d += QUAD_OK[fam]
         d.append(f'int dispatch_{fam}(const {P}& p, hipStream_t stream, bool run) {{')
+        d.append('    const int spec = (run && !getenv("SQ_NO_SPEC")) ? serving_case(p) : 0;')
         if fam in QUAD_FAMILIES:
             d.append(f'    const bool quad = !getenv("SQ_NO_QUAD") && (!run || {fam}_quad_ok(p));')
             d.append('    const int ghmax = getenv("SQ_GHMAX") ? atoi(getenv("SQ_GHMAX")) : 64;')
-            d.append(f'    const int spec = (run && !getenv("SQ_NO_SPEC")) ? {fam}_quad_spec(p) : 0;')
         # smallest sufficient buffer bound first
         for c in sorted(rows, key=lambda c: c[5]):
             bits, dk, dv, group, qbuf, mmax, axv = c
@@ -228,7 +231,9 @@ def generate():
             for v in quad_variants(fam, c):
                 want = f'spec == {v[3]} && ' if v[3] else ''             # the general instance takes whatever is left
                 d.append(f'    if (quad && {want}p.gqa % {v[1]} == 0 && {v[1]} <= ghmax && {cond}) return run ? {_quad_name(fam, c, v)}(p, stream) : 0;')
-            d.append(f'    if ({cond}) return run ? launch_{fam}<{_tile(c)}>(p, stream) : 0;')
+            for sp in specs_of(fam, c, False):
+                want = f'spec == {sp} && ' if sp else ''
+                d.append(f'    if ({want}{cond}) return run ? launch_{fam}<{_tile(c)}, {sp}>(p, stream) : 0;')
         d.append('    return -1;\n}')
     d.append('template <int BITS, int DK, int GROUP, bool AXV> int launch_pack(const PackParams&, hipStream_t);')
     d.append('int dispatch_pack(const PackParams& p, hipStream_t stream, bool run) {')
@@ -317,8 +322,8 @@ def build(jobs=None, force=False, verbose=True):
             print(f'[build] {LIB} is up to date')
         return LIB
     if verbose:
-        n = sum(len(r) for r in CASES.values())
-        print(f'[build] hipcc {ARCH}: {n} kernel instances in {len(units)} translation units, {jobs} jobs')
+        n = sum(len(specs_of(fam, c, False)) + len(quad_variants(fam, c)) for fam, r in CASES.items() for c in r)
+        print(f'[build] hipcc {ARCH}: {n} step-kernel instances in {len(units)} translation units, {jobs} jobs')
     with cf.ThreadPoolExecutor(jobs) as ex:
         objs = list(ex.map(lambda u: _compile(u, force), units))
     cmd = ['hipcc', '--offload-arch=' + ARCH, '-shared', '-fPIC', '-o', LIB, *objs]

@@ -125,8 +125,10 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < nl ? i : nl - 1]; }
 }
 
-template <class T>
-__global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
+template <class T, int SPEC>
+__global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams args) {
+    GdnParams p = args;
+    assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 2>;
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_q = reinterpret_cast<float*>(lds + L::X);
@@ -303,9 +305,9 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams p) {
     }
 }
 
-template <class T>
+template <class T, int SPEC>
 int launch_gdn(const GdnParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL(gdn_step_kernel<T>, dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    hipLaunchKernelGGL((gdn_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     return int(hipGetLastError());
 }
 

@@ -14,8 +14,10 @@
 
 namespace sq {
 
-template <class T>
-__global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
+template <class T, int SPEC>
+__global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args) {
+    KdaParams p = args;
+    assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 3, 2>;                                   // q, k (normalised), G_n
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_q = reinterpret_cast<float*>(lds + L::X);
@@ -280,9 +282,9 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams p) {
     if (l.lane == 0) *np = full ? 0 : n + 1;
 }
 
-template <class T>
+template <class T, int SPEC>
 int launch_kda(const KdaParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL(kda_step_kernel<T>, dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     return int(hipGetLastError());
 }
 

@@ -14,8 +14,10 @@ namespace sq {
 
 // Occupancy target: four wavefronts per SIMD; the d_state-256 tile does not fit 128 registers, and asked for two it
 // is compiled at 234 without spills (asked for four the compiler gives up at 364, one wavefront per SIMD).
-template <class T>
-__global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(const Mamba2Params p) {
+template <class T, int SPEC>
+__global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(const Mamba2Params args) {
+    Mamba2Params p = args;
+    assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 1, 1>;
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     float* lds_cv = reinterpret_cast<float*>(lds + L::X);
@@ -211,9 +213,9 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
     }
 }
 
-template <class T>
+template <class T, int SPEC>
 int launch_mamba2(const Mamba2Params& p, hipStream_t stream) {
-    hipLaunchKernelGGL(mamba2_step_kernel<T>, dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    hipLaunchKernelGGL((mamba2_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
     return int(hipGetLastError());
 }
 

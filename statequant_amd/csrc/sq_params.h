@@ -121,6 +121,62 @@ struct GgaParams {
     float* Y;                                     // load
 };
 
+// The serving cases a step kernel can be compiled for (template argument SPEC; 0 = read every choice from the
+// arguments): bf16 operands and output, no dispatch order, head counts that are powers of two, and per family
+//   GDN     1: g and beta given as fp32;  2: the gate formed in the kernel from bf16 a, b and fp32 A_log, dt_bias
+//   KDA     1: fp32 g and beta
+//   Mamba2  1: fp32 dt, A, D, dt_bias
+// `serving_case` tells which one a call is (host); `assume_serving_case<SPEC>` overwrites those fields of a kernel's
+// private copy of its arguments with the constants (device), after which the compiler drops the scalar branches on
+// them -- about a microsecond per launch on the 128 x 128 steps.  Dtype codes: 0 fp32, 1 bf16.
+inline int serving_case(const GdnParams& p) {
+    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;
+    if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;
+    if (!p.gate) return (p.a_dt == 0 && p.bt_dt == 0) ? 1 : 0;
+    return (p.a_dt == 1 && p.bt_dt == 1 && p.A_log_dt == 0 && p.dt_bias_dt == 0) ? 2 : 0;
+}
+inline int serving_case(const KdaParams& p) {
+    if (p.order || p.hv_shift < 0) return 0;
+    if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;
+    return (p.g_dt == 0 && p.beta_dt == 0) ? 1 : 0;
+}
+inline int serving_case(const Mamba2Params& p) {
+    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;
+    if (p.x_dt != 1 || p.B_dt != 1 || p.C_dt != 1 || p.out_dt != 1) return 0;
+    return (p.dt_dt == 0 && p.A_dt == 0 && p.D_dt == 0 && p.dt_bias_dt == 0) ? 1 : 0;
+}
+template <int SPEC>
+__device__ __forceinline__ void assume_serving_case(GdnParams& p) {
+    if constexpr (SPEC > 0) {
+        p.q_dt = p.k_dt = p.v_dt = p.out_dt = 1;
+        p.a_dt = p.bt_dt = SPEC == 1 ? 0 : 1;
+        p.A_log_dt = p.dt_bias_dt = 0;
+        p.gate = SPEC == 2;
+        p.order = nullptr;
+        __builtin_assume(p.hv_shift >= 0);
+        __builtin_assume(p.gqa_shift >= 0);
+    }
+}
+template <int SPEC>
+__device__ __forceinline__ void assume_serving_case(KdaParams& p) {
+    if constexpr (SPEC > 0) {
+        p.q_dt = p.k_dt = p.v_dt = p.out_dt = 1;
+        p.g_dt = p.beta_dt = 0;
+        p.order = nullptr;
+        __builtin_assume(p.hv_shift >= 0);
+    }
+}
+template <int SPEC>
+__device__ __forceinline__ void assume_serving_case(Mamba2Params& p) {
+    if constexpr (SPEC > 0) {
+        p.x_dt = p.B_dt = p.C_dt = p.out_dt = 1;
+        p.dt_dt = p.A_dt = p.D_dt = p.dt_bias_dt = 0;
+        p.order = nullptr;
+        __builtin_assume(p.hv_shift >= 0);
+        __builtin_assume(p.gqa_shift >= 0);
+    }
+}
+
 // hipError_t of the launch (0 = enqueued), or -1 if no kernel is compiled for the layout.  run = false: probe only.
 int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
 int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);

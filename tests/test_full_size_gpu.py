@@ -172,7 +172,7 @@ def _stepped_twice(step, blobs):
     assert torch.equal(blobs[0], blobs[1])
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32), (4, 'k', 64)])
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32), (4, 'k', 64), (4, 'v', 32), 'bf16'])      # the last two: one wavefront per tile
 @pytest.mark.parametrize('gated', [False, True])
 def test_gdn_serving_case_instances_match_the_general_one(fmt, gated):
     """bf16 q / k / v / out with fp32 g, beta -- or the gate formed in the kernel from bf16 a, b and fp32 A_log, dt_bias
@@ -180,7 +180,7 @@ def test_gdn_serving_case_instances_match_the_general_one(fmt, gated):
     general instance (two fold periods, a padding row, slots out of step)."""
     from statequant_amd.kernels import SlotLayout
     HV, HK, D, m, rows = 8, 4, 128, 8, 5
-    lay = SlotLayout(sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
+    lay = SlotLayout(fmt if fmt == 'bf16' else sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
     gen = torch.Generator().manual_seed(31)
     blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
     views = [lay.views(b) for b in blobs]
@@ -225,4 +225,27 @@ def test_mamba2_serving_case_instance_matches_the_general_one():
         def step(i):
             out = torch.full((rows, H, DV), 7.0, device=DEV, dtype=torch.bfloat16)
             return lay.step(views[i], idx, x, dt, Bm, C, out, A, D_, dtb).clone()
+        _stepped_twice(step, blobs)
+
+
+@pytest.mark.parametrize('fmt', [(4, 'k', 32), (8, 'v', 32)])
+def test_kda_serving_case_instance_matches_the_general_one(fmt):
+    H, D, m, rows = 4, 128, 8, 5
+    lay = KDASlotLayout(sq.Quantizer(*fmt), H, D, D, m=m, buffer_bits=8)
+    gen = torch.Generator().manual_seed(33)
+    blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
+    views = [lay.views(b) for b in blobs]
+    idx = torch.tensor([4, 0, 2, 5, 1], dtype=torch.int32, device=DEV)
+    live = idx > 0
+    S0 = (torch.randn(rows, H, D, D, generator=gen) * 0.4).to(DEV)
+    for v in views:
+        lay.write(v, idx[live].long(), S0[live])
+        v['NPTR'][idx[live].long()] = torch.tensor([0, 3, 6, 7], dtype=torch.int32, device=DEV)[:, None]
+    for t in range(2 * m + 1):
+        q, k, v, g, beta = kda_token(gen, rows, H, D, D)
+        q, k, v, g, beta = q.bfloat16().to(DEV), k.bfloat16().to(DEV), v.bfloat16().to(DEV), g.to(DEV), beta.to(DEV)
+
+        def step(i):
+            out = torch.full((rows, H, D), 7.0, device=DEV, dtype=torch.bfloat16)
+            return lay.step(views[i], idx, q, k, v, g, beta, out).clone()
         _stepped_twice(step, blobs)
