@@ -20,29 +20,39 @@
 
 namespace sq {
 
-// NE consecutive elements of a float vector of run-time dtype, one load per lane: raw[t] = element NE lane + t as
-// `load_raw` leaves it (fp32 bits, or the 16-bit pattern).  The vector's base must be 4-byte aligned.
+// NE consecutive elements of a float vector of run-time dtype, one load per lane, kept AS LOADED: w holds the
+// lane's NE fp32 words, or its NE 16-bit patterns packed two per word (NE = 1: the pattern itself).  Nothing is
+// computed from the loaded words here -- not even the split of a packed pair -- because any use would make the
+// wavefront wait for this load before it has issued the ones behind it; `vec_elem` unpacks at the point of use.
+// The vector's base must be 16-byte aligned.
 template <int NE>
-__device__ __forceinline__ void load_vec(const void* base, int dt, int lane, uint32_t (&raw)[NE]) {
+__device__ __forceinline__ void load_vec(const void* base, int dt, int lane, uint32_t (&w)[NE]) {
     if (dt == F32) {
-        if constexpr (NE == 1) raw[0] = reinterpret_cast<const uint32_t*>(base)[lane];
+        if constexpr (NE == 1) w[0] = reinterpret_cast<const uint32_t*>(base)[lane];
         else if constexpr (NE == 2) {
             const v2u x = reinterpret_cast<const v2u*>(base)[lane];
-            raw[0] = x.x; raw[1] = x.y;
+            w[0] = x.x; w[1] = x.y;
         } else {
             const v4u x = reinterpret_cast<const v4u*>(base)[lane];
-            raw[0] = x.x; raw[1] = x.y; raw[2] = x.z; raw[3] = x.w;
+            w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
         }
     } else {
-        if constexpr (NE == 1) raw[0] = reinterpret_cast<const uint16_t*>(base)[lane];
+        if constexpr (NE == 1) w[0] = reinterpret_cast<const uint16_t*>(base)[lane];
         else if constexpr (NE == 2) {
-            const uint32_t x = reinterpret_cast<const uint32_t*>(base)[lane];
-            raw[0] = x & 0xFFFFu; raw[1] = x >> 16;
+            w[0] = reinterpret_cast<const uint32_t*>(base)[lane];
+            w[1] = 0;
         } else {
             const v2u x = reinterpret_cast<const v2u*>(base)[lane];
-            raw[0] = x.x & 0xFFFFu; raw[1] = x.x >> 16; raw[2] = x.y & 0xFFFFu; raw[3] = x.y >> 16;
+            w[0] = x.x; w[1] = x.y; w[2] = 0; w[3] = 0;
         }
     }
+}
+// Element t of what `load_vec` loaded, as fp32.
+template <int NE>
+__device__ __forceinline__ float vec_elem(const uint32_t (&w)[NE], int dt, int t) {
+    if (dt == F32) return as_f32(w[t]);
+    const uint32_t h = NE == 1 ? w[0] : (w[t / 2] >> (16 * (t % 2))) & 0xFFFFu;
+    return raw_to_f(h, dt);
 }
 
 // Everything a wavefront loads for one item, as issued loads (raw bits; nothing here waits for memory).
@@ -156,20 +166,28 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         F.vr = load_raw(advance(p.v, v_dt, uint64_t(b) * p.s_v + h * DV), v_dt, uint32_t(row));
     };
     // ... and the slot's side (not for a padding row: nothing of a slot is touched then)
-    auto issue_slot = [&](const GdnAddr<T>& A, int lane, int n32) {
-        F.np = *A.np;
-        F.gcur = *A.gcp;
+    // The counters and the row blocks go out first and by themselves: the scheduling barrier behind them keeps the
+    // address arithmetic of the other eight fields, and the first use of the fill count, from being scheduled in
+    // among them (the compiler had put half of the row-block loads behind the wait for the fill count).
+    auto issue_codes = [&](const TileId& tid, int32_t slot, int lane) {
+        const uint32_t seq = slot, h = tid.h;
+        F.np = *field(p.st.NPTR, seq, p.st.sN, h);
+        F.gcur = *field(p.st.GCUR, seq, p.st.sGC, h);
+        const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
             for (int t = 0; t < Q::NLD; ++t)
-                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto issue_slot = [&](const GdnAddr<T>& A, int lane, int n32) {
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
             for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(A.SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
-        // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count, a
-        // scalar load issued ahead of everything above, is here by now
+        // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count,
+        // requested ahead of the row blocks, is here by now
         const uint32_t nfill = uint32_t(F.np & (m - 1));
         const uint32_t nl = nfill > 0 ? nfill : 1u;
         // buffered values of this wavefront's rows: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
@@ -201,12 +219,14 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);    // chunk `lane` of a 1 KB piece in the LDS image
         issue(cur, lane, n32, row);
         const TileId tid = tile_of(cur);
-        const GdnAddr<T> A = gdn_addr<T>(p, tid, cur.slot);
-        void* const outp = advance(p.out, out_dt, A.obase);
-        if (!A.live) {                                   // padding row: zero output, touch nothing else
-            for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(outp, out_dt, r, 0.0f);
+        if (idx && cur.slot <= 0) {                      // padding row: zero output, touch nothing else
+            void* const o0 = advance(p.out, out_dt, (uint64_t(uint32_t(tid.b)) * uint32_t(p.hv) + uint32_t(tid.h)) * DV);
+            for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(o0, out_dt, r, 0.0f);
             return;
         }
+        issue_codes(tid, cur.slot, lane);
+        const GdnAddr<T> A = gdn_addr<T>(p, tid, cur.slot);
+        void* const outp = advance(p.out, out_dt, A.obase);
         issue_slot(A, lane, n32);
         // every load of the item is in flight from here on: keep the compiler from sinking any of them to its use,
         // and from scheduling a use (a conversion, with its wait) up among them
@@ -218,7 +238,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
             float xe[NE], ss = 0.0f;
 #pragma unroll
             for (int t = 0; t < NE; ++t) {
-                xe[t] = raw_to_f(raw[t], dt);
+                xe[t] = vec_elem<NE>(raw, dt, t);
                 ss = __builtin_fmaf(xe[t], xe[t], ss);
             }
             const float nrm = sqrtf(lanes_sum<WAVE>(ss) + 1e-6f);

@@ -115,14 +115,10 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         return;
     }
     // ... and the slot's side
+    // the counters and the row blocks first and by themselves: the scheduling barrier behind them keeps the address
+    // arithmetic of the other fields, and the first use of the fill count, from being scheduled in among them
     const uint32_t seq = slot, um = m;
     uint8_t* const Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
-    uint16_t* const SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
-    uint8_t* const KBp = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
-    uint8_t* const UBp = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
-    uint16_t* const KBSp = field(p.st.KBS, seq, p.st.sKBS, hk * um);
-    uint16_t* const UBSp = field(p.st.UBS, seq, p.st.sUBS, h * um);
-    float* const GBh = field(p.st.GB, seq, p.st.sGB, h * um);
     float* const gcp = field(p.st.GCUR, seq, p.st.sGC, h);
     int32_t* const np = field(p.st.NPTR, seq, p.st.sN, h);
     F.np = *np;
@@ -132,12 +128,19 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
 #pragma unroll
         for (int t = 0; t < Q::NLD; ++t)
             F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+    __builtin_amdgcn_sched_barrier(0);
+    uint16_t* const SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
+    uint8_t* const KBp = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
+    uint8_t* const UBp = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
+    uint16_t* const KBSp = field(p.st.KBS, seq, p.st.sKBS, hk * um);
+    uint16_t* const UBSp = field(p.st.UBS, seq, p.st.sUBS, h * um);
+    float* const GBh = field(p.st.GB, seq, p.st.sGB, h * um);
 #pragma unroll
     for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
         for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
-    // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count, a
-    // scalar load issued ahead of everything above, is here by now
+    // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count,
+    // requested ahead of the row blocks, is here by now
     const uint32_t nfill = uint32_t(F.np & (m - 1));
     const uint32_t nl = nfill > 0 ? nfill : 1u;
     // buffered values of this wavefront's rows: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
@@ -169,7 +172,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     auto role_vector = [&](const uint32_t (&raw)[NE], int dt, int v) {
         float xe[NE];
 #pragma unroll
-        for (int t = 0; t < NE; ++t) xe[t] = raw_to_f(raw[t], dt);
+        for (int t = 0; t < NE; ++t) xe[t] = vec_elem<NE>(raw, dt, t);
         if constexpr (NE == 1) lds_xn[v * DK + lane] = xe[0];
         else if constexpr (NE == 2) *reinterpret_cast<float2*>(lds_xn + v * DK + 2 * lane) = make_float2(xe[0], xe[1]);
         else *reinterpret_cast<float4*>(lds_xn + v * DK + 4 * lane) = make_float4(xe[0], xe[1], xe[2], xe[3]);
