@@ -277,7 +277,11 @@ __device__ __forceinline__ float lds_raw(const uint8_t* base, int idx) {
 // w = codes ^ 0x80.. and o = -128 s this is (code x s) rounded once, bit-identical to convert-then-multiply).
 template <int B>
 __device__ __forceinline__ float ubyte_fma(uint32_t w, float s, float o) {
-    const float f = float((w >> (8 * B)) & 0xFFu);          // v_cvt_f32_ubyteB
+    float f;                                                 // one instruction whichever byte (left to the compiler,
+    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(w));      // bytes 1 .. 3 of a masked word
+    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(w)); // cost a shift each)
+    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(w));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(w));
     return __builtin_fmaf(f, s, o);
 }
 
