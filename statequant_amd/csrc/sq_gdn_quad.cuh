@@ -112,35 +112,33 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
 
     // ---- this workgroup's item: (batch row, head group), dealt so that every XCD walks a contiguous range ----
     const int ngrp = hv / GH;                                     // head groups per batch row
-    struct Item { int b, grp, slot; };
-    Item cur;
+    TileId tid;
+    int32_t slot;
     {
         const int wg = blockIdx.x;
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
-        cur.b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
-        cur.grp = item - cur.b * ngrp;
+        tid.b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
+        tid.h = (item - tid.b * ngrp) * GH + hl;
         if (!FIX && order) {
-            int pos = cur.b;
+            int pos = tid.b;
             if (rows_per_xcd) {
                 const int x = pos / rows_per_xcd;
                 pos = (pos - x * rows_per_xcd) * 8 + x;
             }
-            cur.b = order[pos];
+            tid.b = order[pos];
         }
-        cur.slot = idx ? idx[cur.b] : cur.b;
+        slot = idx ? idx[tid.b] : tid.b;
+        tid.hk = (FIX || p.gqa_shift >= 0) ? tid.h >> p.gqa_shift : tid.h / p.gqa;
     }
-    auto tile_of = [&](const Item& it) {
-        TileId t;
-        t.b = it.b;
-        t.h = it.grp * GH + hl;
-        t.hk = (FIX || p.gqa_shift >= 0) ? t.h >> p.gqa_shift : t.h / p.gqa;
-        return t;
-    };
+    const int lane = lane0;
+    const int n32 = lane & 31, kb = lane >> 5;
+    // the row of the head this lane finishes after the pass (NB = 2: the wavefront's halves take a block each)
+    const int row = (wh * NB + (NB == 2 ? kb : 0)) * T::MR + n32;
+    const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);        // chunk `lane` of a 1 KB piece in the LDS image
 
-    // ---- issue every load of an item: first the token's own operands (their addresses need the batch row only) ...
+    // ---- issue every load: first the token's own operands (their addresses need the batch row only) ...
     GdnLoads<T, Q> F;
-    auto issue = [&](const Item& it, int lane, int n32, int row) {
-        const TileId tid = tile_of(it);
+    {
         const uint32_t b = tid.b, h = tid.h;
         if constexpr (RQ == RK) {                                 // a single wavefront carries both vectors
             if (w == RQ) {
@@ -156,7 +154,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         if (wh == 0) {
             F.g0 = load_raw_uniform(p.a, a_dt, uint64_t(b) * p.s_a + h);
             F.g1 = load_raw_uniform(p.bt, bt_dt, uint64_t(b) * p.s_bt + h);
-            if constexpr (SPEC != 1) {                    // without a gate they alias g (readable, unused)
+            if constexpr (SPEC != 1) {                            // without a gate they alias g (readable, unused)
                 F.g2 = load_raw_uniform(p.A_log, A_log_dt, h);
                 F.g3 = load_raw_uniform(p.dt_bias, dt_bias_dt, h);
             } else {
@@ -164,12 +162,17 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
             }
         }
         F.vr = load_raw(advance(p.v, v_dt, uint64_t(b) * p.s_v + h * DV), v_dt, uint32_t(row));
-    };
-    // ... and the slot's side (not for a padding row: nothing of a slot is touched then)
-    // The counters and the row blocks go out first and by themselves: the scheduling barrier behind them keeps the
-    // address arithmetic of the other eight fields, and the first use of the fill count, from being scheduled in
-    // among them (the compiler had put half of the row-block loads behind the wait for the fill count).
-    auto issue_codes = [&](const TileId& tid, int32_t slot, int lane) {
+    }
+    if (idx && slot <= 0) {                              // padding row: zero output, touch nothing of a slot
+        void* const o0 = advance(p.out, out_dt, (uint64_t(uint32_t(tid.b)) * uint32_t(p.hv) + uint32_t(tid.h)) * DV);
+        for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(o0, out_dt, r, 0.0f);
+        return;
+    }
+    // ... then the slot's side.  The counters and the row blocks go out first and by themselves: the scheduling
+    // barrier behind them keeps the address arithmetic of the other eight fields, and the first use of the fill count,
+    // from being scheduled in among them (the compiler had put half of the row-block loads behind the wait for the
+    // fill count).
+    {
         const uint32_t seq = slot, h = tid.h;
         F.np = *field(p.st.NPTR, seq, p.st.sN, h);
         F.gcur = *field(p.st.GCUR, seq, p.st.sGC, h);
@@ -180,8 +183,10 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
             for (int t = 0; t < Q::NLD; ++t)
                 F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
         __builtin_amdgcn_sched_barrier(0);
-    };
-    auto issue_slot = [&](const GdnAddr<T>& A, int lane, int n32) {
+    }
+    const GdnAddr<T> A = gdn_addr<T>(p, tid, slot);
+    void* const outp = advance(p.out, out_dt, A.obase);
+    {
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
@@ -209,319 +214,299 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         const uint32_t li = uint32_t(lane) < nl ? lane : 0;
         F.gbl = A.GBh[li];
         F.ubs = T::QBUF ? A.buf.UBS[li] : uint16_t(0);
-    };
+    }
+    // every load of the item is in flight from here on: keep the compiler from sinking any of them to its use, and
+    // from scheduling a use (a conversion, with its wait) up among them
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
-    {
-        const int lane = lane0;
-        const int n32 = lane & 31, kb = lane >> 5;
-        // the row of the head this lane finishes after the pass (NB = 2: the wavefront's halves take a block each)
-        const int row = (wh * NB + (NB == 2 ? kb : 0)) * T::MR + n32;
-        const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);    // chunk `lane` of a 1 KB piece in the LDS image
-        issue(cur, lane, n32, row);
-        const TileId tid = tile_of(cur);
-        if (idx && cur.slot <= 0) {                      // padding row: zero output, touch nothing else
-            void* const o0 = advance(p.out, out_dt, (uint64_t(uint32_t(tid.b)) * uint32_t(p.hv) + uint32_t(tid.h)) * DV);
-            for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(o0, out_dt, r, 0.0f);
-            return;
+    // ---- shared roles (their inputs were issued first) ----
+    auto role_vector = [&](const uint32_t (&raw)[NE], int dt, float post, int v) {
+        float xe[NE], ss = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NE; ++t) {
+            xe[t] = vec_elem<NE>(raw, dt, t);
+            ss = __builtin_fmaf(xe[t], xe[t], ss);
         }
-        issue_codes(tid, cur.slot, lane);
-        const GdnAddr<T> A = gdn_addr<T>(p, tid, cur.slot);
-        void* const outp = advance(p.out, out_dt, A.obase);
-        issue_slot(A, lane, n32);
-        // every load of the item is in flight from here on: keep the compiler from sinking any of them to its use,
-        // and from scheduling a use (a conversion, with its wait) up among them
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        {
-        // ---- shared roles (their inputs were issued first) ----
-        auto role_vector = [&](const uint32_t (&raw)[NE], int dt, float post, int v) {
-            float xe[NE], ss = 0.0f;
+        const float nrm = sqrtf(lanes_sum<WAVE>(ss) + 1e-6f);
 #pragma unroll
-            for (int t = 0; t < NE; ++t) {
-                xe[t] = vec_elem<NE>(raw, dt, t);
-                ss = __builtin_fmaf(xe[t], xe[t], ss);
-            }
-            const float nrm = sqrtf(lanes_sum<WAVE>(ss) + 1e-6f);
-#pragma unroll
-            for (int t = 0; t < NE; ++t) xe[t] = xe[t] / nrm * post;
-            if constexpr (NE == 1) lds_xn[v * DK + lane] = xe[0];
-            else if constexpr (NE == 2) *reinterpret_cast<float2*>(lds_xn + v * DK + 2 * lane) = make_float2(xe[0], xe[1]);
-            else *reinterpret_cast<float4*>(lds_xn + v * DK + 4 * lane) = make_float4(xe[0], xe[1], xe[2], xe[3]);
-            quad_stage_planes<T, NE>(xe, v, lane, lds_pl, lds_xs);
-        };
-        if constexpr (RQ == RK) {
-            if (w == RQ) {
-                role_vector(F.xr, q_dt, p.scale, 0);
-                role_vector(F.xr2, k_dt, 1.0f, 1);
-            }
+        for (int t = 0; t < NE; ++t) xe[t] = xe[t] / nrm * post;
+        if constexpr (NE == 1) lds_xn[v * DK + lane] = xe[0];
+        else if constexpr (NE == 2) *reinterpret_cast<float2*>(lds_xn + v * DK + 2 * lane) = make_float2(xe[0], xe[1]);
+        else *reinterpret_cast<float4*>(lds_xn + v * DK + 4 * lane) = make_float4(xe[0], xe[1], xe[2], xe[3]);
+        quad_stage_planes<T, NE>(xe, v, lane, lds_pl, lds_xs);
+    };
+    if constexpr (RQ == RK) {
+        if (w == RQ) {
+            role_vector(F.xr, q_dt, p.scale, 0);
+            role_vector(F.xr2, k_dt, 1.0f, 1);
+        }
+    } else {
+        if (w == RQ) role_vector(F.xr, q_dt, p.scale, 0);
+        if (w == RK) role_vector(F.xr, k_dt, 1.0f, 1);
+    }
+    if (wh == 0) {                                   // this head's gates and decays
+        float g, beta;
+        if (gate) {
+            const float x = raw_to_f(F.g0, a_dt) + raw_to_f(F.g3, dt_bias_dt);
+            const float sp = x <= 20.0f ? logf(1.0f + expf(x)) : x;
+            g = -expf(raw_to_f(F.g2, A_log_dt)) * sp;
+            beta = 1.0f / (1.0f + expf(-raw_to_f(F.g1, bt_dt)));
         } else {
-            if (w == RQ) role_vector(F.xr, q_dt, p.scale, 0);
-            if (w == RK) role_vector(F.xr, k_dt, 1.0f, 1);
+            g = raw_to_f(F.g0, a_dt);
+            beta = raw_to_f(F.g1, bt_dt);
         }
-        if (wh == 0) {                                   // this head's gates and decays
-            float g, beta;
-            if (gate) {
-                const float x = raw_to_f(F.g0, a_dt) + raw_to_f(F.g3, dt_bias_dt);
-                const float sp = x <= 20.0f ? logf(1.0f + expf(x)) : x;
-                g = -expf(raw_to_f(F.g2, A_log_dt)) * sp;
-                beta = 1.0f / (1.0f + expf(-raw_to_f(F.g1, bt_dt)));
-            } else {
-                g = raw_to_f(F.g0, a_dt);
-                beta = raw_to_f(F.g1, bt_dt);
-            }
-            if (lane == 0) {
-                lds_scal[0] = beta;
-                lds_scal[1] = expf(F.gcur);
-                lds_scal[2] = expf(g);
-                lds_scal[3] = F.gcur + g;
-            }
+        if (lane == 0) {
+            lds_scal[0] = beta;
+            lds_scal[1] = expf(F.gcur);
+            lds_scal[2] = expf(g);
+            lds_scal[3] = F.gcur + g;
         }
-        // ---- the loads land: LDS images of the row blocks, scales, raw buffer pieces ----
-        const int n = F.np & (m - 1);
-        const float gcur = F.gcur;
-        const uint32_t vr = F.vr;
-        uint16_t scw[NB][NG];
+    }
+    // ---- the loads land: LDS images of the row blocks, scales, raw buffer pieces ----
+    const int n = F.np & (m - 1);
+    const float gcur = F.gcur;
+    const uint32_t vr = F.vr;
+    uint16_t scw[NB][NG];
 #pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
+    for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                scw[bi][g] = F.sc[bi][g];
-                if (kb == 0) lds_sc[((wh * NB + bi) * T::MR + n32) * NG + g] = F.sc[bi][g];
-            }
+        for (int g = 0; g < NG; ++g) {
+            scw[bi][g] = F.sc[bi][g];
+            if (kb == 0) lds_sc[((wh * NB + bi) * T::MR + n32) * NG + g] = F.sc[bi][g];
+        }
 #pragma unroll
-        for (int t = 0; t < Q::UT; ++t) {
-            const int i = lane / Q::LU + Q::SU * t;
-            if (i < m) store_raw4<T::QBUF>(lds_ubr + (i * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE, F.uraw[t]);
+    for (int t = 0; t < Q::UT; ++t) {
+        const int i = lane / Q::LU + Q::SU * t;
+        if (i < m) store_raw4<T::QBUF>(lds_ubr + (i * DV + wh * Q::RW + 4 * (lane % Q::LU)) * T::BE, F.uraw[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < Q::KT; ++t) {
+        const int i = Q::SPP * (NW * t + w) + lane / Q::LPS;
+        if (i < m) {
+            store_raw4<T::QBUF>(lds_kbr + (i * DK + 4 * (lane % Q::LPS)) * T::BE, F.kraw[t]);
+            if (T::QBUF && lane % Q::LPS == 0) lds_kbsf[i] = f16_to_f32(F.kbs[t]);
+        }
+    }
+    if (wh == 0 && lane < m) {
+        lds_gbf[lane] = F.gbl;
+        if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
+    }
+#pragma unroll
+    for (int bi = 0; bi < NB; ++bi)
+#pragma unroll
+        for (int t = 0; t < Q::NLD; ++t)
+            *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+    const bool full = n == m - 1;
+    lds_barrier();
+
+    // ---- every wavefront: state pass over its row blocks ----
+    float sq, sk;                                    // (S0 q)[row], (S0 k)[row], scales applied
+    {
+        v4i aop[T::NKS];
+        quad_fetch_planes<T, 2>(lds_pl, lane, aop);
+        float xs[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) xs[g] = lds_xs[kb * NG + g];
+        float own[NB];
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi) {
+            float sc[NG];
+#pragma unroll
+            for (int g = 0; g < NG; ++g) sc[g] = f16_to_f32(scw[bi][g]);
+            own[bi] = quad_block_pass<Q, T>(my_codes + bi * Q::BLK, aop, xs, sc, lane);
+        }
+        if constexpr (NB == 2) {                     // lane (n, kb) takes over row n of block kb: both sums
+            const auto r = __builtin_amdgcn_permlane32_swap(as_u32(own[0]), as_u32(own[1]), false, false);
+            sq = as_f32(r[0]);
+            sk = as_f32(r[1]);
+        } else {
+            const Pair qk = pair32(own[0]);
+            sq = qk.lo;
+            sk = qk.hi;
+        }
+    }
+    // ---- K_i . q, K_i . k of this wavefront's share of the slots ----
+    {
+        float x[2][4];
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const float4 f = *reinterpret_cast<const float4*>(lds_xn + v * DK + 4 * (lane % Q::LPS));
+            x[v][0] = f.x; x[v][1] = f.y; x[v][2] = f.z; x[v][3] = f.w;
         }
 #pragma unroll
         for (int t = 0; t < Q::KT; ++t) {
             const int i = Q::SPP * (NW * t + w) + lane / Q::LPS;
-            if (i < m) {
-                store_raw4<T::QBUF>(lds_kbr + (i * DK + 4 * (lane % Q::LPS)) * T::BE, F.kraw[t]);
-                if (T::QBUF && lane % Q::LPS == 0) lds_kbsf[i] = f16_to_f32(F.kbs[t]);
+            const int ic = i < m ? i : m - 1;
+            float kf[4];
+            decode_raw4<T::QBUF>(load_raw4<T::QBUF>(lds_kbr + (ic * DK + 4 * (lane % Q::LPS)) * T::BE), kf);
+            if constexpr (T::QBUF) {
+                const float s = lds_kbsf[ic];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) kf[c] = kf[c] * s;
             }
-        }
-        if (wh == 0 && lane < m) {
-            lds_gbf[lane] = F.gbl;
-            if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
-        }
-#pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
-#pragma unroll
-            for (int t = 0; t < Q::NLD; ++t)
-                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
-        const bool full = n == m - 1;
-        lds_barrier();
-
-        // ---- every wavefront: state pass over its row blocks ----
-        float sq, sk;                                    // (S0 q)[row], (S0 k)[row], scales applied
-        {
-            v4i aop[T::NKS];
-            quad_fetch_planes<T, 2>(lds_pl, lane, aop);
-            float xs[NG];
-#pragma unroll
-            for (int g = 0; g < NG; ++g) xs[g] = lds_xs[kb * NG + g];
-            float own[NB];
-#pragma unroll
-            for (int bi = 0; bi < NB; ++bi) {
-                float sc[NG];
-#pragma unroll
-                for (int g = 0; g < NG; ++g) sc[g] = f16_to_f32(scw[bi][g]);
-                own[bi] = quad_block_pass<Q, T>(my_codes + bi * Q::BLK, aop, xs, sc, lane);
-            }
-            if constexpr (NB == 2) {                     // lane (n, kb) takes over row n of block kb: both sums
-                const auto r = __builtin_amdgcn_permlane32_swap(as_u32(own[0]), as_u32(own[1]), false, false);
-                sq = as_f32(r[0]);
-                sk = as_f32(r[1]);
-            } else {
-                const Pair qk = pair32(own[0]);
-                sq = qk.lo;
-                sk = qk.hi;
-            }
-        }
-        // ---- K_i . q, K_i . k of this wavefront's share of the slots ----
-        {
-            float x[2][4];
 #pragma unroll
             for (int v = 0; v < 2; ++v) {
-                const float4 f = *reinterpret_cast<const float4*>(lds_xn + v * DK + 4 * (lane % Q::LPS));
-                x[v][0] = f.x; x[v][1] = f.y; x[v][2] = f.z; x[v][3] = f.w;
-            }
+                float pr = kf[0] * x[v][0];
 #pragma unroll
-            for (int t = 0; t < Q::KT; ++t) {
-                const int i = Q::SPP * (NW * t + w) + lane / Q::LPS;
-                const int ic = i < m ? i : m - 1;
-                float kf[4];
-                decode_raw4<T::QBUF>(load_raw4<T::QBUF>(lds_kbr + (ic * DK + 4 * (lane % Q::LPS)) * T::BE), kf);
-                if constexpr (T::QBUF) {
-                    const float s = lds_kbsf[ic];
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) kf[c] = kf[c] * s;
-                }
-#pragma unroll
-                for (int v = 0; v < 2; ++v) {
-                    float pr = kf[0] * x[v][0];
-#pragma unroll
-                    for (int c = 1; c < 4; ++c) pr = __builtin_fmaf(kf[c], x[v][c], pr);
-                    pr = lanes_sum<Q::LPS>(pr);
-                    if (lane % Q::LPS == 0 && i < MM) lds_dots[v * MM + i] = pr;
-                }
+                for (int c = 1; c < 4; ++c) pr = __builtin_fmaf(kf[c], x[v][c], pr);
+                pr = lanes_sum<Q::LPS>(pr);
+                if (lane % Q::LPS == 0 && i < MM) lds_dots[v * MM + i] = pr;
             }
         }
-        // ---- k . q ----
-        if (w == RK) {
-            float kqp = 0.0f;
+    }
+    // ---- k . q ----
+    if (w == RK) {
+        float kqp = 0.0f;
 #pragma unroll
-            for (int t = 0; t < NE; ++t) kqp = __builtin_fmaf(lds_xn[DK + NE * lane + t], lds_xn[NE * lane + t], kqp);
-            kqp = lanes_sum<WAVE>(kqp);
-            if (lane == 0) lds_gsc[0] = kqp;
-        }
-        lds_barrier();                                   // the raw keys of slot n may be overwritten from here on
+        for (int t = 0; t < NE; ++t) kqp = __builtin_fmaf(lds_xn[DK + NE * lane + t], lds_xn[NE * lane + t], kqp);
+        kqp = lanes_sum<WAVE>(kqp);
+        if (lane == 0) lds_gsc[0] = kqp;
+    }
+    lds_barrier();                                   // the raw keys of slot n may be overwritten from here on
 
-        // ---- the buffered key of this token: the rounded k, for this workgroup's folds and (first head group of
-        //      the key head only) for the slot ----
-        if (w == RX) {
-            float kxe[NE], kmax = 0.0f;
+    // ---- the buffered key of this token: the rounded k, for this workgroup's folds and (first head group of
+    //      the key head only) for the slot ----
+    if (w == RX) {
+        float kxe[NE], kmax = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NE; ++t) {
+            kxe[t] = lds_xn[DK + NE * lane + t];
+            kmax = fmaxf(kmax, fabsf(kxe[t]));
+        }
+        float ks = 1.0f;
+        if constexpr (T::QBUF) ks = fp16_scale(lanes_max<WAVE>(kmax), 127.0f);
+        const bool write = tid.h - hl == tid.hk * p.gqa;
+        if (T::QBUF && lane == 0) {
+            lds_kbsf[n] = ks;
+            if (write) A.buf.KBS[n] = f32_to_f16(ks);
+        }
+        if constexpr (T::QBUF) {
+            uint32_t pk = 0;
+#pragma unroll
+            for (int t = 0; t < NE; ++t) pk |= (uint32_t(int(round_buf(kxe[t], ks))) & 0xFFu) << (8 * t);
+            uint8_t* dl = lds_kbr + n * DK + NE * lane;
+            uint8_t* dg = A.buf.KB + n * DK + NE * lane;
+            if constexpr (NE == 1) { *dl = uint8_t(pk); if (write) *dg = uint8_t(pk); }
+            else if constexpr (NE == 2) {
+                *reinterpret_cast<uint16_t*>(dl) = uint16_t(pk);
+                if (write) *reinterpret_cast<uint16_t*>(dg) = uint16_t(pk);
+            } else {
+                *reinterpret_cast<uint32_t*>(dl) = pk;
+                if (write) *reinterpret_cast<uint32_t*>(dg) = pk;
+            }
+        } else {
 #pragma unroll
             for (int t = 0; t < NE; ++t) {
-                kxe[t] = lds_xn[DK + NE * lane + t];
-                kmax = fmaxf(kmax, fabsf(kxe[t]));
-            }
-            float ks = 1.0f;
-            if constexpr (T::QBUF) ks = fp16_scale(lanes_max<WAVE>(kmax), 127.0f);
-            const bool write = tid.h - hl == tid.hk * p.gqa;
-            if (T::QBUF && lane == 0) {
-                lds_kbsf[n] = ks;
-                if (write) A.buf.KBS[n] = f32_to_f16(ks);
-            }
-            if constexpr (T::QBUF) {
-                uint32_t pk = 0;
-#pragma unroll
-                for (int t = 0; t < NE; ++t) pk |= (uint32_t(int(round_buf(kxe[t], ks))) & 0xFFu) << (8 * t);
-                uint8_t* dl = lds_kbr + n * DK + NE * lane;
-                uint8_t* dg = A.buf.KB + n * DK + NE * lane;
-                if constexpr (NE == 1) { *dl = uint8_t(pk); if (write) *dg = uint8_t(pk); }
-                else if constexpr (NE == 2) {
-                    *reinterpret_cast<uint16_t*>(dl) = uint16_t(pk);
-                    if (write) *reinterpret_cast<uint16_t*>(dg) = uint16_t(pk);
-                } else {
-                    *reinterpret_cast<uint32_t*>(dl) = pk;
-                    if (write) *reinterpret_cast<uint32_t*>(dg) = pk;
-                }
-            } else {
-#pragma unroll
-                for (int t = 0; t < NE; ++t) {
-                    const uint16_t hb = f32_to_bf16(kxe[t]);
-                    reinterpret_cast<uint16_t*>(lds_kbr)[n * DK + NE * lane + t] = hb;
-                    if (write) reinterpret_cast<uint16_t*>(A.buf.KB)[n * DK + NE * lane + t] = hb;
-                }
+                const uint16_t hb = f32_to_bf16(kxe[t]);
+                reinterpret_cast<uint16_t*>(lds_kbr)[n * DK + NE * lane + t] = hb;
+                if (write) reinterpret_cast<uint16_t*>(A.buf.KB)[n * DK + NE * lane + t] = hb;
             }
         }
+    }
 
-        // ---- this wavefront's rows: buffer term, u, o ----
-        const float beta = lds_scal[0], alpha = lds_scal[1], a = lds_scal[2], gnew = lds_scal[3];
-        const float kq = lds_gsc[0];
-        // coefficients of the head's slots, lane i: c_x[i] = exp(gcur - G_i) (K_i . x), times the slot's value scale;
-        // dead slots (i >= n) may hold anything: select, never multiply
-        const int li = lane < m ? lane : 0;
-        float cq, ck;
-        {
-            const float dec = expf(gcur - lds_gbf[li]);
-            const float dq = lds_dots[li], dk_ = lds_dots[MM + li];
-            const float us_i = T::QBUF ? lds_ubsf[li] : 1.0f;
-            const bool alive = lane < n;
-            cq = alive ? (T::QBUF ? (dec * dq) * us_i : dec * dq) : 0.0f;
-            ck = alive ? (T::QBUF ? (dec * dk_) * us_i : dec * dk_) : 0.0f;
-        }
-        // every slot's value is fetched up front (one wait for all of them), dead slots then add c = 0 times a finite
-        // int8 value, or are skipped (bf16 values of a dead slot may be NaNs)
-        float uv[MM];
+    // ---- this wavefront's rows: buffer term, u, o ----
+    const float beta = lds_scal[0], alpha = lds_scal[1], a = lds_scal[2], gnew = lds_scal[3];
+    const float kq = lds_gsc[0];
+    // coefficients of the head's slots, lane i: c_x[i] = exp(gcur - G_i) (K_i . x), times the slot's value scale;
+    // dead slots (i >= n) may hold anything: select, never multiply
+    const int li = lane < m ? lane : 0;
+    float cq, ck;
+    {
+        const float dec = expf(gcur - lds_gbf[li]);
+        const float dq = lds_dots[li], dk_ = lds_dots[MM + li];
+        const float us_i = T::QBUF ? lds_ubsf[li] : 1.0f;
+        const bool alive = lane < n;
+        cq = alive ? (T::QBUF ? (dec * dq) * us_i : dec * dq) : 0.0f;
+        ck = alive ? (T::QBUF ? (dec * dk_) * us_i : dec * dk_) : 0.0f;
+    }
+    // every slot's value is fetched up front (one wait for all of them), dead slots then add c = 0 times a finite
+    // int8 value, or are skipped (bf16 values of a dead slot may be NaNs)
+    float uv[MM];
 #pragma unroll
-        for (int i = 0; i < MM; ++i) uv[i] = lds_raw<T::QBUF>(lds_ubr, (i < m ? i : 0) * DV + row);
-        float accq = alpha * sq, acck = alpha * sk;
+    for (int i = 0; i < MM; ++i) uv[i] = lds_raw<T::QBUF>(lds_ubr, (i < m ? i : 0) * DV + row);
+    float accq = alpha * sq, acck = alpha * sk;
 #pragma unroll
-        for (int i = 0; i < MM; ++i) {
-            const float u_i = T::QBUF ? uv[i] : (i < n ? uv[i] : 0.0f);
-            accq = __builtin_fmaf(u_i, lane_bcast(cq, i), accq);
-            acck = __builtin_fmaf(u_i, lane_bcast(ck, i), acck);
-        }
-        const float vt = raw_to_f(vr, v_dt);
-        const float u = beta * __builtin_fmaf(-a, acck, vt);
-        const float o = __builtin_fmaf(kq, u, a * accq);
-        if (NB == 2 || kb == 0) store_f(outp, out_dt, row, o);
+    for (int i = 0; i < MM; ++i) {
+        const float u_i = T::QBUF ? uv[i] : (i < n ? uv[i] : 0.0f);
+        accq = __builtin_fmaf(u_i, lane_bcast(cq, i), accq);
+        acck = __builtin_fmaf(u_i, lane_bcast(ck, i), acck);
+    }
+    const float vt = raw_to_f(vr, v_dt);
+    const float u = beta * __builtin_fmaf(-a, acck, vt);
+    const float o = __builtin_fmaf(kq, u, a * accq);
+    if (NB == 2 || kb == 0) store_f(outp, out_dt, row, o);
 
-        // ---- append ----
-        float us = 1.0f;
+    // ---- append ----
+    float us = 1.0f;
+    if constexpr (T::QBUF) {
+        float amax = lanes_max<WAVE>(fabsf(u));
+        if constexpr (NWH > 1) {
+            if (lane == 0) lds_red[w] = amax;
+            lds_barrier();
+#pragma unroll
+            for (int ww = 0; ww < NWH; ++ww) amax = fmaxf(amax, lds_red[hl * NWH + ww]);
+        }
+        us = fp16_scale(amax, 127.0f);
+        if (wh == 0 && lane == 0) { A.buf.UBS[n] = f32_to_f16(us); lds_ubsf[n] = us; }
+    }
+    if (NB == 2 || kb == 0) {
         if constexpr (T::QBUF) {
-            float amax = lanes_max<WAVE>(fabsf(u));
-            if constexpr (NWH > 1) {
-                if (lane == 0) lds_red[w] = amax;
-                lds_barrier();
-#pragma unroll
-                for (int ww = 0; ww < NWH; ++ww) amax = fmaxf(amax, lds_red[hl * NWH + ww]);
-            }
-            us = fp16_scale(amax, 127.0f);
-            if (wh == 0 && lane == 0) { A.buf.UBS[n] = f32_to_f16(us); lds_ubsf[n] = us; }
+            const int8_t c = int8_t(int(round_buf(u, us)));
+            reinterpret_cast<int8_t*>(A.buf.UB)[n * DV + row] = c;
+            reinterpret_cast<int8_t*>(lds_ubr)[n * DV + row] = c;
+        } else {
+            const uint16_t hb = f32_to_bf16(u);
+            reinterpret_cast<uint16_t*>(A.buf.UB)[n * DV + row] = hb;
+            reinterpret_cast<uint16_t*>(lds_ubr)[n * DV + row] = hb;
         }
-        if (NB == 2 || kb == 0) {
-            if constexpr (T::QBUF) {
-                const int8_t c = int8_t(int(round_buf(u, us)));
-                reinterpret_cast<int8_t*>(A.buf.UB)[n * DV + row] = c;
-                reinterpret_cast<int8_t*>(lds_ubr)[n * DV + row] = c;
-            } else {
-                const uint16_t hb = f32_to_bf16(u);
-                reinterpret_cast<uint16_t*>(A.buf.UB)[n * DV + row] = hb;
-                reinterpret_cast<uint16_t*>(lds_ubr)[n * DV + row] = hb;
-            }
-        }
-        if (wh == 0 && lane == 0) {
-            A.GBh[n] = gnew;
-            *A.gcp = full ? 0.0f : gnew;                 // advance
-            *A.np = full ? 0 : n + 1;
-        }
+    }
+    if (wh == 0 && lane == 0) {
+        A.GBh[n] = gnew;
+        *A.gcp = full ? 0.0f : gnew;                 // advance
+        *A.np = full ? 0 : n + 1;
+    }
 
-        // ---- fold ----
-        if (full) {
-            lds_barrier();                               // `full` is the same in every head of a slot
-            constexpr int MT4 = (MM + 3) / 4, CL = DK / 4;
-            const int fn = lane & 15, fq = lane >> 4;
-            // decay ratios a_m / a_i of the lane's slots 4 t + q (this token: 1)
-            float decf[MT4];
+    // ---- fold ----
+    if (full) {
+        lds_barrier();                               // `full` is the same in every head of a slot
+        constexpr int MT4 = (MM + 3) / 4, CL = DK / 4;
+        const int fn = lane & 15, fq = lane >> 4;
+        // decay ratios a_m / a_i of the lane's slots 4 t + q (this token: 1)
+        float decf[MT4];
 #pragma unroll
-            for (int t = 0; t < MT4; ++t) {
-                const int sl = 4 * t + fq;
-                decf[t] = sl < m - 1 ? expf(gnew - lds_gbf[sl < m - 1 ? sl : 0]) : 1.0f;
-            }
-            const float cmul = expf(gnew);
-            const int fg = (fq * CL) / T::KGROUP;
-            float kop[DK / 16][MT4];
-            quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lane, kop);
-#pragma unroll
-            for (int bi = 0; bi < NB; ++bi) {
-                uint8_t* blk = my_codes + bi * Q::BLK;
-#pragma unroll
-                for (int hf = 0; hf < 2; ++hf) {
-                    const int frow = (wh * NB + bi) * T::MR + 16 * hf + fn;
-                    float bop[MT4];
-#pragma unroll
-                    for (int t = 0; t < MT4; ++t) {
-                        const int sl = 4 * t + fq;
-                        const int sc_ = sl < m ? sl : 0;
-                        float uv = lds_raw<T::QBUF>(lds_ubr, sc_ * DV + frow);
-                        if constexpr (T::QBUF) uv = uv * lds_ubsf[sc_];
-                        uv = decf[t] * uv;
-                        bop[t] = sl < m ? uv : 0.0f;
-                    }
-                    quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
-                                                A.SCh + frow * NG + fg, lane);
-                }
-                wave_sync();
-#pragma unroll
-                for (int t = 0; t < Q::NLD; ++t)
-                    stream_store(reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16),
-                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
-            }
+        for (int t = 0; t < MT4; ++t) {
+            const int sl = 4 * t + fq;
+            decf[t] = sl < m - 1 ? expf(gnew - lds_gbf[sl < m - 1 ? sl : 0]) : 1.0f;
         }
+        const float cmul = expf(gnew);
+        const int fg = (fq * CL) / T::KGROUP;
+        float kop[DK / 16][MT4];
+        quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lane, kop);
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi) {
+            uint8_t* blk = my_codes + bi * Q::BLK;
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const int frow = (wh * NB + bi) * T::MR + 16 * hf + fn;
+                float bop[MT4];
+#pragma unroll
+                for (int t = 0; t < MT4; ++t) {
+                    const int sl = 4 * t + fq;
+                    const int sc_ = sl < m ? sl : 0;
+                    float uv = lds_raw<T::QBUF>(lds_ubr, sc_ * DV + frow);
+                    if constexpr (T::QBUF) uv = uv * lds_ubsf[sc_];
+                    uv = decf[t] * uv;
+                    bop[t] = sl < m ? uv : 0.0f;
+                }
+                quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
+                                            A.SCh + frow * NG + fg, lane);
+            }
+            wave_sync();
+#pragma unroll
+            for (int t = 0; t < Q::NLD; ++t)
+                stream_store(reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16),
+                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
         }
     }
 }
