@@ -35,6 +35,9 @@ SHADER_SETS = {
               'SQ_INSTS_SMEM', 'SQ_INSTS_MFMA'],
     'time': ['SQ_WAVE_CYCLES', 'SQ_BUSY_CYCLES', 'SQ_WAIT_ANY', 'SQ_WAIT_INST_ANY', 'SQ_ACTIVE_INST_VALU',
              'SQ_ACTIVE_INST_SCA', 'SQ_ACTIVE_INST_LDS', 'SQ_LDS_BANK_CONFLICT', 'GRBM_GUI_ACTIVE'],
+    # instruction fetch: requests of the wavefronts, and the instruction caches' (one per two compute units) side
+    'ifetch': ['SQ_IFETCH', 'SQC_ICACHE_REQ', 'SQC_ICACHE_HITS', 'SQC_ICACHE_MISSES', 'SQC_ICACHE_BUSY_CYCLES',
+               'SQ_BUSY_CYCLES', 'GRBM_GUI_ACTIVE'],
 }
 
 

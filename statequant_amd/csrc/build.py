@@ -1,6 +1,6 @@
 """Build libsqhip.so (the C-ABI library of include/statequant_hip.h) for gfx950 with hipcc.
 
-    python -m statequant_amd.csrc.build [-j N] [--force]
+    python -m statequant_amd.csrc.build [-j N] [--force] [--timeline]
 
 The step kernels are templates on (bits, d_k, d_v, group, int8-buffer, max m).  ``CASES`` below lists the instances
 that are compiled; this script writes one small translation unit per chunk of instances plus the dispatch table into
@@ -378,10 +378,18 @@ if __name__ == '__main__':
     ap = argparse.ArgumentParser()
     ap.add_argument('-j', type=int, default=None)
     ap.add_argument('--force', action='store_true')
+    ap.add_argument('--timeline', action='store_true',
+                    help='build libsqhip_timeline.so instead: the same library with the workgroup-per-key-head Gated '
+                         'DeltaNet kernel instrumented (-DSQ_TIMELINE, see sq_gdn_quad.cuh); profile_timeline.py '
+                         'loads it.  Objects go to csrc/build_timeline/')
     ap.add_argument('--resources', metavar='PATTERN', nargs='?', const='', default=None,
                     help="instead of building, print the compiler's resource usage (registers, spills, LDS, "
                          'occupancy) of every kernel whose name contains PATTERN')
     a = ap.parse_args()
+    if a.timeline:
+        OUT = os.path.join(HERE, 'build_timeline')
+        LIB = os.path.join(PKG, 'libsqhip_timeline.so')
+        HIPCC_FLAGS = HIPCC_FLAGS + ['-DSQ_TIMELINE']
     if a.resources is not None:
         resources(a.resources, a.j)
         sys.exit(0)

@@ -67,6 +67,28 @@ struct GdnLoads {
     uint32_t xr[Q::NE], xr2[Q::NE], g0, g1, g2, g3, vr;
 };
 
+// Optional instrumentation, compiled in with -DSQ_TIMELINE only (build.py --timeline writes a library of its own):
+// every wavefront records the 100 MHz real-time counter at fixed points of its life, 16 x 8 bytes per wavefront,
+// workgroup-major, into the buffer whose device address the environment variable SQ_TIMELINE_BUF holds (decimal) at
+// the time of the launch; a launch can then be laid out as a timeline of its workgroups (profile_timeline.py).  A
+// mark waits for the scalar loads in flight, so the marks cost a wavefront about a microsecond altogether.  Without
+// the define they compile to nothing.
+#ifdef SQ_TIMELINE
+#include <stdlib.h>
+#define SQ_TL_PARAM uint64_t* tl,
+#define SQ_MARK(k)                                                                                                 \
+    do {                                                                                                           \
+        if (tl) {                                                                                                  \
+            uint64_t t_;                                                                                           \
+            asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_)::"memory");                         \
+            if ((threadIdx.x & 63) == 0) tl[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + (k)] = t_; \
+        }                                                                                                          \
+    } while (0)
+#else
+#define SQ_TL_PARAM
+#define SQ_MARK(k) do { } while (0)
+#endif
+
 // SPEC > 0 compiles the serving cases in, so that dtypes and options cost no scalar branches on the way to the first
 // load (measured on the 128 x 128 int8 step: 35.4 -> 34.2 us per launch): bf16 q / k / v / out, no dispatch order,
 // head counts that are powers of two, and  1: g and beta given as fp32;  2: the gate formed in the kernel from bf16
@@ -74,7 +96,8 @@ struct GdnLoads {
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
 void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd, int hv, int hv_shift,
-                     const GdnParams p) {
+                     SQ_TL_PARAM const GdnParams p) {
+    SQ_MARK(0);                                                   // entry
     // the leading arguments (copies of fields of `p`) are what the slot index load needs: as separate scalar
     // arguments they are preloaded into registers at wave launch, so that load goes out first thing
     constexpr bool FIX = SPEC > 0;
@@ -127,6 +150,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
             }
             tid.b = order[pos];
         }
+        SQ_MARK(1);                                               // item known (the leading arguments are here)
         slot = idx ? idx[tid.b] : tid.b;
         tid.hk = (FIX || p.gqa_shift >= 0) ? tid.h >> p.gqa_shift : tid.h / p.gqa;
     }
@@ -168,6 +192,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(o0, out_dt, r, 0.0f);
         return;
     }
+    SQ_MARK(2);                                                   // slot known, the token's loads issued
     // ... then the slot's side.  The counters and the row blocks go out first and by themselves: the scheduling
     // barrier behind them keeps the address arithmetic of the other eight fields, and the first use of the fill count,
     // from being scheduled in among them (the compiler had put half of the row-block loads behind the wait for the
@@ -177,6 +202,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         F.np = *field(p.st.NPTR, seq, p.st.sN, h);
         F.gcur = *field(p.st.GCUR, seq, p.st.sGC, h);
         const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
+        SQ_MARK(3);                                               // counters issued
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
@@ -184,6 +210,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
                 F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
         __builtin_amdgcn_sched_barrier(0);
     }
+    SQ_MARK(4);                                                   // row blocks issued
     const GdnAddr<T> A = gdn_addr<T>(p, tid, slot);
     void* const outp = advance(p.out, out_dt, A.obase);
     {
@@ -219,6 +246,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
     // from scheduling a use (a conversion, with its wait) up among them
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+    SQ_MARK(5);                                                   // fill count here, buffer loads issued
 
     // ---- shared roles (their inputs were issued first) ----
     auto role_vector = [&](const uint32_t (&raw)[NE], int dt, float post, int v) {
@@ -298,7 +326,9 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         for (int t = 0; t < Q::NLD; ++t)
             *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
     const bool full = n == m - 1;
+    SQ_MARK(6);                                                   // roles done, every load landed in LDS
     lds_barrier();
+    SQ_MARK(7);                                                   // first barrier passed
 
     // ---- every wavefront: state pass over its row blocks ----
     float sq, sk;                                    // (S0 q)[row], (S0 k)[row], scales applied
@@ -326,6 +356,10 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
             sk = qk.hi;
         }
     }
+#ifdef SQ_TIMELINE
+    asm volatile("" ::"v"(sq), "v"(sk));                          // the sums are here before the mark is taken
+#endif
+    SQ_MARK(8);                                                   // state pass done
     // ---- K_i . q, K_i . k of this wavefront's share of the slots ----
     {
         float x[2][4];
@@ -363,7 +397,9 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         kqp = lanes_sum<WAVE>(kqp);
         if (lane == 0) lds_gsc[0] = kqp;
     }
+    SQ_MARK(9);                                                   // buffer dot products done
     lds_barrier();                                   // the raw keys of slot n may be overwritten from here on
+    SQ_MARK(10);                                                  // second barrier passed
 
     // ---- the buffered key of this token: the rounded k, for this workgroup's folds and (first head group of
     //      the key head only) for the slot ----
@@ -436,6 +472,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
     const float u = beta * __builtin_fmaf(-a, acck, vt);
     const float o = __builtin_fmaf(kq, u, a * accq);
     if (NB == 2 || kb == 0) store_f(outp, out_dt, row, o);
+    SQ_MARK(11);                                                  // output stored
 
     // ---- append ----
     float us = 1.0f;
@@ -447,6 +484,10 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
 #pragma unroll
             for (int ww = 0; ww < NWH; ++ww) amax = fmaxf(amax, lds_red[hl * NWH + ww]);
         }
+#ifdef SQ_TIMELINE
+        asm volatile("" ::"v"(amax));
+#endif
+        SQ_MARK(12);                                              // largest |u| of the head known (a barrier)
         us = fp16_scale(amax, 127.0f);
         if (wh == 0 && lane == 0) { A.buf.UBS[n] = f32_to_f16(us); lds_ubsf[n] = us; }
     }
@@ -467,6 +508,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         *A.np = full ? 0 : n + 1;
     }
 
+    SQ_MARK(13);                                                  // appended, counters advanced
     // ---- fold ----
     if (full) {
         lds_barrier();                               // `full` is the same in every head of a slot
@@ -509,6 +551,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
                              *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
         }
     }
+    SQ_MARK(14);                                                  // fold done and stored (if any)
 }
 
 template <class T, int NB, int GH, int WPE, int SPEC>
@@ -516,8 +559,15 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     GdnParams p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     if (p.per_xcd == 0) p.rows_per_xcd = 0;
+#ifdef SQ_TIMELINE
+    const char* tl_env = getenv("SQ_TIMELINE_BUF");
+    uint64_t* tl = tl_env ? reinterpret_cast<uint64_t*>(strtoull(tl_env, nullptr, 10)) : nullptr;
+    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
+                       0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, tl, p);
+#else
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
                        0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
+#endif
     return int(hipGetLastError());
 }
 

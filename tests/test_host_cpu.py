@@ -205,6 +205,24 @@ def test_bench_contract_off_the_gpu():
     assert bench.state_bytes_per_slot(8, 128, 32, 128, 128, 8) * 256 == 153354240
 
 
+def test_timeline_marks_stay_out_of_the_product_library():
+    """The timeline marks of the workgroup-per-key-head kernel exist only behind -DSQ_TIMELINE: the default build
+    never passes the define, `--timeline` builds a library and an object directory of their own, and the profiling
+    script refuses to run without that library or without a GPU instead of falling back to anything."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    from statequant_amd.csrc import build
+    assert '-DSQ_TIMELINE' not in build.HIPCC_FLAGS and build.LIB.endswith('libsqhip.so')
+    src = open(os.path.join(root, 'statequant_amd', 'csrc', 'build.py')).read()
+    assert "libsqhip_timeline.so" in src and "build_timeline" in src
+    kern = open(os.path.join(root, 'statequant_amd', 'csrc', 'sq_gdn_quad.cuh')).read()
+    assert kern.count('#ifdef SQ_TIMELINE') >= 2 and '#define SQ_MARK(k) do { } while (0)' in kern
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(root, 'profile_timeline.py')], capture_output=True, text=True)
+        assert r.returncode != 0 and ('is missing' in r.stderr or 'no GPU visible' in r.stderr), r.stderr
+
+
 def test_gga_packed_tables_match_the_reference(golden):
     """``GGAPacked``: per-layer offset tables, window placement, slot size and bits per value as the reference's class
     computes them for the plan of its own tests (recorded in tests/golden/gga.pt); no GPU, no library call."""
