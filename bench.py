@@ -31,7 +31,9 @@ Secondary figures: ``--workload`` (the other formats and families; ``gga4-pw8`` 
 which re-fits every head at every token), ``--slots N`` (other batch sizes), ``--op write |
 read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots)
 with or without ``--fold-first`` (the step calls' optional dispatch order, folding rows first), ``--calibrate-copy``
-(the known-size copy that the HBM counters are scaled by).
+(the known-size copy that the HBM counters are scaled by), ``--calibrate-stream`` (runs the stand-alone probe
+``statequant_amd/probe_stream``, built by ``python -m statequant_amd.csrc.build --probes``: the rate at which kernels
+that do nothing else read a layer step's codes through the slot index, i.e. the ceiling of this access pattern).
 """
 import argparse
 import json
@@ -376,6 +378,26 @@ def calibrate_copy(dev, nbytes=1 << 30, reps=20):
                       'us_per_copy': round(us, 2), 'gbs_read_plus_write': round(2 * nbytes / us * 1e-3, 1)}))
 
 
+def calibrate_stream():
+    """Run the memory-system probe (csrc/probe_stream.hip) as a child process and print its figures as one JSON line."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'statequant_amd', 'probe_stream')
+    if not os.path.exists(exe):
+        sys.exit(f'bench.py: {exe} is missing; build it with `python -m statequant_amd.csrc.build --probes`')
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    if r.returncode:
+        sys.exit(f'bench.py: {exe} failed:\n{r.stdout}\n{r.stderr}')
+    rows, clock = {}, None
+    for line in r.stdout.splitlines():
+        if 'us per launch' in line:
+            name, rest = line[:34].strip(), line[34:].split()
+            rows[name] = {'us_per_launch': float(rest[0]), 'gbs': float(rest[4])}
+        elif 'shader clock' in line:
+            clock = float(line.split()[-2])
+    print(json.dumps({'calibrate_stream': True, 'codes_bytes_per_launch': 8192 * 16384, 'variants': rows,
+                      'shader_clock_mhz': clock}))
+
+
 def bench_convert(a, lay, views, idx, dev):
     """`SlotLayout.write` (fp32 state -> codes + scales, buffers emptied) or `.read` (stored state advanced across
     the pending buffer -> fp32) over all slots of every layer blob; one launch per layer.  Algorithmic bytes: the fp32
@@ -445,6 +467,9 @@ def main():
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='instead of the workload, run plain device copies of 1 GiB (the known-size kernel that '
                          'rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by) and print their rate')
+    ap.add_argument('--calibrate-stream', action='store_true',
+                    help='instead of the workload, run statequant_amd/probe_stream (read-only kernels over the codes '
+                         'of a layer step: the ceiling of the access pattern) and print its figures')
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit('bench.py: this build measures one GPU; the decode step has no cross-GPU exchange (slots shard '
@@ -455,6 +480,8 @@ def main():
     torch.cuda.set_device(dev)
     if a.calibrate_copy:
         return calibrate_copy(dev)
+    if a.calibrate_stream:
+        return calibrate_stream()
     m = a.m
     if a.slots:
         w = WORKLOADS[a.workload]

@@ -1,6 +1,6 @@
 """Build libsqhip.so (the C-ABI library of include/statequant_hip.h) for gfx950 with hipcc.
 
-    python -m statequant_amd.csrc.build [-j N] [--force] [--timeline]
+    python -m statequant_amd.csrc.build [-j N] [--force] [--timeline] [--probes]
 
 The step kernels are templates on (bits, d_k, d_v, group, int8-buffer, max m).  ``CASES`` below lists the instances
 that are compiled; this script writes one small translation unit per chunk of instances plus the dispatch table into
@@ -337,6 +337,19 @@ def build(jobs=None, force=False, verbose=True):
     return LIB
 
 
+def build_probes(verbose=True):
+    """Compile the stand-alone memory-system probe (probe_stream.hip) next to the library; returns its path."""
+    exe = os.path.join(PKG, 'probe_stream')
+    cmd = ['hipcc', '--offload-arch=' + ARCH, '-O3', '-std=c++17', '-Wno-unused-result',
+           os.path.join(HERE, 'probe_stream.hip'), '-o', exe]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode:
+        raise RuntimeError(f'{" ".join(cmd)}\n{r.stdout}\n{r.stderr}')
+    if verbose:
+        print(f'[build] wrote {exe}')
+    return exe
+
+
 _REMARK = re.compile(r'remark: +(Function Name|VGPRs|AGPRs|SGPRs Spill|VGPRs Spill|ScratchSize \[bytes/lane\]|'
                      r'Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]): +(\S+)')
 
@@ -385,7 +398,17 @@ if __name__ == '__main__':
     ap.add_argument('--resources', metavar='PATTERN', nargs='?', const='', default=None,
                     help="instead of building, print the compiler's resource usage (registers, spills, LDS, "
                          'occupancy) of every kernel whose name contains PATTERN')
+    ap.add_argument('--probes', action='store_true',
+                    help='build statequant_amd/probe_stream instead (probe_stream.hip: how fast the codes of a layer '
+                         'step can be read by kernels that do nothing else; bench.py --calibrate-stream runs it)')
     a = ap.parse_args()
+    if a.probes:
+        try:
+            build_probes()
+        except RuntimeError as e:
+            print(e, file=sys.stderr)
+            sys.exit(1)
+        sys.exit(0)
     if a.timeline:
         OUT = os.path.join(HERE, 'build_timeline')
         LIB = os.path.join(PKG, 'libsqhip_timeline.so')

@@ -563,10 +563,10 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     const char* tl_env = getenv("SQ_TIMELINE_BUF");
     uint64_t* tl = tl_env ? reinterpret_cast<uint64_t*>(strtoull(tl_env, nullptr, 10)) : nullptr;
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, tl, p);
+                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, tl, p);
 #else
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       0, stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
+                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
 #endif
     return int(hipGetLastError());
 }

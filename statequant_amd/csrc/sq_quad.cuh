@@ -21,6 +21,8 @@
 // writes (lanes along a row) and the operand-shaped reads (lanes down a column of chunks) are conflict free without
 // padding.
 #pragma once
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "sq_tile.cuh"
@@ -34,6 +36,14 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Diagnostic switch: SQ_LDS_PAD=<bytes> in the environment adds that much unused dynamic LDS to every launch of the
+// workgroup kernels, so that a compute unit holds fewer workgroups (static + dynamic LDS must stay within 64 KB) --
+// for measuring how the step time depends on the number of resident workgroups.  Read once per process.
+inline int quad_lds_pad() {
+    static const int pad = getenv("SQ_LDS_PAD") ? atoi(getenv("SQ_LDS_PAD")) : 0;
+    return pad > 0 ? pad : 0;
 }
 
 template <class T, int NB_, int GH_ = 1>
