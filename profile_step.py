@@ -35,6 +35,10 @@ SHADER_SETS = {
               'SQ_INSTS_SMEM', 'SQ_INSTS_MFMA'],
     'time': ['SQ_WAVE_CYCLES', 'SQ_BUSY_CYCLES', 'SQ_WAIT_ANY', 'SQ_WAIT_INST_ANY', 'SQ_ACTIVE_INST_VALU',
              'SQ_ACTIVE_INST_SCA', 'SQ_ACTIVE_INST_LDS', 'SQ_LDS_BANK_CONFLICT', 'GRBM_GUI_ACTIVE'],
+    # the vector memory path of a compute unit: texture addresser busy (average over the units), L1 stalled on its
+    # outstanding misses, L1 -> L2 read requests, addresser stalled by the L1
+    'vmem': ['TA_BUSY_avr', 'TCP_PENDING_STALL_CYCLES_sum', 'TCP_TCC_READ_REQ_sum', 'TCP_TOTAL_CACHE_ACCESSES_sum',
+             'TA_ADDR_STALLED_BY_TC_CYCLES_sum', 'GRBM_GUI_ACTIVE'],
     # instruction fetch: requests of the wavefronts, and the instruction caches' (one per two compute units) side
     'ifetch': ['SQ_IFETCH', 'SQC_ICACHE_REQ', 'SQC_ICACHE_HITS', 'SQC_ICACHE_MISSES', 'SQC_ICACHE_BUSY_CYCLES',
                'SQ_BUSY_CYCLES', 'GRBM_GUI_ACTIVE'],
