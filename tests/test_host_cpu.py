@@ -221,6 +221,19 @@ def test_timeline_marks_stay_out_of_the_product_library():
     if not torch.cuda.is_available():
         r = subprocess.run([sys.executable, os.path.join(root, 'profile_timeline.py')], capture_output=True, text=True)
         assert r.returncode != 0 and ('is missing' in r.stderr or 'no GPU visible' in r.stderr), r.stderr
+    # the marked kernel still compiles (device pass of one instance, nothing linked)
+    import shutil
+    import tempfile
+    if shutil.which('hipcc'):
+        with tempfile.TemporaryDirectory() as d:
+            unit = os.path.join(d, 'one.hip')
+            with open(unit, 'w') as f:
+                f.write('#include "%s"\nnamespace sq {\ntemplate int launch_gdn_quad<Tile<8, 128, 128, 128, true, 8>, 2, '
+                        '2, 4, 1>(const GdnParams&, hipStream_t);\n}\n'
+                        % os.path.join(root, 'statequant_amd', 'csrc', 'sq_gdn_quad.cuh'))
+            r = subprocess.run(['hipcc', *build.HIPCC_FLAGS, '-DSQ_TIMELINE', '--cuda-device-only', '-c', unit, '-o',
+                                os.path.join(d, 'one.o')], capture_output=True, text=True)
+            assert r.returncode == 0, r.stderr[-2000:]
 
 
 def test_gga_packed_tables_match_the_reference(golden):
