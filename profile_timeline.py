@@ -95,7 +95,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--workload', default='gdn-int8-g128', choices=sorted(bench.WORKLOADS))
     ap.add_argument('--steps', default='3,7', help='steps of the fold period to mark (the last one, m - 1, folds)')
-    ap.add_argument('--out', default='gpurun_out')
+    ap.add_argument('--out', default='profiles')
     a = ap.parse_args()
     lib = os.path.join(os.path.dirname(_hip.LIB_PATH), 'libsqhip_timeline.so')
     if not os.path.exists(lib):

@@ -513,7 +513,12 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
     if (full) {
         lds_barrier();                               // `full` is the same in every head of a slot
         constexpr int MT4 = (MM + 3) / 4, CL = DK / 4;
-        const int fn = lane & 15, fq = lane >> 4;
+        // what the fold derives from the lane id it derives anew (from a copy the compiler cannot trace back): offsets
+        // formed at the top of the kernel would otherwise be kept in registers all the way to here
+        int lf = lane;
+        asm volatile("" : "+v"(lf));
+        const int fn = lf & 15, fq = lf >> 4;
+        const int swzf = swz<Q>(lf / Q::CPR, lf % Q::CPR);
         // decay ratios a_m / a_i of the lane's slots 4 t + q (this token: 1)
         float decf[MT4];
 #pragma unroll
@@ -524,7 +529,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         const float cmul = expf(gnew);
         const int fg = (fq * CL) / T::KGROUP;
         float kop[DK / 16][MT4];
-        quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lane, kop);
+        quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lf, kop);
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi) {
             uint8_t* blk = my_codes + bi * Q::BLK;
@@ -542,13 +547,13 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
                     bop[t] = sl < m ? uv : 0.0f;
                 }
                 quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
-                                            A.SCh + frow * NG + fg, lane);
+                                            A.SCh + frow * NG + fg, lf);
             }
             wave_sync();
 #pragma unroll
             for (int t = 0; t < Q::NLD; ++t)
-                stream_store(reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16),
-                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
+                stream_store(reinterpret_cast<v4u*>(A.Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lf * 16),
+                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swzf));
         }
     }
     SQ_MARK(14);                                                  // fold done and stored (if any)
