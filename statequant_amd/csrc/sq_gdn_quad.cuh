@@ -529,7 +529,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         const float cmul = expf(gnew);
         const int fg = (fq * CL) / T::KGROUP;
         float kop[DK / 16][MT4];
-        quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lf, kop);
+        quad_fold_keys<T>(lds_kbr, lds_kbsf, m, lf, kop);
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi) {
             uint8_t* blk = my_codes + bi * Q::BLK;
@@ -546,7 +546,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
                     uv = decf[t] * uv;
                     bop[t] = sl < m ? uv : 0.0f;
                 }
-                quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
+                quad_fold_half<Q, T>(blk, hf, kop, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
                                             A.SCh + frow * NG + fg, lf);
             }
             wave_sync();

@@ -398,7 +398,12 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
     if (full) {
         lds_barrier();                                   // `full` is the same in every head of a slot
         constexpr int MT4 = (MM + 3) / 4, CL = DK / 4;
-        const int fn = lane & 15, fq = lane >> 4;
+        // lane offsets derived anew (from a copy of the lane id the compiler cannot trace back), so that the ones
+        // formed at the top of the kernel are not kept in registers all the way to here
+        int lf = lane;
+        asm volatile("" : "+v"(lf));
+        const int fn = lf & 15, fq = lf >> 4;
+        const int swzf = swz<Q>(lf / Q::CPR, lf % Q::CPR);
         float decf[MT4];                                 // decay ratios a_m / a_i of the lane's slots 4 t + q
 #pragma unroll
         for (int t = 0; t < MT4; ++t) {
@@ -408,7 +413,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         const float cmul = expf(gnew);
         const int fg = (fq * CL) / T::KGROUP;
         float kop[DK / 16][MT4];
-        quad_fold_keys<T, false>(lds_kbr, lds_kbsf, nullptr, m, lane, kop);
+        quad_fold_keys<T>(lds_kbr, lds_kbsf, m, lf, kop);
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi) {
             uint8_t* blk = my_codes + bi * Q::BLK;
@@ -425,14 +430,14 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
                     fv = decf[t] * fv;
                     bop[t] = sl < m ? fv : 0.0f;
                 }
-                quad_fold_half<Q, T, false>(blk, hf, kop, nullptr, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
-                                            SCh + frow * NG + fg, lane);
+                quad_fold_half<Q, T>(blk, hf, kop, bop, cmul, f16_to_f32(lds_sc[frow * NG + fg]),
+                                            SCh + frow * NG + fg, lf);
             }
             wave_sync();
 #pragma unroll
             for (int t = 0; t < Q::NLD; ++t)
-                stream_store(reinterpret_cast<v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16),
-                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swz0));
+                stream_store(reinterpret_cast<v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lf * 16),
+                             *reinterpret_cast<const v4u*>(blk + t * 1024 + swzf));
         }
     }
 }

@@ -1,7 +1,6 @@
 // The state tile of one (sequence, value head) shared by the wavefronts of one workgroup: every wavefront owns NB of
 // the tile's 32-row blocks.  Shared by the Gated DeltaNet and Mamba2 workgroup-per-key-head step kernels (int4 / int8
-// codes with key-axis scale groups and a power-of-two row size); the fold also carries the per-column factors a
-// per-channel decay needs (COLVEC).
+// codes with key-axis scale groups and a power-of-two row size).
 //
 // What this buys over one wavefront per tile (sq_tile.cuh, kept for the other formats):
 //   * a tile's life is a quarter as long, so the launch's ramp-up and tail shrink and the dispatcher balances the
@@ -305,15 +304,14 @@ __device__ __forceinline__ float ubyte_fma(uint32_t w, float s, float o) {
 // row needs 32 accumulator registers.
 //   lds_kbr / kbsf   buffered keys, raw, and their scales (slot m - 1: this token's, as stored)
 //   bop[t]           the lane's folded values: slot 4 t + q, row n (decay ratio x stored value)
-//   COLVEC           per-column factors on the old state (KDA) from lds_cv, and per-(slot, column) key factors from
-//                    lds_kd [m][DK]; else the scalar cmul
+//   cmul             the decay of the old state over the buffer
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // The folded keys as the matrix core's first operand, once per wavefront (they are the same for every half block):
 // kop[ct][t] = kx_{4 t + q}[column (n / 4) CL + 4 ct + n % 4] for lane (n, q); 0 for slots >= m.
-template <class T, bool COLVEC>
-__device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const float* lds_kbsf, const float* lds_kd,
-                                               int m, int lane, float (&kop)[T::DK / 16][(T::MMAX + 3) / 4]) {
+template <class T>
+__device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const float* lds_kbsf, int m, int lane,
+                                               float (&kop)[T::DK / 16][(T::MMAX + 3) / 4]) {
     constexpr int MT4 = (T::MMAX + 3) / 4, CL = T::DK / 4, NT = CL / 4;
     const int n = lane & 15, q = lane >> 4;
     const int kcol = (n >> 2) * CL + (n & 3);
@@ -326,16 +324,15 @@ __device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const flo
         for (int ct = 0; ct < NT; ++ct) {
             float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
             if constexpr (T::QBUF) kv = kv * ks;
-            if constexpr (COLVEC) kv = kv * lds_kd[sl * T::DK + kcol + 4 * ct];
             kop[ct][t] = slot < m ? kv : 0.0f;
         }
     }
 }
 
-template <class Q, class T, bool COLVEC>
+template <class Q, class T>
 __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float (&kop)[T::DK / 16][(T::MMAX + 3) / 4],
-                                               const float* lds_cv, const float (&bop)[(T::MMAX + 3) / 4], float cmul,
-                                               float s_old, uint16_t* sc_out, int lane) {
+                                               const float (&bop)[(T::MMAX + 3) / 4], float cmul, float s_old,
+                                               uint16_t* sc_out, int lane) {
     constexpr int MT4 = (T::MMAX + 3) / 4;
     constexpr int CL = T::DK / 4;                            // columns per lane
     constexpr int NT = CL / 4;                               // accumulator tiles per lane
@@ -363,7 +360,7 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     }
     // dequantize: (code x scale) x factor, one conversion + one fma per code
     const float s = T::BITS == 8 ? s_old : s_old * 0.0625f;
-    const float sm = COLVEC ? s : s * cmul;
+    const float sm = s * cmul;
     const float off = -128.0f * sm;
     v4f acc[NT];
     // int8 with one scale group per row: the whole half block is folded in units of the row's old scale x decay
@@ -371,7 +368,7 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     // ALU -- they enter the accumulators through the matrix core: each byte, biased to unsigned, becomes the fp16
     // number 1024 + byte by a byte permute (exponent byte 0x64 on top), and one v_mfma_f32_16x16x16_f16 against the
     // 16 x 16 identity hands every lane its own four numbers back as fp32 on top of the constant -1152 (exact).
-    constexpr bool UNITS = T::BITS == 8 && T::NG == 1 && !COLVEC;
+    constexpr bool UNITS = T::BITS == 8 && T::NG == 1;
     float unit = 1.0f;                                       // what one accumulator unit is worth
     if constexpr (UNITS) {
         typedef _Float16 v4h __attribute__((ext_vector_type(4)));
@@ -404,13 +401,6 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
             acc[2 * d][2] = ubyte_fma<1>(lo, sm, off); acc[2 * d][3] = ubyte_fma<1>(hi, sm, off);
             acc[2 * d + 1][0] = ubyte_fma<2>(lo, sm, off); acc[2 * d + 1][1] = ubyte_fma<2>(hi, sm, off);
             acc[2 * d + 1][2] = ubyte_fma<3>(lo, sm, off); acc[2 * d + 1][3] = ubyte_fma<3>(hi, sm, off);
-        }
-    }
-    if constexpr (COLVEC) {
-#pragma unroll
-        for (int ct = 0; ct < NT; ++ct) {
-            const float4 f = *reinterpret_cast<const float4*>(lds_cv + q * CL + 4 * ct);
-            acc[ct][0] *= f.x; acc[ct][1] *= f.y; acc[ct][2] *= f.z; acc[ct][3] *= f.w;
         }
     }
     // the m rank-1 updates: first operand = keys (result row i = 4 q' + b <-> column q' CL + 4 ct + b), second = values
