@@ -59,9 +59,10 @@ __global__ __launch_bounds__(WAVE) void pack_kernel(const PackParams p) {
         for (int t = 0; t < CPL; ++t) amax = fmaxf(amax, live ? fabsf(x[t]) : 0.0f);
         amax = block_max<T::LPG>(amax);
         const float s = fp16_scale(amax, T::QMAX);
+        const Divisor ds = scale_divisor(s);                 // x / s below is the IEEE quotient (sq_device.cuh)
         float q[CPL];
 #pragma unroll
-        for (int t = 0; t < CPL; ++t) q[t] = fminf(fmaxf(rintf(x[t] / s), -T::QMAX), T::QMAX);
+        for (int t = 0; t < CPL; ++t) q[t] = fminf(fmaxf(rintf(div_by(x[t], ds)), -T::QMAX), T::QMAX);
         if (in && live) store_row<BITS>(Sh + row * T::ROW_BYTES + l.cg * T::LANE_BYTES, encode_row<BITS>(q));
         if (in && lead) SCh[row * T::NG + gi] = f32_to_f16(s);
     }
@@ -95,10 +96,11 @@ __global__ __launch_bounds__(WAVE) void pack_v_kernel(const PackParams p) {
         const float s0 = fp16_scale(a0, QMAX), s1 = fp16_scale(a1, QMAX);
         if (live)
             *reinterpret_cast<uint32_t*>(SCh + (r0 / G) * DK + c0) = uint32_t(f32_to_f16(s0)) | (uint32_t(f32_to_f16(s1)) << 16);
+        const Divisor d0 = scale_divisor(s0), d1 = scale_divisor(s1);      // IEEE quotients (sq_device.cuh)
 #pragma unroll
         for (int r = 0; r < G; ++r) {
-            const int q0 = int(fminf(fmaxf(rintf(x[r].x / s0), -QMAX), QMAX));
-            const int q1 = int(fminf(fmaxf(rintf(x[r].y / s1), -QMAX), QMAX));
+            const int q0 = int(fminf(fmaxf(rintf(div_by(x[r].x, d0)), -QMAX), QMAX));
+            const int q1 = int(fminf(fmaxf(rintf(div_by(x[r].y, d1)), -QMAX), QMAX));
             uint8_t* row = Sh + (r0 + r) * ROW_BYTES;
             if (live) {
                 if constexpr (BITS == 8)

@@ -83,16 +83,53 @@ __device__ __forceinline__ void store_f(void* p, int dt, uint32_t i, float v) {
 // ---------------------------------------------------------------------------------------------------------------
 // rounding (reference: _fold_triton.py:52-62, _fused_triton.py:471-501)
 // ---------------------------------------------------------------------------------------------------------------
-// Quantizer scale: max(amax, 1e-8) / qmax -> fp16 (nearest even, subnormals kept) -> fp32, floored at 2^-24.
+// x / d with the divisor's reciprocal rc = RN(1 / d): q = RN(x rc), the exact remainder r = x - q d (one fma),
+// q + r rc rounded once.  With a correctly rounded reciprocal this is the correctly rounded quotient (Markstein's
+// division; the exception, a divisor whose significand is all ones, cannot occur: the divisors here are fp16 values
+// or the code ranges 3, 7, 31, 127), i.e. the IEEE quotient at a third of its instructions -- and of its latency,
+// which is what counts on a wavefront's serial path.  Checked in exact rational arithmetic over every fp16 divisor
+// and the four constants in tests/test_gga_division_cpu.py.
+__device__ __forceinline__ float div_rc(float x, float d, float rc) {
+    const float q = x * rc;
+    const float r = __builtin_fmaf(-q, d, x);
+    return __builtin_fmaf(r, rc, q);
+}
+// RN(1 / d) for a divisor that is an fp16 value (2^-24 and up): the hardware estimate (1 ulp) and one Newton step
+// with the exact residual.  The step leaves a relative error of 2^-46 before its single rounding, and the reciprocal
+// of an 11-bit significand is never closer than 2^-12 ulp to a rounding boundary, so the result is the correctly
+// rounded one.
+__device__ __forceinline__ float rcp_f16(float d) {
+    const float r = __builtin_amdgcn_rcpf(d);
+    return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+}
+// A scale as a divisor: the scale itself, or -- a scale that overflowed fp16 to infinity (values beyond 65504 qmax)
+// -- the largest finite float, which sends every finite value to code 0 as a division by infinity does, without an
+// infinity times zero on the way.
+struct Divisor {
+    float d, rc;
+};
+__device__ __forceinline__ Divisor scale_divisor(float scale) {
+    Divisor v;
+    v.d = fminf(scale, 3.0e38f);
+    v.rc = rcp_f16(v.d);
+    return v;
+}
+__device__ __forceinline__ float div_by(float x, const Divisor& v) { return div_rc(x, v.d, v.rc); }
+
+// Quantizer scale: max(amax, 1e-8) / qmax -> fp16 (nearest even, subnormals kept) -> fp32, floored at 2^-24.  qmax is
+// 7 or 127 at every call (a constant there, so 1 / qmax is folded).
 __device__ __forceinline__ float fp16_scale(float amax, float qmax) {
-    float s = fmaxf(amax, 1e-8f) / qmax;
+    float s = div_rc(fmaxf(amax, 1e-8f), qmax, 1.0f / qmax);
+    // the quotient is rounded to fp32 first and to fp16 second, as the reference's: without this the compiler folds
+    // the division's last fma and the conversion into one instruction with a single rounding (v_fma_mixlo_f16)
+    asm volatile("" : "+v"(s));
     s = float(_Float16(s));
     return fmaxf(s, FP16_TINY);
 }
 
-// Buffer entry: clamp(rint(x / scale), +-127) as a float.
+// Buffer entry: clamp(rint(x / scale), +-127) as a float; `scale` comes from `fp16_scale`.
 __device__ __forceinline__ float round_buf(float x, float scale) {
-    return fminf(fmaxf(rintf(x / scale), -127.0f), 127.0f);
+    return fminf(fmaxf(rintf(div_by(x, scale_divisor(scale))), -127.0f), 127.0f);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

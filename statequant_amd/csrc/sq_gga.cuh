@@ -60,23 +60,10 @@ __host__ __device__ constexpr int gga_code_bytes(int b, int dk, int dv) { return
 // fp16 with the fit's clamp: [2^-24, 65504], round to nearest even.
 __device__ __forceinline__ float gga_half(float x) { return float(_Float16(fminf(fmaxf(x, FP16_TINY), 65504.0f))); }
 
-// x / d with the divisor's reciprocal rc = RN(1 / d) computed once per row or column: q = RN(x rc), the exact
-// remainder r = x - q d (one fma), q + r rc rounded once.  With a correctly rounded reciprocal this is the correctly
-// rounded quotient (Markstein's division; the exception, a divisor whose significand is all ones, cannot occur: the
-// divisors here are fp16 values or 3, 7, 31, 127), so the codes are those of an IEEE division at a third of its
-// instructions.
-__device__ __forceinline__ float gga_div(float x, float d, float rc) {
-    const float q = x * rc;
-    const float r = __builtin_fmaf(-q, d, x);
-    return __builtin_fmaf(r, rc, q);
-}
-// RN(1 / d) for a divisor that is an fp16 value: the hardware estimate (1 ulp) and one Newton step with the exact
-// residual.  The step leaves a relative error of 2^-46 before its single rounding, and the reciprocal of an 11-bit
-// significand is never closer than 2^-12 ulp to a rounding boundary, so the result is the correctly rounded one.
-__device__ __forceinline__ float gga_rcp_f16(float d) {
-    const float r = __builtin_amdgcn_rcpf(d);
-    return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
-}
+// The fit's divisions go through `div_rc` / `rcp_f16` (sq_device.cuh): reciprocals once per row or column, IEEE
+// quotients at a third of the instructions.
+__device__ __forceinline__ float gga_div(float x, float d, float rc) { return div_rc(x, d, rc); }
+__device__ __forceinline__ float gga_rcp_f16(float d) { return rcp_f16(d); }
 
 // ---------------------------------------------------------------------------------------------------------------
 // sums / maxima along d_k: every thread ends with the totals of its CT columns (the same value in all row groups)

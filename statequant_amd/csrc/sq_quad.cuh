@@ -406,7 +406,9 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     // the m rank-1 updates: first operand = keys (result row i = 4 q' + b <-> column q' CL + 4 ct + b), second = values
     float bv[MT4];
     {
-        const float runit = UNITS ? 1.0f / unit : 1.0f;
+        // units are this kernel's own device (no reference quantity): an estimate plus one Newton step is plenty
+        const float r0 = __builtin_amdgcn_rcpf(unit);
+        const float runit = UNITS ? __builtin_fmaf(__builtin_fmaf(-unit, r0, 1.0f), r0, r0) : 1.0f;
 #pragma unroll
         for (int t = 0; t < MT4; ++t) bv[t] = UNITS ? bop[t] * runit : bop[t];
     }
@@ -425,7 +427,7 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
     if constexpr (LPG >= 2) { const Pair pm = pair16(mx); mx = fmaxf(pm.lo, pm.hi); }
     if constexpr (LPG >= 4) { const Pair pm = pair32(mx); mx = fmaxf(pm.lo, pm.hi); }
     const float sc = fp16_scale(UNITS ? mx * unit : mx, T::QMAX);
-    const float rs = UNITS ? unit * (1.0f / sc) : 1.0f / sc;
+    const float rs = UNITS ? unit * scale_divisor(sc).rc : scale_divisor(sc).rc;        // sc is an fp16 value: the exact reciprocal
     if (q % LPG == 0) *sc_out = f32_to_f16(sc);
     // new codes, back into the LDS image.  A scale in fp16's normal range cannot push a quotient past qmax + 1/2, so
     // the clamp is only compiled into the path taken when some lane's scale is subnormal (or at its floor).

@@ -943,7 +943,7 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
         for (int g = 0; g < T::NG; ++g) {
             const float other = __shfl_xor(gmax[g], 32);
             const float sc = fp16_scale(fmaxf(gmax[g], other), T::QMAX);
-            rs[g] = 1.0f / sc;
+            rs[g] = scale_divisor(sc).rc;
             if (kb == 0 && (!T::RAGV || row < T::DV)) sc_head[row * T::NG + g] = f32_to_f16(sc);
         }
 #pragma unroll
@@ -1094,7 +1094,7 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
                     mx = gmx[cs];
                 }
                 const float sc = fp16_scale(mx, T::QMAX);
-                rs[cs][hf] = 1.0f / sc;
+                rs[cs][hf] = scale_divisor(sc).rc;
                 // the group's last block writes the scale: the earlier ones' codes were decoded with the old one by then
                 if (kb == 0 && last_phase && v % VB == VB - 1 && grp * VH + hf < NGRP)
                     sc_head[(grp * VH + hf) * T::DK + 32 * cs + j] = f32_to_f16(sc);

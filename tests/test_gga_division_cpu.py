@@ -1,5 +1,6 @@
-"""The two shortcuts the GGA fit kernel takes for its divisions (statequant_amd/csrc/sq_gga.cuh: ``gga_rcp_f16``,
-``gga_div``), checked in exact rational arithmetic on the CPU: with fp32 fused multiply-adds modelled exactly,
+"""The two shortcuts the kernels take for their divisions (statequant_amd/csrc/sq_device.cuh: ``rcp_f16``, ``div_rc``
+-- the GGA fit's divisions, every quantizer scale ``absmax / qmax``, the buffer entries ``x / scale`` and the pack
+kernels' ``x / scale``), checked in exact rational arithmetic on the CPU: with fp32 fused multiply-adds modelled exactly,
 
   * one Newton step from ANY estimate within 1 ulp of 1 / d gives the correctly rounded fp32 reciprocal, for every
     fp16-valued divisor d (the row and column factors of the fit are fp16 values);
@@ -93,3 +94,47 @@ def test_reciprocal_division_is_the_ieee_quotient():
             bad += got != rn32(x / d)
             total += 1
     assert total > 10000 and bad == 0, (bad, total)
+
+
+def rn16_of_f32(fr32):
+    """fp16 (as an exact Fraction) nearest to an fp32 value, ties to even, subnormals kept; below the overflow range."""
+    if fr32 == 0:
+        return Fraction(0)
+    a = abs(fr32)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, -14)
+    ulp = Fraction(2) ** (e - 10)
+    n, rem = divmod(a, ulp)
+    n = int(n)
+    if rem * 2 > ulp or (rem * 2 == ulp and n % 2 == 1):
+        n += 1
+    return n * ulp
+
+
+def test_scale_is_rounded_twice_as_the_reference_does():
+    """``fp16_scale``: absmax / qmax as an fp32 quotient, THEN to fp16 -- two roundings, as torch's
+    ``(amax / qmax).to(float16)``.  A single rounding of the exact value of the division's last fused multiply-add
+    (what a fused fma-and-convert instruction would do) differs where the fp32 quotient is an fp16 tie; the absmax
+    below, 7 x an fp16 midpoint, is one that the pack test's data contains."""
+    rng = np.random.default_rng(1)
+    xs = [fr(np.float32(1.45391845703125))]
+    for qmax in (7, 127):
+        # fp32 values that are exactly qmax x (an fp16 midpoint): the quotient is the midpoint itself
+        mids = rng.integers(1024, 2048, 60) * 2 + 1                     # odd 12-bit significands
+        xs += [Fraction(int(m), 4096) * Fraction(2) ** int(e) * qmax for m, e in zip(mids, rng.integers(-6, 6, 60))]
+    xs += [fr(np.float32(v)) for v in np.abs(rng.standard_normal(400)) * 3]
+    single = 0
+    for qmax in (7, 127):
+        d, rc = Fraction(qmax), rn32(Fraction(1, qmax))
+        for x in xs:
+            if rn32(x) != x:
+                continue
+            q = rn32(x * rc)
+            r = fma32(-q, d, x)
+            s32 = fma32(r, rc, q)
+            assert s32 == rn32(x / d)
+            assert rn16_of_f32(s32) == rn16_of_f32(rn32(x / d))         # what the kernel computes == the reference
+            single += rn16_of_f32(r * rc + q) != rn16_of_f32(s32)       # one rounding of the unrounded sum instead
+    assert single > 0                                                   # the fused form would differ on some of these
