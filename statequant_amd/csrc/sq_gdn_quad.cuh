@@ -528,7 +528,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         }
         const float cmul = expf(gnew);
         const int fg = (fq * CL) / T::KGROUP;
-        float kop[DK / 16][MT4];
+        FoldKeys<T> kop;
         quad_fold_keys<T>(lds_kbr, lds_kbsf, m, lf, kop);
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi) {

@@ -412,7 +412,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         }
         const float cmul = expf(gnew);
         const int fg = (fq * CL) / T::KGROUP;
-        float kop[DK / 16][MT4];
+        FoldKeys<T> kop;
         quad_fold_keys<T>(lds_kbr, lds_kbsf, m, lf, kop);
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi) {

@@ -23,6 +23,7 @@
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "sq_tile.cuh"
 #include "sq_params.h"
@@ -35,6 +36,17 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant in
+// the body (a template argument there).
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // Diagnostic switch: SQ_LDS_PAD=<bytes> in the environment adds that much unused dynamic LDS to every launch of the
@@ -308,10 +320,27 @@ __device__ __forceinline__ float ubyte_fma(uint32_t w, float s, float o) {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // The folded keys as the matrix core's first operand, once per wavefront (they are the same for every half block):
-// kop[ct][t] = kx_{4 t + q}[column (n / 4) CL + 4 ct + n % 4] for lane (n, q); 0 for slots >= m.
+// key(ct, t) = kx_{4 t + q}[column (n / 4) CL + 4 ct + n % 4] for lane (n, q); 0 for slots >= m.  Held as fp32, or --
+// int4 states with the int8 buffer, whose kernels run at 80 registers where 16 more long-lived ones made the compiler
+// shuffle and spill -- as the raw bytes (biased to unsigned, four per register) with the slot's scale, expanded where
+// they are used: (byte - 128) x scale in one conversion and one fma, the same number as the product it replaces.
+template <class T>
+struct FoldKeys {
+    static constexpr int MT4 = (T::MMAX + 3) / 4, NT = T::DK / 16;
+    static constexpr bool PACKED = T::BITS == 4 && T::QBUF && NT % 4 == 0;
+    float f[PACKED ? 1 : NT][PACKED ? 1 : MT4];
+    uint32_t raw[PACKED ? MT4 : 1][PACKED ? NT / 4 : 1];
+    float ks[PACKED ? MT4 : 1], off[PACKED ? MT4 : 1];
+    template <int CT, int TT>
+    __device__ __forceinline__ float get() const {
+        if constexpr (PACKED) return ubyte_fma<CT % 4>(raw[TT][CT / 4], ks[TT], off[TT]);
+        else return f[CT][TT];
+    }
+};
+
 template <class T>
 __device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const float* lds_kbsf, int m, int lane,
-                                               float (&kop)[T::DK / 16][(T::MMAX + 3) / 4]) {
+                                               FoldKeys<T>& kop) {
     constexpr int MT4 = (T::MMAX + 3) / 4, CL = T::DK / 4, NT = CL / 4;
     const int n = lane & 15, q = lane >> 4;
     const int kcol = (n >> 2) * CL + (n & 3);
@@ -320,17 +349,29 @@ __device__ __forceinline__ void quad_fold_keys(const uint8_t* lds_kbr, const flo
         const int slot = 4 * t + q;
         const int sl = slot < m ? slot : 0;
         const float ks = T::QBUF ? lds_kbsf[sl] : 1.0f;
+        if constexpr (FoldKeys<T>::PACKED) {
 #pragma unroll
-        for (int ct = 0; ct < NT; ++ct) {
-            float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
-            if constexpr (T::QBUF) kv = kv * ks;
-            kop[ct][t] = slot < m ? kv : 0.0f;
+            for (int c4 = 0; c4 < NT / 4; ++c4) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) w |= uint32_t(lds_kbr[sl * T::DK + kcol + 4 * (4 * c4 + b)]) << (8 * b);
+                kop.raw[t][c4] = w ^ 0x80808080u;
+            }
+            kop.ks[t] = slot < m ? ks : 0.0f;                 // a slot beyond m contributes nothing
+            kop.off[t] = -128.0f * kop.ks[t];
+        } else {
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct) {
+                float kv = lds_raw<T::QBUF>(lds_kbr, sl * T::DK + kcol + 4 * ct);
+                if constexpr (T::QBUF) kv = kv * ks;
+                kop.f[ct][t] = slot < m ? kv : 0.0f;
+            }
         }
     }
 }
 
 template <class Q, class T>
-__device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float (&kop)[T::DK / 16][(T::MMAX + 3) / 4],
+__device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldKeys<T>& kop,
                                                const float (&bop)[(T::MMAX + 3) / 4], float cmul, float s_old,
                                                uint16_t* sc_out, int lane) {
     constexpr int MT4 = (T::MMAX + 3) / 4;
@@ -412,11 +453,11 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const float
 #pragma unroll
         for (int t = 0; t < MT4; ++t) bv[t] = UNITS ? bop[t] * runit : bop[t];
     }
-#pragma unroll
-    for (int ct = 0; ct < NT; ++ct)
-#pragma unroll
-        for (int t = 0; t < MT4; ++t)
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop[ct][t], bv[t], acc[ct], 0, 0, 0);
+    static_for<NT>([&](auto ct) {
+        static_for<MT4>([&](auto t) {
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop.template get<decltype(ct)::value, decltype(t)::value>(), bv[t], acc[ct], 0, 0, 0);
+        });
+    });
     // absmax of the lane's columns (three-operand maxima), then of its scale group
     float mx = 0.0f;
 #pragma unroll
