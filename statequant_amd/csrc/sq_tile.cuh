@@ -82,6 +82,9 @@ struct Tile {
     static constexpr int B_BYTES = FLT ? 2 * KROW * 4 : (DK / CPL) * PSLOTS * CPL;
     static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
     static constexpr int A_BYTES = FLT ? 0 : MR * A_PITCH;
+    // LDS pitch of one result column's 32 integer sums: a lane parks 16 bytes per store and the 32 lanes of a store
+    // hold 32 different columns, which at a pitch of 32 words would all meet in the same four banks
+    static constexpr int C_PITCH = MR + 4;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
     static constexpr int SC_ELEMS = FLT ? 0 : AXV ? (DV / GROUP) * DK : DV * NG;      // fp16 scales of one head
     static constexpr int SC_BYTES = FLT ? 16 : round_up(SC_ELEMS * 2, 16);
@@ -102,7 +105,7 @@ struct LdsPlan {
     static constexpr int B = XS + round_up(NV * T::VH * T::NG * 4, 16);
     static constexpr int A = B + (T::AXV ? T::B_BYTES : 0);    // value-axis: planes are rebuilt per row block
     static constexpr int C = A;
-    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::VH * T::PLANES * NV * T::MR * 4;
+    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::VH * T::PLANES * NV * T::C_PITCH * 4;
     static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
                                                     : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
     static constexpr int OWN = A + BAC;
@@ -494,7 +497,7 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
         }
         wave_sync();                                     // every lane has its codes: the sums may take their place
         if (j < NCOL) {
-            int4* dst = reinterpret_cast<int4*>(lds_c + j * T::MR + 4 * kb);
+            int4* dst = reinterpret_cast<int4*>(lds_c + j * T::C_PITCH + 4 * kb);
 #pragma unroll
             for (int a = 0; a < 4; ++a)
                 dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
@@ -505,16 +508,16 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
             float s = 0.0f;
             if constexpr (T::VH > 1) {                       // the columns of the row's own half
                 const int g = j / T::GROUP;
-                const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
-                const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
-                                               __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
+                const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::C_PITCH + j;
+                const float f = __builtin_fmaf(float(c[2 * T::C_PITCH]), 65536.0f,
+                                               __builtin_fmaf(float(c[T::C_PITCH]), 256.0f, float(c[0])));
                 s = f * (g == 0 ? xs[0] : xs[T::VH - 1]);
             } else {
 #pragma unroll
                 for (int g = 0; g < T::NG; ++g) {
-                    const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::MR + j;
-                    const float f = __builtin_fmaf(float(c[2 * T::MR]), 65536.0f,
-                                                   __builtin_fmaf(float(c[T::MR]), 256.0f, float(c[0])));
+                    const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::C_PITCH + j;
+                    const float f = __builtin_fmaf(float(c[2 * T::C_PITCH]), 65536.0f,
+                                                   __builtin_fmaf(float(c[T::C_PITCH]), 256.0f, float(c[0])));
                     const float term = T::AXV ? f * xs[g] : (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
                     s = g == 0 ? term : s + term;
                 }
