@@ -138,7 +138,6 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams args)
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
     uint8_t* lds_a = lds + L::A;
-    int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);          // the fold's operands overlay the above
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
@@ -237,7 +236,7 @@ __global__ __launch_bounds__(WAVE, 4) void gdn_step_kernel(const GdnParams args)
     float xe2[2][T::NE];
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) { xe2[0][t] = qe[t]; xe2[1][t] = ke[t]; }
-    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, xe2, own);
+    state_pass<T, 2>(lane_base, F.win, lds_b, lds_xs, lds_sc, lds_a, lds_own, l, xe2, own);
 
     const KeyBuf<T>& kbuf = F.kbuf;
     const float gb_lane = F.gb_lane;

@@ -33,7 +33,6 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
     uint8_t* lds_a = lds + L::A;
-    int32_t* lds_ci = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
@@ -204,7 +203,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
 
     // ---- state pass against A*q, A*k ----
     float own[2][T::NOWN];
-    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_ci, lds_own, l, xa, own);
+    state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_own, l, xa, own);
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll

@@ -26,7 +26,6 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
     uint8_t* lds_b = lds + L::B;
     float* lds_xs = reinterpret_cast<float*>(lds + L::XS);
     uint8_t* lds_a = lds + L::A;
-    int32_t* lds_c = reinterpret_cast<int32_t*>(lds + L::C);
     float* lds_own = reinterpret_cast<float*>(lds + L::OWN);
     float* lds_k = reinterpret_cast<float*>(lds + L::FK);
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
@@ -150,7 +149,7 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
     float xe1[1][T::NE];
 #pragma unroll
     for (int t = 0; t < T::NE; ++t) xe1[0][t] = ce[t];
-    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_c, lds_own, l, xe1, own);
+    state_pass<T, 1>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_own, l, xe1, own);
 
     // ---- owned rows: y, and the value to buffer ----
     float u[T::NOWN], amax = 0.0f;

@@ -82,9 +82,6 @@ struct Tile {
     static constexpr int B_BYTES = FLT ? 2 * KROW * 4 : (DK / CPL) * PSLOTS * CPL;
     static constexpr int A_PITCH = ROW_BYTES + LANE_BYTES;  // LDS row pitch of a row block on its way to operand shape
     static constexpr int A_BYTES = FLT ? 0 : MR * A_PITCH;
-    // LDS pitch of one result column's 32 integer sums: a lane parks 16 bytes per store and the 32 lanes of a store
-    // hold 32 different columns, which at a pitch of 32 words would all meet in the same four banks
-    static constexpr int C_PITCH = MR + 4;
     static constexpr int UB_BYTES = round_up(MMAX * DV * BE, 16);
     static constexpr int SC_ELEMS = FLT ? 0 : AXV ? (DV / GROUP) * DK : DV * NG;      // fp16 scales of one head
     static constexpr int SC_BYTES = FLT ? 16 : round_up(SC_ELEMS * 2, 16);
@@ -92,23 +89,19 @@ struct Tile {
 
 // LDS plan of a step kernel that stages NX d_k vectors and reads the state out against NV of them.  Front end: the
 // vectors, the raw buffered values, the raw scales, the digit planes with their exponents, one row block of codes,
-// its integer sums, the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay
-// each other.
+// the finished row sums.  Fold: folded keys, folded values, column multipliers.  The two overlay each other.
 template <class T, int NX, int NV = 2>
 struct LdsPlan {
     static constexpr int X = 0;
     static constexpr int UB = X + NX * T::KROW * 4;
     static constexpr int SC = UB + T::UB_BYTES;
     static constexpr int XS = SC + T::SC_BYTES;
-    // one region, three tenants in turn: the digit planes (until the pass has them in registers), then per row block
-    // the codes on their way to operand shape and, once the block's products are issued, its integer sums
+    // one region, two tenants in turn: the digit planes (until the pass has them in registers), then per row block
+    // the codes on their way to operand shape
     static constexpr int B = XS + round_up(NV * T::VH * T::NG * 4, 16);
     static constexpr int A = B + (T::AXV ? T::B_BYTES : 0);    // value-axis: planes are rebuilt per row block
-    static constexpr int C = A;
-    static constexpr int C_BYTES = T::FLT ? 0 : T::NG * T::VH * T::PLANES * NV * T::C_PITCH * 4;
-    static constexpr int BAC = T::A_BYTES > C_BYTES ? (T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES)
-                                                    : (C_BYTES > T::B_BYTES ? C_BYTES : T::B_BYTES);
-    static constexpr int OWN = A + BAC;
+    static constexpr int BA = T::A_BYTES > T::B_BYTES ? T::A_BYTES : T::B_BYTES;
+    static constexpr int OWN = A + BA;
     static constexpr int FRONT = OWN + NV * T::UROW * 4;
     static constexpr int FK = 0;
     static constexpr int FU = FK + T::MMAX * T::KROW * 4;
@@ -414,45 +407,52 @@ __device__ __forceinline__ void float_pass(const uint8_t* lane_base, Window<T>& 
 }
 
 // Row sums of the whole tile against NV read-out vectors: own[v][t] = (S0 x_v)[lane + 64 t], scales applied.
-// Per block of 32 rows: one matrix instruction per column step accumulates, per scale group, the 32 x (3 NV) integer
-// sums (row x digit plane); the lanes holding a plane's column park them in LDS; then lane (i, v) turns row i's sums
-// for vector v into fp32 -- (d0 + 2^8 d1 + 2^16 d2) 2^(e-22) is the group's dot product, times the group's scale,
-// groups added in order (the reference's "(group sum) x scale, group by group", _fold_triton.py:191-196).  The block
+// Per block of 32 rows, one matrix instruction per column step accumulates, per scale group, the (3 NV) x 32 integer
+// sums (digit plane x row): the digit planes are the FIRST operand and the codes the second, so the result leaves
+// row n's sums in lane n -- operand row 8 a + 4 v + b carries, for vector v, entry q = 4 a + b of the list (scale
+// group g, digit d) at q = 3 g + d, and the instruction hands lane (n, kb) rows 8 a + 4 kb + b in element 4 a + b:
+// lane (n, v) ends with all of row n's sums against vector v in its own registers and turns them into fp32 --
+// (d0 + 2^8 d1 + 2^16 d2) 2^(e-22) is the group's dot product, times the group's scale, groups added in order (the
+// reference's "(group sum) x scale, group by group", _fold_triton.py:191-196).  A plane takes part only in the column
+// steps of its own scale group (zero elsewhere), so ONE accumulation over all steps keeps the groups apart.  The block
 // just consumed is refilled with the block after next.  A block changes from row shape to operand shape through LDS
 // (lds_a, row pitch = row + one lane piece: both the row-shaped writes and the operand-shaped reads are conflict
-// free): operand lane (i = lane % 32, kb = lane / 32) takes, for column step ks, the 16 codes at row i, columns
-// 32 ks + 16 kb.  Result layout of the instruction: lane (j, kb) holds column j (= plane), rows 8 a + 4 kb + b in
-// element 4 a + b.
+// free): operand lane (n = lane % 32, kb = lane / 32) takes, for column step ks, the 16 codes at row n, columns
+// 32 ks + 16 kb.
 // Value-axis scales: the scale belongs to (row block, column), so it goes into the read-out vector instead --
-// x'_k = x_k s[rb][k] -- and the digit planes are rebuilt from `xe` (element lane + 64 t of each vector) per block.
+// x'_k = x_k s[rb][k] -- and the digit planes are rebuilt from `xe` (element lane + 64 t of each vector) per block;
+// scale groups of half a row block take the key groups' place in the list (entry 3 h + d: the read-out against the
+// scales of half h), and a row keeps its own half's.
 template <class T, int NV>
 __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& w, uint8_t* lds_b, float* lds_xs,
-                                           const uint16_t* lds_sc, uint8_t* lds_a, int32_t* lds_c, float* lds_own,
+                                           const uint16_t* lds_sc, uint8_t* lds_a, float* lds_own,
                                            const LaneId& l, const float (&xe)[NV][T::NE], float (&own)[NV][T::NOWN]) {
     if constexpr (T::FLT) {
         float_pass<T, NV>(lane_base, w, lds_b, lds_own, l, xe, own);
         return;
     } else {
-    constexpr int NPL = T::PLANES * NV;
-    // result columns in use: (scale group, vector, digit); value-axis groups of half a row block take the group's
-    // place: columns [h NPL, (h + 1) NPL) carry the read-out against the scales of half h, and a row keeps its own half's
-    constexpr int NGC = T::NG * T::VH;
-    constexpr int NCOL = NPL * NGC;
-    static_assert(NCOL <= T::MR && NV <= 2, "groups x digit planes must fit the instruction's 32 result columns");
+    constexpr int NGC = T::NG * T::VH;                       // entries of the list / 3
+    // one vector and more groups than a lane's 16 elements hold (d_k 256 in groups of 32): the second half of the
+    // operand rows carries groups 5 .. instead of a second vector, and lane (n, 1) continues lane (n, 0)'s sum
+    constexpr bool WIDE = NV == 1 && T::PLANES * NGC > 16;
+    constexpr int GPL = 5;                                   // groups per lane of a wide list
+    static_assert(NV <= 2 && (WIDE ? NGC <= 2 * GPL && T::VH == 1 : T::PLANES * NGC <= 16),
+                  "groups x digit planes must fit the 16 result rows of a lane (one vector: of its two lanes)");
     const int j = l.lane % T::MR, kb = l.lane / T::MR;
-    // second operand, per column step: result column j = g NPL + p takes digit plane p, but only on the column steps
-    // that belong to scale group g (zero elsewhere), so ONE accumulation over all steps leaves every group's sums in
-    // its own columns
-    const int colg = j / NPL, colp = j - colg * NPL;
-    v4i bop[T::NKS];
+    // first operand: which (vector, list entry) this lane's operand row stands for
+    const int rv = (j >> 2) & 1, rq = 4 * (j >> 3) + (j & 3);
+    const int pgl = rq / T::PLANES, rd = rq - pgl * T::PLANES;
+    const int pg = WIDE ? GPL * rv + pgl : pgl, pv = WIDE ? 0 : rv;
+    const bool rlive = WIDE ? pgl < GPL && pg < NGC : rv < NV && pg < NGC;
+    v4i pop[T::NKS];
     float xs[NGC];
     auto fetch_planes = [&] {
+        const int slot = rlive ? (T::VH > 1 ? (pg * NV + pv) * T::PLANES + rd : T::PLANES * pv + rd) : 0;
 #pragma unroll
         for (int ks = 0; ks < T::NKS; ++ks) {
-            const int slot = T::VH > 1 ? (colg < T::VH ? colg * NPL + colp : 0) : (colp & 7);
             const v4i d = *reinterpret_cast<const v4i*>(lds_b + ((2 * ks + kb) * T::PSLOTS + slot) * CPL);
-            const bool mine = T::VH > 1 ? true : colg == (ks * T::MK) / T::KGROUP;
-            bop[ks] = mine ? d : v4i{0, 0, 0, 0};
+            const bool mine = rlive && (T::VH > 1 ? true : pg == (ks * T::MK) / T::KGROUP);
+            pop[ks] = mine ? d : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int g = 0; g < NGC; ++g)
@@ -493,38 +493,50 @@ __device__ __forceinline__ void state_pass(const uint8_t* lane_base, Window<T>& 
 #pragma unroll
         for (int ks = 0; ks < T::NKS; ++ks) {
             const RawRow<T::BITS> r = load_row<T::BITS>(lds_a + j * T::A_PITCH + (2 * ks + kb) * T::LANE_BYTES);
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(operand<T::BITS>(r), bop[ks], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(pop[ks], operand<T::BITS>(r), acc, 0, 0, 0);
         }
-        wave_sync();                                     // every lane has its codes: the sums may take their place
-        if (j < NCOL) {
-            int4* dst = reinterpret_cast<int4*>(lds_c + j * T::C_PITCH + 4 * kb);
+        if constexpr (WIDE) {
+            const int row = rb * T::MR + j;
+            float t[GPL];
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
-                dst[2 * a] = make_int4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
-        }
-        wave_sync();
-        if (kb < NV) {
+            for (int g = 0; g < GPL; ++g) {
+                const int gg = GPL * kb + g;                 // this lane's g-th group
+                const float f = __builtin_fmaf(float(acc[3 * g + 2]), 65536.0f,
+                                               __builtin_fmaf(float(acc[3 * g + 1]), 256.0f, float(acc[3 * g])));
+                const float x = kb ? xs[GPL + g < NGC ? GPL + g : 0] : xs[g];
+                t[g] = (f * x) * f16_to_f32(lds_sc[row * T::NG + (gg < NGC ? gg : 0)]);
+            }
+            float s = t[0];
+#pragma unroll
+            for (int g = 1; g < GPL; ++g) s = s + t[g];
+            const float lo = __shfl(s, j);                   // groups 0 .. 4, from lane (n, 0)
+            s = lo;
+#pragma unroll
+            for (int g = 0; g < GPL; ++g)
+                if (GPL + g < NGC) s = s + t[g];
+            if (kb == 1) lds_own[row] = s;
+        } else if (kb < NV) {
             const int row = rb * T::MR + j;
             float s = 0.0f;
-            if constexpr (T::VH > 1) {                       // the columns of the row's own half
-                const int g = j / T::GROUP;
-                const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::C_PITCH + j;
-                const float f = __builtin_fmaf(float(c[2 * T::C_PITCH]), 65536.0f,
-                                               __builtin_fmaf(float(c[T::C_PITCH]), 256.0f, float(c[0])));
-                s = f * (g == 0 ? xs[0] : xs[T::VH - 1]);
+            if constexpr (T::VH > 1) {                       // the entries of the row's own half
+                static_assert(T::VH == 2, "two halves per row block");
+                const bool up = j >= T::GROUP;
+                const float f = __builtin_fmaf(float(up ? acc[5] : acc[2]), 65536.0f,
+                                               __builtin_fmaf(float(up ? acc[4] : acc[1]), 256.0f,
+                                                              float(up ? acc[3] : acc[0])));
+                s = f * (up ? xs[T::VH - 1] : xs[0]);
             } else {
 #pragma unroll
                 for (int g = 0; g < T::NG; ++g) {
-                    const int32_t* c = lds_c + (g * NPL + T::PLANES * kb) * T::C_PITCH + j;
-                    const float f = __builtin_fmaf(float(c[2 * T::C_PITCH]), 65536.0f,
-                                                   __builtin_fmaf(float(c[T::C_PITCH]), 256.0f, float(c[0])));
+                    const float f = __builtin_fmaf(float(acc[3 * g + 2]), 65536.0f,
+                                                   __builtin_fmaf(float(acc[3 * g + 1]), 256.0f, float(acc[3 * g])));
                     const float term = T::AXV ? f * xs[g] : (f * xs[g]) * f16_to_f32(lds_sc[row * T::NG + g]);
                     s = g == 0 ? term : s + term;
                 }
             }
             lds_own[kb * T::UROW + row] = s;
         }
-        wave_sync();
+        wave_sync();                                     // every lane has its codes: the next block may take their place
     }
 #pragma unroll
     for (int v = 0; v < NV; ++v)
