@@ -1,11 +1,13 @@
 #!/usr/bin/env python3
-"""Where the life of a workgroup goes: a timeline of one launch of the Gated DeltaNet workgroup-per-key-head step.
+"""Where the life of a workgroup goes: a timeline of one launch of the Gated DeltaNet workgroup-per-key-head step or
+of the KDA one-wavefront step.
 
     python -m statequant_amd.csrc.build --timeline        # once, here: writes statequant_amd/libsqhip_timeline.so
-    python profile_timeline.py [--workload gdn-int8-g128] [--steps 3,7] [--out profiles]
+    python profile_timeline.py [--workload gdn-int8-g128 | kda-int4-g32] [--steps 3,7] [--out profiles]
 
-The timeline library is the product library with marks compiled into `gdn_quad_kernel` (sq_gdn_quad.cuh,
--DSQ_TIMELINE): every wavefront stores the GPU's 100 MHz real-time counter at 15 points of its life.  This script
+The timeline library is the product library with marks compiled into `gdn_quad_kernel` (sq_gdn_quad.cuh) and
+`kda_step_kernel` (sq_kda.cuh) by -DSQ_TIMELINE (sq_timeline.cuh): every wavefront stores the GPU's 100 MHz
+real-time counter at 15 (KDA: 9) points of its life.  This script
 builds bench.py's workload, runs whole fold periods back to back (eager launches, the 24 layer states in turn, as
 bench.py does without a graph), and for each requested step of the fold period (0 .. m - 1; the last one folds) has
 the last layer's launch of that step write its marks.  It prints and writes `<out>/<workload>_step_timeline.txt`:
@@ -27,6 +29,9 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 import bench  # noqa: E402
 from statequant_amd.kernels import _hip  # noqa: E402
 
+MARKS_KDA = ['entry', 'slot known, token loads issued', 'fill count here, every load issued',
+             'vectors, scales, buffered values staged', 'keys and decays here, coefficients done', 'state pass done',
+             'outputs stored', 'appended', 'folded (full buffer), counters advanced']
 MARKS = ['entry', 'item known (leading arguments here)', 'slot known, token loads issued', 'counters issued',
          'row blocks issued', 'fill count here, buffer loads issued', 'roles done, all loads landed in LDS',
          'first barrier passed', 'state pass done', 'buffer dot products done', 'second barrier passed',
@@ -39,8 +44,8 @@ def timeline(workload, step, dev, m=8):
     fam, lay, views, idx = bench.build(workload, m, dev)
     inputs, extra = bench.make_inputs(fam, lay, slots, layers, m, dev)
     out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
-    waves = 4                                                # two value heads x two wavefronts
-    nwg = slots * hv // 2
+    waves = 4 if fam == 'gdn' else 1                         # GDN: two value heads x two wavefronts; KDA: one per head
+    nwg = slots * hv // 2 if fam == 'gdn' else slots * hv
     buf = torch.zeros(nwg * waves * 16, dtype=torch.int64, device=dev)
 
     def run(s, upto):
@@ -59,29 +64,33 @@ def timeline(workload, step, dev, m=8):
     torch.cuda.synchronize()
     t = buf.cpu().numpy().reshape(nwg, waves, 16)[:, :, :15].astype(np.float64)
     if not (t[:, :, 0] > 0).all():
-        sys.exit(f'profile_timeline.py: {workload} did not run on the instrumented kernel (gdn_quad_kernel serves '
-                 'Gated DeltaNet int4 / int8 states with key-axis groups, two value heads per key head)')
-    return t, nwg
+        sys.exit(f'profile_timeline.py: {workload} did not run on an instrumented kernel (gdn_quad_kernel serves '
+                 'Gated DeltaNet int4 / int8 states with key-axis groups, two value heads per key head; '
+                 'kda_step_kernel every KDA state)')
+    return t, nwg, fam
 
 
-def report(workload, step, t, nwg, m=8):
-    last = 14 if step == m - 1 else 13
+def report(workload, step, t, nwg, fam, m=8):
+    marks = MARKS if fam == 'gdn' else MARKS_KDA
+    last = (14 if step == m - 1 else 13) if fam == 'gdn' else 8
+    waves = t.shape[1]
     T = (t - t[:, :, 0].min()) * TICK_US                     # us since the first wavefront started
     life = T[:, :, last] - T[:, :, 0]
     d = np.diff(T, axis=2)
     lines = [f'-- step {step} of the fold period ({"the fold step" if step == m - 1 else "a plain step"}), '
-             f'{nwg} workgroups of 4 wavefronts --',
+             f'{nwg} workgroups of {waves} wavefront{"s" if waves > 1 else ""} --',
              f'launch: first wavefront starts at 0, last one ends at {T[:, :, :last + 1].max():.2f} us',
              f'wavefront life, us: mean {life.mean():.2f}  median {np.median(life):.2f}  10 % {np.percentile(life, 10):.2f}'
              f'  90 % {np.percentile(life, 90):.2f}',
              'interval, us over all wavefronts:                                                 mean  median   90 %']
     for k in range(last):
-        lines.append(f'  {MARKS[k]:<38} -> {MARKS[k + 1]:<38} {d[:, :, k].mean():6.2f} {np.median(d[:, :, k]):6.2f} '
+        lines.append(f'  {marks[k]:<38} -> {marks[k + 1]:<38} {d[:, :, k].mean():6.2f} {np.median(d[:, :, k]):6.2f} '
                      f'{np.percentile(d[:, :, k], 90):6.2f}')
-    lines.append('mean of each interval by wavefront of the workgroup (1 and 3: q and k vectors; 0 and 2: gates; '
-                 '2: key append):')
-    for w in range(4):
-        lines.append(f'  wavefront {w}: ' + ' '.join(f'{d[:, w, k].mean():5.2f}' for k in range(last)))
+    if waves > 1:
+        lines.append('mean of each interval by wavefront of the workgroup (1 and 3: q and k vectors; 0 and 2: gates; '
+                     '2: key append):')
+        for w in range(waves):
+            lines.append(f'  wavefront {w}: ' + ' '.join(f'{d[:, w, k].mean():5.2f}' for k in range(last)))
     st, en = T[:, 0, 0], T[:, :, last].max(axis=1)
     edges = np.arange(0, T[:, :, :last + 1].max() + 2, 2.0)
     lines.append('workgroups starting per 2 us: ' + ' '.join(str(x) for x in np.histogram(st, edges)[0]))
@@ -103,8 +112,9 @@ def main():
     _hip.LIB_PATH = lib
     if not torch.cuda.is_available():
         sys.exit('profile_timeline.py: no GPU visible')
-    if bench.WORKLOADS[a.workload][0] != 'gdn':
-        sys.exit('profile_timeline.py: only the Gated DeltaNet workgroup-per-key-head kernel carries the marks')
+    if bench.WORKLOADS[a.workload][0] not in ('gdn', 'kda'):
+        sys.exit('profile_timeline.py: only the Gated DeltaNet workgroup-per-key-head kernel and the KDA kernel carry '
+                 'the marks')
     dev = torch.device('cuda:0')
     torch.cuda.set_device(dev)
     lines = [f'timeline of the decode-step kernel, bench.py workload {a.workload}',
@@ -113,8 +123,8 @@ def main():
              'marks: s_memrealtime (100 MHz) in every wavefront of one launch, the last of 24 back-to-back layer '
              'launches of the step; a marked launch runs about 10 % longer than the product kernel', '']
     for step in (int(x) for x in a.steps.split(',')):
-        t, nwg = timeline(a.workload, step, dev)
-        lines += report(a.workload, step, t, nwg) + ['']
+        t, nwg, fam = timeline(a.workload, step, dev)
+        lines += report(a.workload, step, t, nwg, fam) + ['']
     text = '\n'.join(lines)
     print(text)
     os.makedirs(a.out, exist_ok=True)

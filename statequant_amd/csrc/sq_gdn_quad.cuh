@@ -17,6 +17,7 @@
 #pragma once
 #include "sq_gdn.cuh"
 #include "sq_quad.cuh"
+#include "sq_timeline.cuh"
 
 namespace sq {
 
@@ -66,28 +67,6 @@ struct GdnLoads {
     int np;
     uint32_t xr[Q::NE], xr2[Q::NE], g0, g1, g2, g3, vr;
 };
-
-// Optional instrumentation, compiled in with -DSQ_TIMELINE only (build.py --timeline writes a library of its own):
-// every wavefront records the 100 MHz real-time counter at fixed points of its life, 16 x 8 bytes per wavefront,
-// workgroup-major, into the buffer whose device address the environment variable SQ_TIMELINE_BUF holds (decimal) at
-// the time of the launch; a launch can then be laid out as a timeline of its workgroups (profile_timeline.py).  A
-// mark waits for the scalar loads in flight, so the marks cost a wavefront about a microsecond altogether.  Without
-// the define they compile to nothing.
-#ifdef SQ_TIMELINE
-#include <stdlib.h>
-#define SQ_TL_PARAM uint64_t* tl,
-#define SQ_MARK(k)                                                                                                 \
-    do {                                                                                                           \
-        if (tl) {                                                                                                  \
-            uint64_t t_;                                                                                           \
-            asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_)::"memory");                         \
-            if ((threadIdx.x & 63) == 0) tl[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16 + (k)] = t_; \
-        }                                                                                                          \
-    } while (0)
-#else
-#define SQ_TL_PARAM
-#define SQ_MARK(k) do { } while (0)
-#endif
 
 // SPEC > 0 compiles the serving cases in, so that dtypes and options cost no scalar branches on the way to the first
 // load (measured on the 128 x 128 int8 step: 35.4 -> 34.2 us per launch): bf16 q / k / v / out, no dispatch order,
@@ -565,8 +544,7 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     if (p.per_xcd == 0) p.rows_per_xcd = 0;
 #ifdef SQ_TIMELINE
-    const char* tl_env = getenv("SQ_TIMELINE_BUF");
-    uint64_t* tl = tl_env ? reinterpret_cast<uint64_t*>(strtoull(tl_env, nullptr, 10)) : nullptr;
+    uint64_t* tl = sq_timeline_buffer();
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
                        quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, tl, p);
 #else

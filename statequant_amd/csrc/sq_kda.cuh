@@ -11,6 +11,7 @@
 #pragma once
 #include "sq_tile.cuh"
 #include "sq_params.h"
+#include "sq_timeline.cuh"
 
 namespace sq {
 
@@ -20,7 +21,10 @@ namespace sq {
 __device__ __forceinline__ float kda_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
 
 template <class T, int SPEC>
-__global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args) {
+__global__ __launch_bounds__(WAVE, 4)
+void kda_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd,
+                     int hv, int hv_shift, SQ_TL_PARAM const KdaParams args) {
+    SQ_MARK(0);                                                   // entry
     KdaParams p = args;
     assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 3, 2>;                                   // q, k (normalised), G_n
@@ -39,14 +43,14 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
     float* lds_c = reinterpret_cast<float*>(lds + L::FC);
 
     const LaneId l = lane_id<T>();
-    const TileId tid = tile_id(p);
+    const TileId tid = tile_id_lead<SPEC>(order, per_xcd, rows_per_xcd, hv, hv_shift);   // from the leading arguments
     const uint32_t b = tid.b, h = tid.h;
     const int m = p.m;
     const uint32_t um = m;
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);          // scalar load: on its way while the inputs are issued
+    const int32_t slot = idx ? idx[b] : int32_t(b);              // scalar load: on its way while the inputs are issued
     // the token's own operands first: their addresses need the batch row only, not the slot
     uint32_t qr[T::NE], kr_[T::NE], gr[T::NE];
     const void* qb = advance(p.q, p.q_dt, uint64_t(b) * p.s_q + h * DK);
@@ -70,10 +74,11 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         vr[t] = load_raw(vb, p.v_dt, r);
     }
     void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
-    if (p.idx && slot <= 0) {
+    if (idx && slot <= 0) {
         for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
+    SQ_MARK(1);                                                   // slot known, the token's loads issued
     const uint32_t seq = slot;
 
     uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
@@ -119,6 +124,8 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         for (int k = 0; k < CPL / 4; ++k) gbp[t][k] = g4[k];
     }
 
+    SQ_MARK(2);                                                   // fill count here, every load issued
+
     // ---- prep: q, k normalised, the running decay per channel ----
     const bool full = n == m - 1;
     float qe[T::NE], ke[T::NE], gn[T::NE];
@@ -161,6 +168,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
 #pragma unroll
     for (int i = 0; i < T::MMAX; ++i) ubs[i] = T::QBUF ? lane_bcast(f16_to_f32(ubs_raw), i) : 1.0f;
     wave_sync();
+    SQ_MARK(3);                                                   // vectors, scales, buffered values here and staged
 
     // ---- buffer coefficients with the per-channel decay ratio folded into the buffered key ----
     float cqk[2][T::MMAX];
@@ -201,9 +209,12 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         }
     }
 
+    SQ_MARK(4);                                                   // buffered keys and decays here, coefficients done
+
     // ---- state pass against A*q, A*k ----
     float own[2][T::NOWN];
     state_pass<T, 2>(lane_base, win, lds_b, lds_xs, lds_sc, lds_a, lds_own, l, xa, own);
+    SQ_MARK(5);                                                   // state pass done (all codes here)
 
     float u[T::NOWN], amax = 0.0f;
 #pragma unroll
@@ -222,6 +233,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         amax = fmaxf(amax, fabsf(u[t]));
     }
 
+    SQ_MARK(6);                                                   // outputs stored
     // ---- append: decay vector, delta value, key ----
     float us = 1.0f, ks = 1.0f;
     if constexpr (T::QBUF) {
@@ -240,6 +252,7 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         if (e < DK) GBh[n * DK + e] = gn[t];
     }
 
+    SQ_MARK(7);                                                   // appended
     // ---- fold ----
     if (full) {
         float uo[T::NOWN][T::MMAX];
@@ -284,11 +297,18 @@ __global__ __launch_bounds__(WAVE, 4) void kda_step_kernel(const KdaParams args)
         if (e < DK) gch[e] = full ? 0.0f : gn[t];
     }
     if (l.lane == 0) *np = full ? 0 : n + 1;
+    SQ_MARK(8);                                                   // folded (a full buffer), counters advanced
 }
 
 template <class T, int SPEC>
 int launch_kda(const KdaParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+#ifdef SQ_TIMELINE
+    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
+                       p.rows_per_xcd, p.hv, p.hv_shift, sq_timeline_buffer(), p);
+#else
+    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
+                       p.rows_per_xcd, p.hv, p.hv_shift, p);
+#endif
     return int(hipGetLastError());
 }
 

@@ -15,7 +15,9 @@ namespace sq {
 // Occupancy target: four wavefronts per SIMD; the d_state-256 tile does not fit 128 registers, and asked for two it
 // is compiled at 234 without spills (asked for four the compiler gives up at 364, one wavefront per SIMD).
 template <class T, int SPEC>
-__global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(const Mamba2Params args) {
+__global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4)
+void mamba2_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd,
+                        int rows_per_xcd, int hv, int hv_shift, const Mamba2Params args) {
     Mamba2Params p = args;
     assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 1, 1>;
@@ -31,15 +33,15 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
     const LaneId l = lane_id<T>();
-    const TileId tid = tile_id(p);
-    const uint32_t b = tid.b, h = tid.h, hk = tid.hk;
+    const TileId tid = tile_id_lead<SPEC>(order, per_xcd, rows_per_xcd, hv, hv_shift);   // from the leading arguments
+    const uint32_t b = tid.b, h = tid.h, hk = p.gqa_shift >= 0 ? tid.h >> p.gqa_shift : tid.h / p.gqa;
     const int gqa = p.gqa;
     const int m = p.m;
     const uint32_t um = m;
     constexpr int DK = T::DK, DV = T::DV;
     constexpr int KT = KeyBuf<T>::KT;
 
-    const int32_t slot = p.idx ? p.idx[b] : int32_t(b);          // scalar load: on its way while the inputs are issued
+    const int32_t slot = idx ? idx[b] : int32_t(b);              // scalar load: on its way while the inputs are issued
     // the token's own operands first: their addresses need the batch row only, not the slot
     uint32_t cr[T::NE], br[T::NE];
     const void* cb = advance(p.C, p.C_dt, uint64_t(b) * p.s_C + hk * DK);
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
         xr_raw[t] = load_raw(xb, p.x_dt, r);
     }
     void* const outp = advance(p.out, p.out_dt, uint64_t(b) * p.s_out + h * DV);
-    if (p.idx && slot <= 0) {
+    if (idx && slot <= 0) {
         for (int r = l.lane; r < DV; r += WAVE) store_f(outp, p.out_dt, r, 0.0f);
         return;
     }
@@ -214,7 +216,8 @@ __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4) void mamba2_step_kernel(
 
 template <class T, int SPEC>
 int launch_mamba2(const Mamba2Params& p, hipStream_t stream) {
-    hipLaunchKernelGGL((mamba2_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p);
+    hipLaunchKernelGGL((mamba2_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
+                       p.rows_per_xcd, p.hv, p.hv_shift, p);
     return int(hipGetLastError());
 }
 

@@ -206,7 +206,7 @@ def test_bench_contract_off_the_gpu():
 
 
 def test_timeline_marks_stay_out_of_the_product_library():
-    """The timeline marks of the workgroup-per-key-head kernel exist only behind -DSQ_TIMELINE: the default build
+    """The timeline marks of the step kernels that carry them exist only behind -DSQ_TIMELINE: the default build
     never passes the define, `--timeline` builds a library and an object directory of their own, and the profiling
     script refuses to run without that library or without a GPU instead of falling back to anything."""
     import subprocess
@@ -216,8 +216,11 @@ def test_timeline_marks_stay_out_of_the_product_library():
     assert '-DSQ_TIMELINE' not in build.HIPCC_FLAGS and build.LIB.endswith('libsqhip.so')
     src = open(os.path.join(root, 'statequant_amd', 'csrc', 'build.py')).read()
     assert "libsqhip_timeline.so" in src and "build_timeline" in src
-    kern = open(os.path.join(root, 'statequant_amd', 'csrc', 'sq_gdn_quad.cuh')).read()
-    assert kern.count('#ifdef SQ_TIMELINE') >= 2 and '#define SQ_MARK(k) do { } while (0)' in kern
+    marks = open(os.path.join(root, 'statequant_amd', 'csrc', 'sq_timeline.cuh')).read()
+    assert marks.count('#ifdef SQ_TIMELINE') == 1 and '#define SQ_MARK(k) do { } while (0)' in marks
+    for name in ('sq_gdn_quad.cuh', 'sq_kda.cuh'):                     # the marked kernels
+        kern = open(os.path.join(root, 'statequant_amd', 'csrc', name)).read()
+        assert '#include "sq_timeline.cuh"' in kern and 'SQ_MARK(0)' in kern and '#ifdef SQ_TIMELINE' in kern
     if not torch.cuda.is_available():
         r = subprocess.run([sys.executable, os.path.join(root, 'profile_timeline.py')], capture_output=True, text=True)
         assert r.returncode != 0 and ('is missing' in r.stderr or 'no GPU visible' in r.stderr), r.stderr
@@ -228,9 +231,12 @@ def test_timeline_marks_stay_out_of_the_product_library():
         with tempfile.TemporaryDirectory() as d:
             unit = os.path.join(d, 'one.hip')
             with open(unit, 'w') as f:
-                f.write('#include "%s"\nnamespace sq {\ntemplate int launch_gdn_quad<Tile<8, 128, 128, 128, true, 8>, 2, '
-                        '2, 4, 1>(const GdnParams&, hipStream_t);\n}\n'
-                        % os.path.join(root, 'statequant_amd', 'csrc', 'sq_gdn_quad.cuh'))
+                csrc = os.path.join(root, 'statequant_amd', 'csrc')
+                f.write('#include "%s"\n#include "%s"\nnamespace sq {\n'
+                        'template int launch_gdn_quad<Tile<8, 128, 128, 128, true, 8>, 2, 2, 4, 1>(const GdnParams&, '
+                        'hipStream_t);\n'
+                        'template int launch_kda<Tile<4, 128, 128, 32, true, 8>, 1>(const KdaParams&, hipStream_t);\n}\n'
+                        % (os.path.join(csrc, 'sq_gdn_quad.cuh'), os.path.join(csrc, 'sq_kda.cuh')))
             r = subprocess.run(['hipcc', *build.HIPCC_FLAGS, '-DSQ_TIMELINE', '--cuda-device-only', '-c', unit, '-o',
                                 os.path.join(d, 'one.o')], capture_output=True, text=True)
             assert r.returncode == 0, r.stderr[-2000:]
