@@ -16,6 +16,10 @@
 //   + N small           N extra one-dword-per-lane loads per wavefront from 64 bytes that the wavefronts of a head
 //                       pair share (cache hits: they add load instructions, hardly any bytes)
 //   resident 4 / CU     40 KB of LDS per workgroup, as the int8 step kernel has: four workgroups per compute unit
+// The last variants read what a KDA step reads of an int4 / group-32 slot (32 heads, 128 x 128, 8 buffer slots of
+// which 4 are live; 509 056 bytes per slot, fields in the reference's order): per head 8 KB of codes, 1 KB of scales,
+// 2 KB of fp32 decays, 512 B of running decay, 512 B each of buffered keys and values, from seven places of the slot
+// -- one wavefront per head as the KDA kernel has it, every load covering consecutive bytes.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -78,6 +82,40 @@ __global__ __launch_bounds__(256) void probe(Args a) {
     if (acc == 0x12345678u) a.sink[blockIdx.x] = acc;        // never true for the buffer's contents: keeps the loads
 }
 
+// KDA: offsets of the fields inside a slot, bytes per head of each
+constexpr size_t KDA_SLOT = 509056, KDA_GB = 0, KDA_GCUR = 131072, KDA_SC = 147584, KDA_S = 181376, KDA_KB = 443520,
+                 KDA_UB = 476288;
+constexpr int KDA_LIVE = 4;
+constexpr double KDA_BYTES = 8192 + 1024 + KDA_LIVE * 512 + 512 + KDA_LIVE * 128 + KDA_LIVE * 128;
+template <bool WIDE>
+__global__ __launch_bounds__(64) void probe_kda(Args a) {
+    const int wg = blockIdx.x;
+    const int tile = (wg & 7) * a.per_xcd + (wg >> 3);
+    const int h = tile & (HEADS - 1), lane = threadIdx.x;
+    const uint8_t* slot = a.base + size_t(a.idx[tile / HEADS]) * KDA_SLOT;
+    uint32_t acc = 0;
+    auto eat = [&](const v4u& x) { acc ^= x.x ^ x.y ^ x.z ^ x.w; };
+    const uint8_t* codes = slot + KDA_S + size_t(h) * 8192;
+    if constexpr (WIDE) {                                    // 1 KB per load
+#pragma unroll
+        for (int j = 0; j < 8; ++j) eat(ld<true>(codes + j * 1024 + lane * 16));
+    } else {                                                 // 512 B per load, as the kernel's row-shaped loads
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            typedef uint32_t v2 __attribute__((ext_vector_type(2)));
+            const v2 x = __builtin_nontemporal_load(reinterpret_cast<const v2*>(codes + j * 512 + lane * 8));
+            acc ^= x.x ^ x.y;
+        }
+    }
+    eat(ld<true>(slot + KDA_SC + size_t(h) * 1024 + lane * 16));
+#pragma unroll
+    for (int j = 0; j < KDA_LIVE / 2; ++j) eat(ld<false>(slot + KDA_GB + size_t(h) * 4096 + j * 1024 + lane * 16));
+    eat(ld<false>(slot + KDA_GCUR + size_t(h) * 512 + (lane & 31) * 16));
+    eat(ld<false>(slot + KDA_KB + size_t(h) * 1024 + (lane & 31) * 16));
+    eat(ld<false>(slot + KDA_UB + size_t(h) * 1024 + (lane & 31) * 16));
+    if (acc == 0x12345678u) a.sink[blockIdx.x] = acc;
+}
+
 // shader clock: the core clock counter against the 100 MHz real-time counter over a streaming read
 __global__ __launch_bounds__(256) void clock_probe(const v4u* src, uint64_t* out, uint32_t* sink, int iters) {
     const uint64_t c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
@@ -111,6 +149,7 @@ struct Variant {
 };
 
 int main() {
+    static_assert(KDA_SLOT <= SLOT_BYTES, "the KDA variants reuse the buffer: slot pitch of the larger layout");
     const size_t per_layer = size_t(SLOTS + 1) * SLOT_BYTES;
     uint8_t* buf;
     uint32_t* sink;
@@ -156,6 +195,28 @@ int main() {
         CHECK(hipEventElapsedTime(&ms, e0, e1));
         const double us = ms * 1e3 / (reps * LAYERS);
         printf("%-34s %7.2f us per launch  %7.1f GB/s\n", v.name, us, code_bytes / us * 1e-3);
+        fflush(stdout);
+    }
+    for (int wide = 0; wide < 2; ++wide) {
+        auto launch = [&](int layer) {
+            Args a{buf + layer * per_layer, idx, sink, TILES / 8};
+            if (wide) hipLaunchKernelGGL(probe_kda<true>, dim3(TILES), dim3(64), 0, 0, a);
+            else hipLaunchKernelGGL(probe_kda<false>, dim3(TILES), dim3(64), 0, 0, a);
+        };
+        for (int r = 0; r < 2; ++r)
+            for (int layer = 0; layer < LAYERS; ++layer) launch(layer);
+        CHECK(hipDeviceSynchronize());
+        const int reps = 10;
+        CHECK(hipEventRecord(e0));
+        for (int r = 0; r < reps; ++r)
+            for (int layer = 0; layer < LAYERS; ++layer) launch(layer);
+        CHECK(hipEventRecord(e1));
+        CHECK(hipEventSynchronize(e1));
+        float ms = 0;
+        CHECK(hipEventElapsedTime(&ms, e0, e1));
+        const double us = ms * 1e3 / (reps * LAYERS);
+        printf("%-34s %7.2f us per launch  %7.1f GB/s\n", wide ? "kda fields, 1 KB code loads" : "kda fields, 512 B code loads", us,
+               KDA_BYTES * TILES / us * 1e-3);
         fflush(stdout);
     }
     {
