@@ -24,5 +24,9 @@ How it is pinned (see tests/test_oracle_*.py; gga.py states its own pins in its 
     format's closed form on the reference tests' edge cases (all-zero groups, scales in the fp16 subnormal range,
     ragged last group); the step algebra with an fp32 state and fp32 buffer against the textbook recurrences; the
     m = 1 special case against per-token rounding of the textbook update; ``read`` + one textbook step against the
-    next packed step; the byte layout against the reference's documented per-slot totals.
+    next packed step; the byte layout against the reference's documented per-slot totals;
+  * the stand-alone helpers that no golden record exercises -- ``gdn_gate``, ``GGAState.gate`` and the one-step
+    textbook recurrences ``gdn_recurrence`` / ``kda_recurrence`` / ``mamba2_recurrence`` -- against torch's library
+    softplus / sigmoid and float64 NumPy recurrences on inputs either side of the softplus threshold, with non-zero
+    A_log / dt_bias, dt limits and the D term (tests/test_oracle_math_cpu.py).
 """

@@ -93,3 +93,138 @@ def test_mamba2_identity_oracle_is_the_ssd_recurrence(h, g_, dk, dv, m):
     assert worst < 1e-5, worst
     st = np.abs(f64(ora.state()) - S).max() / np.abs(S).max()
     assert st < 1e-5, st
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The stand-alone helpers the GPU tests check against: the gates and the three one-line textbook recurrences.
+# Each is compared with an independent formulation (torch's library softplus / sigmoid for the gates, float64 numpy
+# for the recurrences), on inputs chosen so that a dropped term, a wrong sign or a wrong threshold fails.
+# ---------------------------------------------------------------------------------------------------------------
+def _gate_inputs():
+    gen = torch.Generator().manual_seed(11)
+    hv = 6
+    # a + dt_bias on both sides of softplus' pass-through threshold (20), large negatives, and exactly 20
+    a = torch.tensor([-30.0, -3.0, 0.0, 2.5, 19.0, 19.999, 20.0, 20.001, 21.0, 35.0])[:, None].repeat(1, hv)
+    a = a + torch.randn(a.shape, generator=gen) * 1e-3
+    a[6] = 20.0
+    dt_bias = torch.tensor([0.0, 0.75, -1.5, 3.0, -0.25, 1.0])
+    a[6] = a[6] - dt_bias                                      # row 6: a + dt_bias == 20 exactly (<= branch)
+    b = torch.randn(a.shape, generator=gen) * 3
+    A_log = torch.tensor([-2.0, -0.5, 0.0, 0.3, 1.0, 2.0])
+    return a, b, A_log, dt_bias
+
+
+def test_gdn_gate_is_minus_exp_A_softplus_and_sigmoid():
+    """_fused_triton.py:96-100 / families.py:195-202 there: g = -exp(A_log) softplus(a + dt_bias) with softplus
+    passed through above 20, beta = sigmoid(b)."""
+    a, b, A_log, dt_bias = _gate_inputs()
+    g, beta = ST.gdn_gate(a, b, A_log, dt_bias)
+    sp = torch.nn.functional.softplus(a + dt_bias, beta=1.0, threshold=20.0)
+    want = -torch.exp(A_log) * sp
+    assert g.shape == a.shape and beta.shape == b.shape
+    # the reference's device code forms log(1 + exp(x)) in fp32 as written: 1 + exp(x) is rounded to 2^-24, so the
+    # comparison with the library softplus carries an absolute term of that size (times exp(A_log))
+    assert ((g - want).abs() <= 2e-6 * want.abs() + 1.5e-7 * torch.exp(A_log)).all()
+    assert torch.allclose(beta, torch.sigmoid(b), rtol=1e-6, atol=0)
+    # float64, written out: the threshold matters (softplus(21) != 21 by 7.6e-10 -- invisible -- but the sign, the
+    # exp(A_log) factor and dt_bias are not)
+    x = f64(a) + f64(dt_bias)[None]
+    want64 = -np.exp(f64(A_log))[None] * np.where(x <= 20.0, np.log1p(np.exp(x)), x)
+    assert np.abs(f64(g) - want64).max() / np.abs(want64).max() < 1e-6
+    assert (g <= 0).all() and (g[1:] < 0).all()
+    row = f64(g)[6] / -np.exp(f64(A_log))                    # x = 20: both branches agree to 1e-10
+    assert np.allclose(row, np.log1p(np.exp(20.0)), rtol=1e-6)
+    # each ingredient is live: dropping dt_bias / A_log or flipping the sign moves the result far past the bound
+    for wrong in (ST.gdn_gate(a, b, A_log, torch.zeros_like(dt_bias))[0],
+                  ST.gdn_gate(a, b, torch.zeros_like(A_log), dt_bias)[0], -g):
+        assert np.abs(f64(wrong) - want64).max() / np.abs(want64).max() > 1e-2
+
+
+def test_gga_gate_with_nonzero_parameters():
+    """vllm_gga.py's gate there (the same formula as the GDN one, with torch's default softplus threshold 20)."""
+    from oracle import gga as G
+    a, b, A_log, dt_bias = _gate_inputs()
+    g, beta = G.GGAState.gate(a, b, A_log, dt_bias)
+    x = f64(a) + f64(dt_bias)[None]
+    want64 = -np.exp(f64(A_log))[None] * np.where(x <= 20.0, np.log1p(np.exp(x)), x)
+    assert np.abs(f64(g) - want64).max() / np.abs(want64).max() < 1e-6
+    assert np.abs(f64(beta) - 1.0 / (1.0 + np.exp(-f64(b)))).max() < 1e-6
+    g2, beta2 = ST.gdn_gate(a, b, A_log, dt_bias)
+    assert torch.allclose(g, g2, rtol=2e-6, atol=1e-6) and torch.allclose(beta, beta2, rtol=1e-6, atol=0)
+    assert np.abs(f64(G.GGAState.gate(a, b, A_log, torch.zeros_like(dt_bias))[0]) - want64).max() > 1e-2
+
+
+def test_gdn_recurrence_is_the_gated_delta_rule():
+    """kda.py:44-52 there with a scalar decay, per head; q scaled, q / k l2-normalised with eps inside the root."""
+    gen = torch.Generator().manual_seed(12)
+    BH, dk, dv, scale = 6, 48, 80, 0.37
+    S0 = torch.randn(BH, dv, dk, generator=gen)
+    S_t, S = S0.clone(), f64(S0)
+    for _ in range(5):
+        q, k = torch.randn(BH, dk, generator=gen) * 3, torch.randn(BH, dk, generator=gen) * 0.2
+        v = torch.randn(BH, dv, generator=gen)
+        g, beta = -torch.rand(BH, generator=gen) * 2, torch.rand(BH, generator=gen)
+        o = ST.gdn_recurrence(S_t, q, k, v, g, beta, scale)
+        qn, kn = l2n(f64(q)) * scale, l2n(f64(k))
+        S = S * np.exp(f64(g))[:, None, None]
+        u = f64(beta)[:, None] * (f64(v) - np.einsum('bvk,bk->bv', S, kn))
+        S = S + u[:, :, None] * kn[:, None, :]
+        want = np.einsum('bvk,bk->bv', S, qn)
+        assert np.abs(f64(o) - want).max() / np.abs(want).max() < 1e-5
+        assert np.abs(f64(S_t) - S).max() / np.abs(S).max() < 1e-5
+
+
+def test_kda_recurrence_is_the_per_channel_delta_rule():
+    """kda.py:44-52 there: one decay per key channel, default scale d_k^-1/2."""
+    gen = torch.Generator().manual_seed(13)
+    BH, dk, dv = 5, 64, 32
+    S0 = torch.randn(BH, dv, dk, generator=gen)
+    for scale in (None, 0.61):
+        S_t, S = S0.clone(), f64(S0)
+        for _ in range(5):
+            q, k = torch.randn(BH, dk, generator=gen) * 2, torch.randn(BH, dk, generator=gen)
+            v = torch.randn(BH, dv, generator=gen)
+            g = -torch.nn.functional.softplus(torch.randn(BH, dk, generator=gen) * 2)
+            beta = torch.rand(BH, generator=gen)
+            o = ST.kda_recurrence(S_t, q, k, v, g, beta, scale)
+            qn, kn = l2n(f64(q)) * (dk ** -0.5 if scale is None else scale), l2n(f64(k))
+            S = S * np.exp(f64(g))[:, None, :]
+            u = f64(beta)[:, None] * (f64(v) - np.einsum('bvk,bk->bv', S, kn))
+            S = S + u[:, :, None] * kn[:, None, :]
+            want = np.einsum('bvk,bk->bv', S, qn)
+            assert np.abs(f64(o) - want).max() / np.abs(want).max() < 1e-5
+            assert np.abs(f64(S_t) - S).max() / np.abs(S).max() < 1e-5
+
+
+@pytest.mark.parametrize('softplus,limit,with_D,with_bias', [(True, None, True, True), (False, None, False, False),
+                                                             (True, (0.05, 0.2), True, False)])
+def test_mamba2_recurrence_is_the_ssd_step(softplus, limit, with_D, with_bias):
+    """mamba2.py:57-70 with the gate of mamba2.py:45-54 there: dt (+ bias) -> softplus above-20 pass-through ->
+    clamp; S <- exp(A dt) S + (dt x) B^T; y = S C (+ D x); B / C shared by the heads of a group."""
+    gen = torch.Generator().manual_seed(14)
+    Bsz, H, G_, dk, dv = 2, 6, 2, 32, 24
+    S0 = torch.randn(Bsz, H, dv, dk, generator=gen)
+    S_t, S = S0.clone(), f64(S0)
+    A = -torch.exp(torch.rand(H, generator=gen) * 2)
+    D = torch.randn(H, generator=gen) if with_D else None
+    dtb = torch.randn(H, generator=gen) * 0.5 if with_bias else None
+    for t in range(5):
+        x = torch.randn(Bsz, H, dv, generator=gen)
+        dt = torch.randn(Bsz, H, generator=gen) * 0.5 - 2 if softplus else torch.rand(Bsz, H, generator=gen) * 0.3
+        if softplus and t == 2:
+            dt[0, 0] = 25.0                                   # above the softplus threshold
+        Bm, Cm = torch.randn(Bsz, G_, dk, generator=gen), torch.randn(Bsz, G_, dk, generator=gen)
+        y = ST.mamba2_recurrence(S_t, x, dt, Bm, Cm, A, D, dtb, softplus, limit)
+        d = f64(dt) + (f64(dtb)[None] if with_bias else 0.0)
+        if softplus:
+            d = np.where(d <= 20.0, np.log1p(np.exp(d)), d)
+        if limit is not None:
+            d = np.clip(d, *limit)
+        Bh, Ch = np.repeat(f64(Bm), H // G_, axis=1), np.repeat(f64(Cm), H // G_, axis=1)
+        S = S * np.exp(d * f64(A)[None])[..., None, None]
+        S = S + (d[..., None] * f64(x))[..., :, None] * Bh[..., None, :]
+        want = np.einsum('bhvk,bhk->bhv', S, Ch)
+        if with_D:
+            want = want + f64(D)[None, :, None] * f64(x)
+        assert np.abs(f64(y) - want).max() / np.abs(want).max() < 1e-5
+        assert np.abs(f64(S_t) - S).max() / np.abs(S).max() < 1e-5
