@@ -11,10 +11,14 @@ state and advance in lockstep, so one step in m folds and re-quantizes every sta
 the same: benchmarks/decode_state.py:41-66 there times graphs of m steps = one fold).
 
 Timing: whole fold periods only.  K and W are rounded up to multiples of m (``config.steps_requested`` keeps K;
-``steps`` is what was timed), so every timed window holds exactly steps / m folds whatever K is; W untimed warm-up
-steps, then the timed steps between ``torch.cuda.synchronize()`` calls on the wall clock (``ms_per_step``), with HIP
-events on the launch stream around the same region.  The steps are replayed from a HIP graph of m steps (m x 24
-kernel nodes) unless ``--no-graph``.
+``steps`` is what was timed), so every timed window holds exactly steps / m folds whatever K is.  The steps are
+replayed from a HIP graph of m steps (m x 24 kernel nodes) unless ``--no-graph``.  Warm-up: one eager period, the
+capture, and then at least MIN_WARM_PERIODS untimed replays of the graph whatever W says (``warmup`` in the line is
+what was run: the first replay of a graph uploads it, and the clocks need a few milliseconds of load to settle), then
+the timed periods between ``torch.cuda.synchronize()`` calls on the wall clock (``ms_per_step``, ``value``).  Every
+timed period also has its own pair of HIP events on the launch stream: ``per_period_us`` lists them (microseconds per
+launch), ``period_us`` holds their min / median / mean (the reference's benchmark reports the minimum over repeats of
+the same graph, benchmarks/decode_state.py:41-66 there), and ``roofline`` is priced on their mean.
 
 Prints ONE JSON line.  ``value`` = microseconds per layer per decode step (lower is better).  ``roofline`` prices the
 step kernel against HBM: achieved = algorithmic state bytes per launch / average launch duration, where the
@@ -30,10 +34,7 @@ targets.
 Secondary figures: ``--workload`` (the other formats and families; ``gga4-pw8`` is the mixed-width GGA / STEP slot,
 which re-fits every head at every token), ``--slots N`` (other batch sizes), ``--op write |
 read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots)
-with or without ``--fold-first`` (the step calls' optional dispatch order, folding rows first), ``--calibrate-copy``
-(the known-size copy that the HBM counters are scaled by), ``--calibrate-stream`` (runs the stand-alone probe
-``statequant_amd/probe_stream``, built by ``python -m statequant_amd.csrc.build --probes``: the rate at which kernels
-that do nothing else read a layer step's codes through the slot index, i.e. the ceiling of this access pattern).
+and ``--calibrate-copy`` (the known-size copy that the HBM counters are scaled by).
 """
 import argparse
 import json
@@ -47,6 +48,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MIN_WARM_PERIODS = 8           # untimed graph replays before the clock starts (about 50 ms at the headline)
+MAX_LISTED_PERIODS = 128       # per_period_us lists at most this many (the statistics use all)
 
 WORKLOADS = {
     # name: (family, bits, group, hv, hk, dk, dv, slots, layers); group < 0: value-axis groups of -group rows;
@@ -162,15 +165,40 @@ def make_inputs(fam, lay, slots, layers, m, device, seed=1):
     return out, extra
 
 
-def launch(fam, lay, views, idx, inp, extra, out, order=None):
+def launch(fam, lay, views, idx, inp, extra, out):
     if fam == 'gdn':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'],
-                 order=order)
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'])
     elif fam == 'kda':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out, order=order)
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out)
     else:
-        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'],
-                 order=order)
+        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'])
+
+
+def timed_periods(stream, run_period, warm_periods, periods):
+    """`warm_periods` untimed calls of `run_period()`, then `periods` timed ones on `stream`: the wall clock around
+    all of them between device synchronisations, and one HIP event between every two periods.  Returns (wall seconds,
+    [milliseconds of each period])."""
+    for _ in range(warm_periods):
+        run_period()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(periods + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record(stream)
+    for i in range(periods):
+        run_period()
+        ev[i + 1].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, [ev[i].elapsed_time(ev[i + 1]) for i in range(periods)]
+
+
+def period_stats(per_ms, launches_per_period):
+    """Per-launch microseconds of every timed period and their min / median / mean."""
+    us = sorted(x * 1e3 / launches_per_period for x in per_ms)
+    n = len(us)
+    med = us[n // 2] if n % 2 else 0.5 * (us[n // 2 - 1] + us[n // 2])
+    listed = [round(x * 1e3 / launches_per_period, 3) for x in per_ms[:MAX_LISTED_PERIODS]]
+    return listed, {'min': round(us[0], 3), 'median': round(med, 3), 'mean': round(sum(us) / n, 3), 'periods': n}
 
 
 def cpu_baseline(workload, m, budget_s=20.0):
@@ -282,7 +310,6 @@ def bench_gga(a, dev):
 
     requested = (a.steps, a.warmup)
     a.steps = max(-(-a.steps // period_len), 1) * period_len          # whole graphs of period_len steps
-    a.warmup = -(-a.warmup // period_len) * period_len
     use_graph = not a.no_graph
     torch.cuda.synchronize()                                # states and inputs were made on the default stream
     stream = torch.cuda.Stream()
@@ -293,22 +320,17 @@ def bench_gga(a, dev):
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 period()
-            run = lambda n: [graph.replay() for _ in range(n // period_len)]          # noqa: E731
+            run_period = graph.replay
         else:
-            run = lambda n: [period() for _ in range(-(-n // period_len))]            # noqa: E731
-        run(max(a.warmup - period_len, 0))
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
-        run(a.steps)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+            run_period = period
+        warm = max(-(-a.warmup // period_len) - 1, 2)
+        wall, per_ms = timed_periods(stream, run_period, warm, a.steps // period_len)
+    a.warmup = (warm + 1) * period_len
+    per_period_us, pstats = period_stats(per_ms, period_len * layers)
     steps = a.steps
     assert torch.isfinite(out.float()).all(), 'non-finite output'
     n_launch = steps * layers
-    us_wall, us_kernel = wall * 1e6 / n_launch, e0.elapsed_time(e1) * 1e3 / n_launch
+    us_wall, us_kernel = wall * 1e6 / n_launch, sum(per_ms) * 1e3 / n_launch
     alg = sum(gga_bytes_per_slot_step(pk, L) for L in range(layers)) / layers * slots
     achieved = alg / (us_kernel * 1e-6) / 1e9
     res = {
@@ -324,6 +346,7 @@ def bench_gga(a, dev):
                    'bytes_per_slot': pk.nbytes,
                    'algorithmic_bytes_per_slot_step': round(alg / slots)},
         'hbm_gbs': round(achieved, 1),
+        'period_us': pstats, 'per_period_us': per_period_us,
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': measured_traffic(a.workload),
                      'traffic_source': 'profiles/hbm_traffic.json (rocprofv3 run of profile_step.py, not this run)',
@@ -378,26 +401,6 @@ def calibrate_copy(dev, nbytes=1 << 30, reps=20):
                       'us_per_copy': round(us, 2), 'gbs_read_plus_write': round(2 * nbytes / us * 1e-3, 1)}))
 
 
-def calibrate_stream():
-    """Run the memory-system probe (csrc/probe_stream.hip) as a child process and print its figures as one JSON line."""
-    import subprocess
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'statequant_amd', 'probe_stream')
-    if not os.path.exists(exe):
-        sys.exit(f'bench.py: {exe} is missing; build it with `python -m statequant_amd.csrc.build --probes`')
-    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
-    if r.returncode:
-        sys.exit(f'bench.py: {exe} failed:\n{r.stdout}\n{r.stderr}')
-    rows, clock = {}, None
-    for line in r.stdout.splitlines():
-        if 'us per launch' in line:
-            name, rest = line[:34].strip(), line[34:].split()
-            rows[name] = {'us_per_launch': float(rest[0]), 'gbs': float(rest[4])}
-        elif 'shader clock' in line:
-            clock = float(line.split()[-2])
-    print(json.dumps({'calibrate_stream': True, 'codes_bytes_per_launch': 8192 * 16384, 'variants': rows,
-                      'shader_clock_mhz': clock}))
-
-
 def bench_convert(a, lay, views, idx, dev):
     """`SlotLayout.write` (fp32 state -> codes + scales, buffers emptied) or `.read` (stored state advanced across
     the pending buffer -> fp32) over all slots of every layer blob; one launch per layer.  Algorithmic bytes: the fp32
@@ -448,10 +451,6 @@ def main():
     ap.add_argument('--warmup', type=int, default=512)
     ap.add_argument('--workload', default='gdn-int8-g128', choices=list(WORKLOADS))
     ap.add_argument('--m', type=int, default=8)
-    ap.add_argument('--fold-first', action='store_true',
-                    help='hand every launch a dispatch order with the rows that fold on this step first '
-                         '(SlotLayout.fold_first, computed once per step from the first layer\'s counters, inside the '
-                         'timed region); meant for --mixed-fill')
     ap.add_argument('--slots', type=int, default=None,
                     help='number of sequences instead of the workload\'s own (the reference quotes batch 128 and 512)')
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
@@ -467,9 +466,6 @@ def main():
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='instead of the workload, run plain device copies of 1 GiB (the known-size kernel that '
                          'rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by) and print their rate')
-    ap.add_argument('--calibrate-stream', action='store_true',
-                    help='instead of the workload, run statequant_amd/probe_stream (read-only kernels over the codes '
-                         'of a layer step: the ceiling of the access pattern) and print its figures')
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit('bench.py: this build measures one GPU; the decode step has no cross-GPU exchange (slots shard '
@@ -480,8 +476,6 @@ def main():
     torch.cuda.set_device(dev)
     if a.calibrate_copy:
         return calibrate_copy(dev)
-    if a.calibrate_stream:
-        return calibrate_stream()
     m = a.m
     if a.slots:
         w = WORKLOADS[a.workload]
@@ -501,42 +495,29 @@ def main():
 
     def period():                                           # m steps x layers launches
         for s in range(m):
-            order = lay.fold_first(views[0], idx) if a.fold_first else None
             for L in range(layers):
-                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out, order)
+                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out)
 
     requested = (a.steps, a.warmup)
     a.steps = max(-(-a.steps // m), 1) * m                  # whole fold periods, so that any K times steps / m folds
-    a.warmup = -(-a.warmup // m) * m
     use_graph = not a.no_graph
     torch.cuda.synchronize()                                # states and inputs were made on the default stream
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
+        period()                                            # one eager period first (module load etc.)
+        stream.synchronize()
         if use_graph:
-            period()                                        # one eager period first (module load etc.)
-            stream.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 period()
-            run = lambda n: [graph.replay() for _ in range(n // m)]          # noqa: E731
-            done = m
+            run_period = graph.replay
         else:
-            def run(n):
-                for s in range(n):
-                    order = lay.fold_first(views[0], idx) if a.fold_first else None
-                    for L in range(layers):
-                        launch(fam, lay, views[L], idx, inputs[(s % m) * layers + L], extra, out, order)
-            done = 0
-        run(max(a.warmup - done, 0))
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
-        run(a.steps)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-    ev_ms = e0.elapsed_time(e1)
+            run_period = period
+        warm = max(-(-a.warmup // m) - 1, MIN_WARM_PERIODS)  # untimed periods on the timed path itself
+        wall, per_ms = timed_periods(stream, run_period, warm, a.steps // m)
+    a.warmup = (warm + 1) * m                               # steps run before the clock started
+    ev_ms = sum(per_ms)
+    per_period_us, pstats = period_stats(per_ms, m * layers)
     assert torch.isfinite(out.float()).all(), 'non-finite output'
     n_launch = a.steps * layers
     us_wall = wall * 1e6 / n_launch
@@ -555,9 +536,9 @@ def main():
                    'steps_requested': requested[0], 'warmup_requested': requested[1], 'steps_timed': a.steps,
                    'folds_timed': a.steps // m if not a.mixed_fill else None,
                    'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
-                   'dispatch_order': 'folding rows first' if a.fold_first else 'natural',
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),
+        'period_us': pstats, 'per_period_us': per_period_us,
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': measured_traffic(a.workload),
                      'traffic_source': 'profiles/hbm_traffic.json (rocprofv3 run of profile_step.py, not this run)',

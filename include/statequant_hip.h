@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 4
+#define SQ_ABI_VERSION 5
 
 enum { SQ_F32 = 0, SQ_BF16 = 1, SQ_F16 = 2 };                /* dtype codes of float tensors */
 
@@ -99,12 +99,6 @@ typedef struct sq_gdn_args {
     const void* dt_bias; int32_t dt_bias_dtype;
     void* out;          int32_t out_dtype;
     float scale;
-    /* Optional dispatch order of the batch rows: a priority list, earlier entries start earlier (a permutation of
-     * 0 .. rows-1, dealt round-robin to the GPU's eight dies; NULL: the natural order).  Results do not depend on it.
-     * No counterpart in the reference: a scheduling hint for batches whose sequences fill their buffers on different
-     * steps -- the rows that fold on this step take 2.5 x as long, and started first they do not set the end of the
-     * launch.  sq_fold_first() writes such a list. */
-    const int32_t* order;
 } sq_gdn_args;
 
 /* One KDA decode token per batch row (kda.py:192-205, 330-347): per-key-channel log decay g [rows, hv, dk];
@@ -121,7 +115,6 @@ typedef struct sq_kda_args {
     const void* beta;   int64_t s_beta;  int32_t beta_dtype;
     void* out;          int64_t s_out;   int32_t out_dtype;
     float scale;
-    const int32_t* order;   /* optional dispatch order of the rows, as in sq_gdn_args */
 } sq_kda_args;
 
 /* One Mamba2 / SSD decode token per batch row (mamba2.py:223-241, 377-396).
@@ -143,7 +136,6 @@ typedef struct sq_mamba2_args {
     int32_t dt_softplus;
     int32_t dt_clamp;   float dt_min, dt_max;
     void* out;          int64_t s_out;   int32_t out_dtype;
-    const int32_t* order;   /* optional dispatch order of the rows, as in sq_gdn_args */
 } sq_mamba2_args;
 
 /* Store fp32 states in the packed format (fold.py:123-147 `pack_vk`; with idx, GCUR and NPTR given this is
@@ -220,6 +212,14 @@ int sq_abi_version(void);
 const char* sq_strerror(int code);
 const char* sq_last_error(void);
 
+/* Diagnostic, no counterpart in the reference: several compiled kernel instances can serve the same step call (one
+ * with the serving dtypes compiled in or the general one; a workgroup per key head or a wavefront per head; how many
+ * value heads a workgroup takes).  Results do not depend on the choice up to the accumulation order of fp32 sums; the
+ * twin tests and the profiling scripts use this to compare instances.  Non-zero no_specialised / no_group_kernel
+ * exclude those instances, max_heads_per_workgroup <= 0 means no cap.  Process-wide, takes effect on the next call;
+ * the library never reads the environment for it.  Pure host code. */
+void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup);
+
 /* 1 if a kernel is built for this layout (family: 0 GDN, 1 KDA, 2 Mamba2), else 0. Pure host code. */
 int sq_supported(int family, const sq_layout* lay);
 
@@ -227,12 +227,6 @@ int sq_gdn_step(const sq_gdn_args* args, void* stream);
 int sq_kda_step(const sq_kda_args* args, void* stream);
 int sq_mamba2_step(const sq_mamba2_args* args, void* stream);
 int sq_pack_vk(const sq_pack_args* args, void* stream);
-/* order[0 .. rows) <- the rows of `idx` whose buffer fills on the coming step (NPTR[idx[b] * sN] & (m-1) == m-1) first,
- * the other live rows next, padding rows (idx[b] <= 0) last; for the step calls' `order`.  One small launch; the
- * counters of all layers of a model move together, so one list per decode step serves every layer.  No counterpart in
- * the reference. */
-int sq_fold_first(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m, int32_t rows, int32_t* order,
-                  void* stream);
 int sq_read(const sq_read_args* args, void* stream);
 int sq_gga_step(const sq_gga_args* args, void* stream);
 /* Fit + pack canonical fp32 states X [rows, hv, dk, dv] (key-major, contiguous) into slots idx[b]; their counters are

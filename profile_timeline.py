@@ -58,9 +58,11 @@ def timeline(workload, step, dev, m=8):
     for s in range(step):
         run(s, layers)
     run(step, layers - 1)
-    os.environ['SQ_TIMELINE_BUF'] = str(buf.data_ptr())      # read by the library at launch
-    bench.launch(fam, lay, views[layers - 1], idx, inputs[step * layers + layers - 1], extra, out)
-    del os.environ['SQ_TIMELINE_BUF']
+    os.environ['SQ_TIMELINE_BUF'] = f'{buf.data_ptr()}:{nwg * waves}'   # address : capacity in wavefronts, read at launch
+    try:
+        bench.launch(fam, lay, views[layers - 1], idx, inputs[step * layers + layers - 1], extra, out)
+    finally:
+        del os.environ['SQ_TIMELINE_BUF']
     torch.cuda.synchronize()
     t = buf.cpu().numpy().reshape(nwg, waves, 16)[:, :, :15].astype(np.float64)
     if not (t[:, :, 0] > 0).all():

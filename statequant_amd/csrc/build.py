@@ -1,6 +1,6 @@
 """Build libsqhip.so (the C-ABI library of include/statequant_hip.h) for gfx950 with hipcc.
 
-    python -m statequant_amd.csrc.build [-j N] [--force] [--timeline] [--probes]
+    python -m statequant_amd.csrc.build [-j N] [--force] [--timeline] [--resources [PATTERN]]
 
 The step kernels are templates on (bits, d_k, d_v, group, int8-buffer, max m).  ``CASES`` below lists the instances
 that are compiled; this script writes one small translation unit per chunk of instances plus the dispatch table into
@@ -205,12 +205,15 @@ def generate():
                       + ''.join(f'template int launch_gga<GgaTile<{dk}, {dv}>>(const GgaParams&, int, hipStream_t);\n'
                                 for dk, dv in GGA_SHAPES) + '}\n')
     units.append(path)
-    d = ['// generated by build.py: layout -> compiled kernel instance', '#include <stdlib.h>', '#include "../sq_convert.cuh"',
+    d = ['// generated by build.py: layout -> compiled kernel instance', '#include <atomic>', '#include "../sq_convert.cuh"',
          'namespace sq {',
-         'int launch_fold_first(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,',
-         '                      hipStream_t stream) {',
-         '    hipLaunchKernelGGL(fold_first_kernel<FF_THREADS>, dim3(1), dim3(FF_THREADS), 0, stream, idx, NPTR, sN, m, rows, order);',
-         '    return int(hipGetLastError());',
+         '// Which instance serves a call when several could (results do not depend on it): set through sq_debug_select,',
+         '// never read from the environment.',
+         'static std::atomic<int> g_no_spec{0}, g_no_quad{0}, g_ghmax{64};',
+         'void select_instances(int no_spec, int no_quad, int ghmax) {',
+         '    g_no_spec.store(no_spec != 0);',
+         '    g_no_quad.store(no_quad != 0);',
+         '    g_ghmax.store(ghmax > 0 ? ghmax : 64);',
          '}']
     for fam, rows in CASES.items():
         P = PARAMS[fam]
@@ -219,10 +222,10 @@ def generate():
             d.append(f'template <class T, int NB, int GH, int WPE, int SPEC> int launch_{fam}_quad(const {P}&, hipStream_t);')
             d += QUAD_OK[fam]
         d.append(f'int dispatch_{fam}(const {P}& p, hipStream_t stream, bool run) {{')
-        d.append('    const int spec = (run && !getenv("SQ_NO_SPEC")) ? serving_case(p) : 0;')
+        d.append('    const int spec = (run && !g_no_spec.load(std::memory_order_relaxed)) ? serving_case(p) : 0;')
         if fam in QUAD_FAMILIES:
-            d.append(f'    const bool quad = !getenv("SQ_NO_QUAD") && (!run || {fam}_quad_ok(p));')
-            d.append('    const int ghmax = getenv("SQ_GHMAX") ? atoi(getenv("SQ_GHMAX")) : 64;')
+            d.append(f'    const bool quad = !g_no_quad.load(std::memory_order_relaxed) && (!run || {fam}_quad_ok(p));')
+            d.append('    const int ghmax = g_ghmax.load(std::memory_order_relaxed);')
         # smallest sufficient buffer bound first
         for c in sorted(rows, key=lambda c: c[5]):
             bits, dk, dv, group, qbuf, mmax, axv = c
@@ -337,19 +340,6 @@ def build(jobs=None, force=False, verbose=True):
     return LIB
 
 
-def build_probes(verbose=True):
-    """Compile the stand-alone memory-system probe (probe_stream.hip) next to the library; returns its path."""
-    exe = os.path.join(PKG, 'probe_stream')
-    cmd = ['hipcc', '--offload-arch=' + ARCH, '-O3', '-std=c++17', '-Wno-unused-result',
-           os.path.join(HERE, 'probe_stream.hip'), '-o', exe]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode:
-        raise RuntimeError(f'{" ".join(cmd)}\n{r.stdout}\n{r.stderr}')
-    if verbose:
-        print(f'[build] wrote {exe}')
-    return exe
-
-
 _REMARK = re.compile(r'remark: +(Function Name|VGPRs|AGPRs|SGPRs Spill|VGPRs Spill|ScratchSize \[bytes/lane\]|'
                      r'Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]): +(\S+)')
 
@@ -398,17 +388,7 @@ if __name__ == '__main__':
     ap.add_argument('--resources', metavar='PATTERN', nargs='?', const='', default=None,
                     help="instead of building, print the compiler's resource usage (registers, spills, LDS, "
                          'occupancy) of every kernel whose name contains PATTERN')
-    ap.add_argument('--probes', action='store_true',
-                    help='build statequant_amd/probe_stream instead (probe_stream.hip: how fast the codes of a layer '
-                         'step can be read by kernels that do nothing else; bench.py --calibrate-stream runs it)')
     a = ap.parse_args()
-    if a.probes:
-        try:
-            build_probes()
-        except RuntimeError as e:
-            print(e, file=sys.stderr)
-            sys.exit(1)
-        sys.exit(0)
     if a.timeline:
         OUT = os.path.join(HERE, 'build_timeline')
         LIB = os.path.join(PKG, 'libsqhip_timeline.so')

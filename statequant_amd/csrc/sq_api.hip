@@ -51,7 +51,6 @@ int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
     key->hv_shift = pow2(L.hv) ? __builtin_ctz(unsigned(L.hv)) : -1;
     key->gqa_shift = pow2(key->gqa) ? __builtin_ctz(unsigned(key->gqa)) : -1;
     key->per_xcd = 0;
-    key->rows_per_xcd = 0;
     return SQ_OK;
 }
 
@@ -59,7 +58,6 @@ int check_layout(const sq_layout& L, const char* who, sq::LayoutKey* key) {
 void set_rows(sq::LayoutKey* key, int rows) {
     const int64_t tiles = int64_t(rows) * key->hv;
     key->per_xcd = (tiles % 8 == 0) ? int(tiles / 8) : 0;
-    key->rows_per_xcd = (rows % 8 == 0) ? rows / 8 : 0;
 }
 
 // A per-sequence or per-row stride as the kernels take it: non-negative, below 2^31.
@@ -118,6 +116,10 @@ int finish(int rc, const char* who, const sq_layout& L) {
 extern "C" {
 
 int sq_abi_version(void) { return SQ_ABI_VERSION; }
+
+void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup) {
+    sq::select_instances(no_specialised, no_group_kernel, max_heads_per_workgroup);
+}
 
 const char* sq_strerror(int code) {
     switch (code) {
@@ -180,7 +182,6 @@ int sq_gdn_step(const sq_gdn_args* a, void* stream) {
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.order = a->order;
     p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
     p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
     p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
@@ -224,7 +225,6 @@ int sq_kda_step(const sq_kda_args* a, void* stream) {
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.order = a->order;
     p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
     p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
     p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
@@ -253,7 +253,6 @@ int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
-    p.order = a->order;
     p.x = a->x; p.s_x = uint32_t(a->s_x); p.x_dt = a->x_dtype;
     p.dt = a->dt; p.s_dt = uint32_t(a->s_dt); p.dt_dt = a->dt_dtype;
     p.B = a->B; p.s_B = uint32_t(a->s_B); p.B_dt = a->B_dtype;
@@ -324,18 +323,6 @@ int sq_read(const sq_read_args* a, void* stream) {
     p.rows = a->rows; p.idx = a->idx;
     p.out = a->out; p.s_out = uint32_t(a->s_out);
     return finish(sq::dispatch_read(p, static_cast<hipStream_t>(stream), true), who, a->lay);
-}
-
-int sq_fold_first(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m, int32_t rows, int32_t* order,
-                  void* stream) {
-    const char* who = "sq_fold_first";
-    if (rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, rows);
-    if (rows == 0) return SQ_OK;
-    if (!idx || !NPTR || !order) return fail(SQ_E_ARG, "%s: null idx / NPTR / order", who);
-    if (!pow2(m) || !stride_ok(sN)) return fail(SQ_E_ARG, "%s: m %d, counter stride %lld", who, m, (long long)sN);
-    const int rc = sq::launch_fold_first(idx, NPTR, uint32_t(sN), m, rows, order, static_cast<hipStream_t>(stream));
-    if (rc) return fail(SQ_E_LAUNCH, "%s: %s", who, hipGetErrorString(hipError_t(rc)));
-    return SQ_OK;
 }
 
 namespace {

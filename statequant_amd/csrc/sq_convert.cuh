@@ -294,44 +294,4 @@ int launch_read(const ReadParams& p, hipStream_t stream) {
     return int(hipGetLastError());
 }
 
-// A dispatch order for the step kernels (their `order` argument): the rows whose buffer fills on the coming step
-// first, the other live rows next, padding rows (slot index <= 0) last; the natural order inside each class.  One
-// workgroup; per class a ballot-and-prefix pass over the rows.  No counterpart in the reference.
-constexpr int FF_THREADS = 256;
-template <int THREADS>                               // (a template only so that the header can hold it)
-__global__ __launch_bounds__(THREADS) void fold_first_kernel(const int32_t* idx, const int32_t* NPTR, uint32_t sN,
-                                                                int m, int rows, int32_t* order) {
-    __shared__ int wave_count[THREADS / WAVE];
-    __shared__ int base;
-    const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
-    if (tid == 0) base = 0;
-    __syncthreads();
-    for (int cls = 0; cls < 3; ++cls) {
-        for (int r0 = 0; r0 < rows; r0 += THREADS) {
-            const int r = r0 + tid;
-            bool mine = false;
-            if (r < rows) {
-                const int32_t slot = idx[r];
-                int c = 2;
-                if (slot > 0) c = ((NPTR[uint64_t(uint32_t(slot)) * sN] & (m - 1)) == m - 1) ? 0 : 1;
-                mine = c == cls;
-            }
-            const unsigned long long bal = __ballot(mine);
-            const int before = __popcll(bal & ((1ull << lane) - 1ull));
-            if (lane == 0) wave_count[wv] = __popcll(bal);
-            __syncthreads();
-            int off = base;
-            for (int w = 0; w < wv; ++w) off += wave_count[w];
-            if (mine) order[off + before] = r;
-            __syncthreads();
-            if (tid == 0) {
-                int tot = 0;
-                for (int w = 0; w < THREADS / WAVE; ++w) tot += wave_count[w];
-                base += tot;
-            }
-            __syncthreads();
-        }
-    }
-}
-
 }  // namespace sq

@@ -69,12 +69,12 @@ struct GdnLoads {
 };
 
 // SPEC > 0 compiles the serving cases in, so that dtypes and options cost no scalar branches on the way to the first
-// load (measured on the 128 x 128 int8 step: 35.4 -> 34.2 us per launch): bf16 q / k / v / out, no dispatch order,
+// load (measured on the 128 x 128 int8 step: 35.4 -> 34.2 us per launch): bf16 q / k / v / out,
 // head counts that are powers of two, and  1: g and beta given as fp32;  2: the gate formed in the kernel from bf16
 // a, b and fp32 A_log, dt_bias.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd, int hv, int hv_shift,
+void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift,
                      SQ_TL_PARAM const GdnParams p) {
     SQ_MARK(0);                                                   // entry
     // the leading arguments (copies of fields of `p`) are what the slot index load needs: as separate scalar
@@ -121,14 +121,6 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict_
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
         tid.b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
         tid.h = (item - tid.b * ngrp) * GH + hl;
-        if (!FIX && order) {
-            int pos = tid.b;
-            if (rows_per_xcd) {
-                const int x = pos / rows_per_xcd;
-                pos = (pos - x * rows_per_xcd) * 8 + x;
-            }
-            tid.b = order[pos];
-        }
         SQ_MARK(1);                                               // item known (the leading arguments are here)
         slot = idx ? idx[tid.b] : tid.b;
         tid.hk = (FIX || p.gqa_shift >= 0) ? tid.h >> p.gqa_shift : tid.h / p.gqa;
@@ -542,14 +534,13 @@ template <class T, int NB, int GH, int WPE, int SPEC>
 int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     GdnParams p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
-    if (p.per_xcd == 0) p.rows_per_xcd = 0;
 #ifdef SQ_TIMELINE
-    uint64_t* tl = sq_timeline_buffer();
+    const SqTimelineBuf tl = sq_timeline_buffer();
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, tl, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, tl.p, tl.cap, p);
 #else
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p);
 #endif
     return int(hipGetLastError());
 }

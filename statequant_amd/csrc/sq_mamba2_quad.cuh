@@ -27,11 +27,10 @@ struct Mamba2Loads {
 };
 
 // SPEC = 1 compiles the serving case in (as in the Gated DeltaNet kernel): bf16 x / B / C / out, fp32 dt, A, D and
-// dt_bias, no dispatch order, head counts that are powers of two.  SPEC = 0 reads all of it from the arguments.
+// dt_bias, head counts that are powers of two.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int rows_per_xcd, int hv,
-                        int hv_shift, const Mamba2Params p) {
+void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const Mamba2Params p) {
     constexpr bool FIX = SPEC > 0;
     const int x_dt = FIX ? int(BF16) : p.x_dt, B_dt = FIX ? int(BF16) : p.B_dt, C_dt = FIX ? int(BF16) : p.C_dt;
     const int out_dt = FIX ? int(BF16) : p.out_dt, dt_dt = FIX ? int(F32) : p.dt_dt, A_dt = FIX ? int(F32) : p.A_dt;
@@ -70,14 +69,6 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restri
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
         b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
         grp = item - b * ngrp;
-        if (!FIX && order) {
-            int pos = b;
-            if (rows_per_xcd) {
-                const int x = pos / rows_per_xcd;
-                pos = (pos - x * rows_per_xcd) * 8 + x;
-            }
-            b = order[pos];
-        }
         slot = idx ? idx[b] : b;
     }
     const uint32_t h = grp * GH + hl;
@@ -446,9 +437,8 @@ template <class T, int NB, int GH, int WPE, int SPEC>
 int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     Mamba2Params p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
-    if (p.per_xcd == 0) p.rows_per_xcd = 0;
     hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.rows_per_xcd, p.hv, p.hv_shift, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p);
     return int(hipGetLastError());
 }
 

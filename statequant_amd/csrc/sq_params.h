@@ -27,14 +27,12 @@ struct LayoutKey {
     // two (else -1: the kernel divides), and tiles per XCD when the tile count is a multiple of 8 (else 0: no XCD
     // mapping)
     int gqa, hv_shift, gqa_shift, per_xcd;
-    int rows_per_xcd;                             // batch rows per XCD range when those ranges hold whole rows, else 0
 };
 
 struct GdnParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
-    const int32_t* order;                         // optional dispatch order of the rows (null: natural)
     const void *q, *k, *v;
     uint32_t s_q, s_k, s_v;
     int q_dt, k_dt, v_dt;
@@ -52,7 +50,6 @@ struct KdaParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
-    const int32_t* order;
     const void *q, *k, *v, *g, *beta;
     uint32_t s_q, s_k, s_v, s_g, s_beta;
     int q_dt, k_dt, v_dt, g_dt, beta_dt;
@@ -66,7 +63,6 @@ struct Mamba2Params : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
-    const int32_t* order;
     const void *x, *dt, *B, *C, *A, *D, *dt_bias;
     uint32_t s_x, s_dt, s_B, s_C;
     int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
@@ -122,7 +118,7 @@ struct GgaParams {
 };
 
 // The serving cases a step kernel can be compiled for (template argument SPEC; 0 = read every choice from the
-// arguments): bf16 operands and output, no dispatch order, head counts that are powers of two, and per family
+// arguments): bf16 operands and output, head counts that are powers of two, and per family
 //   GDN     1: g and beta given as fp32;  2: the gate formed in the kernel from bf16 a, b and fp32 A_log, dt_bias
 //   KDA     1: fp32 g and beta
 //   Mamba2  1: fp32 dt, A, D, dt_bias
@@ -130,18 +126,18 @@ struct GgaParams {
 // private copy of its arguments with the constants (device), after which the compiler drops the scalar branches on
 // them -- about a microsecond per launch on the 128 x 128 steps.  Dtype codes: 0 fp32, 1 bf16.
 inline int serving_case(const GdnParams& p) {
-    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;
+    if (p.hv_shift < 0 || p.gqa_shift < 0) return 0;
     if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;
     if (!p.gate) return (p.a_dt == 0 && p.bt_dt == 0) ? 1 : 0;
     return (p.a_dt == 1 && p.bt_dt == 1 && p.A_log_dt == 0 && p.dt_bias_dt == 0) ? 2 : 0;
 }
 inline int serving_case(const KdaParams& p) {
-    if (p.order || p.hv_shift < 0) return 0;
+    if (p.hv_shift < 0) return 0;
     if (p.q_dt != 1 || p.k_dt != 1 || p.v_dt != 1 || p.out_dt != 1) return 0;
     return (p.g_dt == 0 && p.beta_dt == 0) ? 1 : 0;
 }
 inline int serving_case(const Mamba2Params& p) {
-    if (p.order || p.hv_shift < 0 || p.gqa_shift < 0) return 0;
+    if (p.hv_shift < 0 || p.gqa_shift < 0) return 0;
     if (p.x_dt != 1 || p.B_dt != 1 || p.C_dt != 1 || p.out_dt != 1) return 0;
     return (p.dt_dt == 0 && p.A_dt == 0 && p.D_dt == 0 && p.dt_bias_dt == 0) ? 1 : 0;
 }
@@ -152,7 +148,6 @@ __device__ __forceinline__ void assume_serving_case(GdnParams& p) {
         p.a_dt = p.bt_dt = SPEC == 1 ? 0 : 1;
         p.A_log_dt = p.dt_bias_dt = 0;
         p.gate = SPEC == 2;
-        p.order = nullptr;
         __builtin_assume(p.hv_shift >= 0);
         __builtin_assume(p.gqa_shift >= 0);
     }
@@ -162,7 +157,6 @@ __device__ __forceinline__ void assume_serving_case(KdaParams& p) {
     if constexpr (SPEC > 0) {
         p.q_dt = p.k_dt = p.v_dt = p.out_dt = 1;
         p.g_dt = p.beta_dt = 0;
-        p.order = nullptr;
         __builtin_assume(p.hv_shift >= 0);
     }
 }
@@ -171,7 +165,6 @@ __device__ __forceinline__ void assume_serving_case(Mamba2Params& p) {
     if constexpr (SPEC > 0) {
         p.x_dt = p.B_dt = p.C_dt = p.out_dt = 1;
         p.dt_dt = p.A_dt = p.D_dt = p.dt_bias_dt = 0;
-        p.order = nullptr;
         __builtin_assume(p.hv_shift >= 0);
         __builtin_assume(p.gqa_shift >= 0);
     }
@@ -182,9 +175,9 @@ int dispatch_gdn(const GdnParams& p, hipStream_t stream, bool run);
 int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
 int dispatch_mamba2(const Mamba2Params& p, hipStream_t stream, bool run);
 int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
-int launch_fold_first(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,
-                      hipStream_t stream);
 int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
 int dispatch_gga(const GgaParams& p, int op, hipStream_t stream, bool run);      // op: 0 step, 1 store, 2 load
+// Diagnostic choice among the instances that can serve a step call (behind sq_debug_select of the C ABI).
+void select_instances(int no_spec, int no_quad, int ghmax);
 
 }  // namespace sq

@@ -133,31 +133,21 @@ __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG
 
 // Which (batch row, value head) a workgroup works on; the caller adds the key head.  Consecutive workgroup ids are
 // dealt round-robin to the 8 XCDs; with `per_xcd` set every XCD walks a contiguous range of tiles, so the heads of one
-// sequence (shared key buffer, neighbouring counters) meet in one L2.  `order` (optional) names the batch row of each
-// position: the caller's order is a priority list, its entries are dealt round-robin to the XCDs' row ranges, so that
-// every XCD starts with its share of the first entries.
+// sequence (shared key buffer, neighbouring counters) meet in one L2.
 // The arguments are the kernel's leading scalar arguments -- copies of those fields of the parameter struct.
 // Separate scalar arguments ahead of the struct are in registers when a wavefront starts, so the slot index load that
-// depends on the batch row need not wait for the argument block to be loaded.  SPEC > 0: the serving cases (no
-// dispatch order, a power-of-two head count).
+// depends on the batch row need not wait for the argument block to be loaded.  SPEC > 0: the serving cases (a
+// power-of-two head count).
 struct TileId {
     int b, h, hk;
 };
 template <int SPEC>
-__device__ __forceinline__ TileId tile_id_lead(const int32_t* order, int per_xcd, int rows_per_xcd, int hv, int hv_shift) {
+__device__ __forceinline__ TileId tile_id_lead(int per_xcd, int hv, int hv_shift) {
     const int wg = blockIdx.x;
     const int tile = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
     TileId t;
     t.b = (SPEC > 0 || hv_shift >= 0) ? tile >> hv_shift : tile / hv;
     t.h = tile - t.b * hv;
-    if (SPEC == 0 && order) {
-        int pos = t.b;
-        if (rows_per_xcd) {
-            const int x = pos / rows_per_xcd;
-            pos = (pos - x * rows_per_xcd) * 8 + x;
-        }
-        t.b = order[pos];
-    }
     t.hk = t.h;
     return t;
 }

@@ -13,14 +13,14 @@ import torch
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, 'libsqhip.so')
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 F32, BF16, F16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 FAMILY = {'gdn': 0, 'kda': 1, 'mamba2': 2}
 
 SYMBOLS = ('sq_abi_version', 'sq_strerror', 'sq_last_error', 'sq_supported', 'sq_gdn_step', 'sq_kda_step',
-           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_fold_first', 'sq_gga_step', 'sq_gga_store', 'sq_gga_load',
+           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_debug_select', 'sq_gga_step', 'sq_gga_store', 'sq_gga_load',
            'sq_gga_supported')
 E_UNSUPPORTED = -2
 
@@ -50,7 +50,7 @@ class SqGdnArgs(C.Structure):
                 ('b', _vp), ('s_b', _i64), ('b_dtype', _i32),
                 ('A_log', _vp), ('A_log_dtype', _i32),
                 ('dt_bias', _vp), ('dt_bias_dtype', _i32),
-                ('out', _vp), ('out_dtype', _i32), ('scale', _f32), ('order', _vp)]
+                ('out', _vp), ('out_dtype', _i32), ('scale', _f32)]
 
 
 class SqKdaArgs(C.Structure):
@@ -60,7 +60,7 @@ class SqKdaArgs(C.Structure):
                 ('v', _vp), ('s_v', _i64), ('v_dtype', _i32),
                 ('g', _vp), ('s_g', _i64), ('g_dtype', _i32),
                 ('beta', _vp), ('s_beta', _i64), ('beta_dtype', _i32),
-                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('scale', _f32), ('order', _vp)]
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('scale', _f32)]
 
 
 class SqMamba2Args(C.Structure):
@@ -72,7 +72,7 @@ class SqMamba2Args(C.Structure):
                 ('A', _vp), ('A_dtype', _i32), ('D', _vp), ('D_dtype', _i32),
                 ('dt_bias', _vp), ('dt_bias_dtype', _i32),
                 ('dt_softplus', _i32), ('dt_clamp', _i32), ('dt_min', _f32), ('dt_max', _f32),
-                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('order', _vp)]
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32)]
 
 
 class SqPackArgs(C.Structure):
@@ -135,6 +135,8 @@ def lib():
             f = getattr(L, name)
             f.restype = C.c_int
             f.argtypes = [C.POINTER(SqGgaSlots), C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
+        L.sq_debug_select.restype = None
+        L.sq_debug_select.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         L.sq_gga_supported.restype = C.c_int
         L.sq_gga_supported.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         if L.sq_abi_version() != ABI_VERSION:
@@ -209,16 +211,10 @@ def read_state(lay, T, strides, nptr_stride, idx, out, kda):
     check(lib().sq_read(C.byref(a), current_stream(out.device)))
 
 
-def fold_first(idx, nptr, m, out=None):
-    """``sq_fold_first``: dispatch order (int32 [rows]) with the rows that fold on the coming step first."""
-    rows = idx.shape[0]
-    if out is None:
-        out = torch.empty(rows, dtype=torch.int32, device=idx.device)
-    assert idx.dtype == torch.int32 and idx.is_contiguous() and out.dtype == torch.int32 and out.is_contiguous()
-    assert nptr.dtype == torch.int32
-    check(lib().sq_fold_first(C.c_void_p(idx.data_ptr()), C.c_void_p(nptr.data_ptr()), C.c_int64(nptr.stride(0)),
-                              C.c_int32(m), C.c_int32(rows), C.c_void_p(out.data_ptr()), current_stream(idx.device)))
-    return out
+def select_instances(no_specialised=False, no_group_kernel=False, max_heads_per_workgroup=0):
+    """``sq_debug_select``: which compiled instance serves a step call when several can (a diagnostic for twin tests
+    and profiles; results do not depend on it).  Call without arguments to restore the default choice."""
+    lib().sq_debug_select(int(no_specialised), int(no_group_kernel), int(max_heads_per_workgroup))
 
 
 def require_gpu(t, what):

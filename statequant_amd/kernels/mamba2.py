@@ -18,7 +18,7 @@ import torch
 from . import _hip
 from ._lockstep import LockstepState, describe_format, power_of_two
 from .fold import _bits, _require_kernel, pack_vk, packed_format, unpack_vk
-from .slots import SlotLayout, _order_ptr, field_table, slot_state, state_fields
+from .slots import SlotLayout, field_table, slot_state, state_fields
 
 
 def _activated_dt(dt, A, dt_bias, dt_softplus, dt_limit):
@@ -70,15 +70,13 @@ def _common(st, fmt, hv, hk, dk, dv, m, buffer_bits):
     st.buffer_bits, st.qbuf = buffer_bits, buffer_bits == 8
 
 
-def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx, T, strides, nptr_stride,
-            order=None):
+def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx, T, strides, nptr_stride):
     """One ``sq_mamba2_step`` call (replaces mamba2.py:223-241)."""
     assert x.stride(-1) == 1 and B.stride(-1) == 1 and C.stride(-1) == 1 and dt.stride(-1) == 1
     assert x.stride(-2) == st.DV and out.stride(-1) == 1 and out.stride(-2) == st.DV
     assert B.stride(-2) == st.DK and C.stride(-2) == st.DK
     assert A.is_contiguous() and (D is None or D.is_contiguous()) and (dt_bias is None or dt_bias.is_contiguous())
-    _hip.same_device('Mamba2 step', T['S'], idx=idx, x=x, dt=dt, B=B, C=C, A=A, D=D, dt_bias=dt_bias, out=out,
-                     order=order)
+    _hip.same_device('Mamba2 step', T['S'], idx=idx, x=x, dt=dt, B=B, C=C, A=A, D=D, dt_bias=dt_bias, out=out)
     clamp = dt_limit is not None and tuple(dt_limit) != (0., float('inf'))
     lo, hi = (float(dt_limit[0]), float(dt_limit[1])) if clamp else (0., 0.)
     a = _hip.SqMamba2Args(
@@ -91,7 +89,7 @@ def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limi
         D=_hip.ptr(D), D_dtype=_hip.dtype_code(D) if D is not None else 0,
         dt_bias=_hip.ptr(dt_bias), dt_bias_dtype=_hip.dtype_code(dt_bias) if dt_bias is not None else 0,
         dt_softplus=int(bool(dt_softplus)), dt_clamp=int(clamp), dt_min=lo, dt_max=hi,
-        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out), order=_order_ptr(order, rows))
+        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out))
     _hip.check(_hip.lib().sq_mamba2_step(ctypes.byref(a), _hip.current_stream(out.device)))
     return out
 
@@ -159,20 +157,19 @@ class Mamba2SlotLayout(SlotLayout):
                 f'm={self.m}, buffer_bits={self.buffer_bits}, {self.nbytes} B/slot)')
 
     def step(self, views, idx, x, dt, B, C, out, A, D=None, dt_bias=None, dt_softplus=True,
-             dt_limit=(0., float('inf')), order=None):
+             dt_limit=(0., float('inf'))):
         """One decode token for every batch row b on slot ``idx[b]`` (int32 [rows]; <= 0 = padding: output zeroed,
         nothing read or written) (mamba2.py:377-396).
 
         x [rows, H, d_v], dt [rows, H] (raw: + dt_bias, softplus, clamp in the kernel), B / C [rows, G, d_k]: any row
-        stride, contiguous rows; out [rows, H, d_v] (row stride free); A [H] (= -exp(A_log)), D, dt_bias [H] or None.
-        ``order``: optional dispatch order of the rows, as in ``SlotLayout.step``."""
+        stride, contiguous rows; out [rows, H, d_v] (row stride free); A [H] (= -exp(A_log)), D, dt_bias [H] or None."""
         rows = idx.shape[0]
         if rows == 0:
             return out
         assert idx.dtype == torch.int32 and idx.is_contiguous()
         T, strides, sN = slot_state(views)
         return _launch(self, self._layout_struct(), rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx,
-                       T, strides, sN, order)
+                       T, strides, sN)
 
 
 __all__ = ['PackedMamba2State', 'Mamba2SlotLayout', 'mamba2_recurrence']

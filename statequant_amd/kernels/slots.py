@@ -76,13 +76,6 @@ def slot_state(views):
     return T, strides, st('NPTR')
 
 
-def _order_ptr(order, rows):
-    if order is None:
-        return None
-    assert order.dtype == torch.int32 and order.is_contiguous() and order.shape[0] == rows and order.is_cuda
-    return order.data_ptr()
-
-
 class SlotLayout:
     """The packed per-slot layout of one GDN layer and the operations on a batch of slots (slots.py:40-121).
 
@@ -150,17 +143,8 @@ class SlotLayout:
         """A standalone zeroed blob [num_slots, nbytes] uint8."""
         return torch.zeros(num_slots, self.nbytes, dtype=torch.uint8, device=device)
 
-    def fold_first(self, views, idx, out=None):
-        """Dispatch order for ``step(order=...)``: the rows whose buffer fills on the coming step (they fold, which
-        takes 2.5 x as long) first, the rest behind them, padding rows last; int32 [B] (``out`` if given), one small
-        launch reading the slots' fill counters.  The counters of every layer of a model move together, so one order
-        per decode step serves all layers.  Worth it when sequences joined the batch at different times; a batch that
-        folds in lockstep gains nothing."""
-        _hip.same_device('SlotLayout.fold_first', views['NPTR'], idx=idx, out=out)
-        return _hip.fold_first(idx, views['NPTR'], self.m, out)
-
     # -- decode -----------------------------------------------------------------------------------------------
-    def step(self, views, idx, q, k, v, out, scale, *, g=None, beta=None, gate=None, fused='layout', order=None):
+    def step(self, views, idx, q, k, v, out, scale, *, g=None, beta=None, gate=None, fused='layout'):
         """One decode token for every batch row b, on slot ``idx[b]`` (int32 [B]; <= 0 = padding row)
         (slots.py:124-187).
 
@@ -169,8 +153,6 @@ class SlotLayout:
         out     [B, hv, d_v] contiguous; written (zeros on padding rows)
         g, beta [B, hv] log decay and (sigmoided) beta;  or ``gate=(a, b, A_log, dt_bias)``: formed in the kernel as
                 g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b)
-        order   optional int32 [B] permutation (``fold_first``): the order in which the rows are dispatched on the GPU;
-                results do not depend on it (not in the reference: a scheduling hint for batches of unequal lengths)
         One kernel launch on the current stream, no allocation, no host synchronization: graph-capturable.  Each
         row's buffer counter advances; rows whose buffer fills are folded and re-rounded in place.
         """
@@ -184,7 +166,7 @@ class SlotLayout:
         assert idx.dtype == torch.int32 and idx.is_contiguous()
         ga, gb, A_log, dt_bias = gate if gate is not None else (None,) * 4
         _hip.same_device('SlotLayout.step', views['S'], idx=idx, q=q, k=k, v=v, out=out, g=g, beta=beta, a=ga, b=gb,
-                         A_log=A_log, dt_bias=dt_bias, order=order)
+                         A_log=A_log, dt_bias=dt_bias)
         lay = self._layout_struct()
         T, strides, sN = slot_state(views)
         a = _hip.SqGdnArgs(
@@ -192,7 +174,7 @@ class SlotLayout:
             q=q.data_ptr(), s_q=q.stride(0), q_dtype=_hip.dtype_code(q),
             k=k.data_ptr(), s_k=k.stride(0), k_dtype=_hip.dtype_code(k),
             v=v.data_ptr(), s_v=v.stride(0), v_dtype=_hip.dtype_code(v), qk_per_key_head=1,
-            out=out.data_ptr(), out_dtype=_hip.dtype_code(out), scale=float(scale), order=_order_ptr(order, B))
+            out=out.data_ptr(), out_dtype=_hip.dtype_code(out), scale=float(scale))
         if gate is not None:
             assert ga.stride(-1) == 1 and gb.stride(-1) == 1 and A_log.is_contiguous() and dt_bias.is_contiguous()
             a.gate = 1

@@ -160,14 +160,15 @@ def test_gdn_pace4_d128_values_scaled_per_head(m, bb):
 
 def _stepped_twice(step, blobs):
     """Run `step(views_index)` on blob 0 with the compiled-in serving case allowed and on blob 1 with it switched off
-    (`SQ_NO_SPEC`: the general instance, which reads dtypes and options from the arguments)."""
-    import os
+    (`select_instances(no_specialised=True)`: the general instance, which reads dtypes and options from the
+    arguments)."""
+    from statequant_amd.kernels import _hip
     a = step(0)
-    os.environ['SQ_NO_SPEC'] = '1'
+    _hip.select_instances(no_specialised=True)
     try:
         b = step(1)
     finally:
-        del os.environ['SQ_NO_SPEC']
+        _hip.select_instances()
     assert torch.equal(a, b)
     assert torch.equal(blobs[0], blobs[1])
 

@@ -38,8 +38,18 @@ def test_settings_and_errors():
         P.config({'STATEQUANT_VLLM': 'pace4', 'STATEQUANT_VLLM_FUSED': 'yes'})
     with pytest.raises(AssertionError, match='no plan file'):
         P.config({'STATEQUANT_VLLM': 'gga:/nonexistent/plan.pt:pw'})
-    with pytest.raises(AssertionError, match='external'):
-        P.config({'STATEQUANT_VLLM': 'external:mod:fn'})
+    # external:<src>:<fn>: an unpacked slot state in the named dtype, GDN layers only
+    assert P.config({'STATEQUANT_VLLM': 'external:pkg.mod:fn'})[0] == 'fp32'
+    assert P.config({'STATEQUANT_VLLM': 'external:/x/q.py:fn', 'STATEQUANT_VLLM_EXTERNAL_DTYPE': 'BF16'})[0] == 'bf16'
+    with pytest.raises(AssertionError, match='external:<file.py or module>:<function>'):
+        P.config({'STATEQUANT_VLLM': 'external:fn'})
+    with pytest.raises(AssertionError, match='fp32 or bf16'):
+        P.config({'STATEQUANT_VLLM': 'external:m:fn', 'STATEQUANT_VLLM_EXTERNAL_DTYPE': 'fp16'})
+    P.configure({'STATEQUANT_VLLM': 'external:m:fn'})
+    assert P.active_kinds() == ('gdn',)
+    with pytest.raises(AssertionError, match='GDN layers only'):
+        P.configure({'STATEQUANT_VLLM': 'external:m:fn', 'STATEQUANT_VLLM_LAYERS': 'mamba2'})
+    P.configure({'STATEQUANT_VLLM': 'off'})
 
 
 def test_layer_kinds():

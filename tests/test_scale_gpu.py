@@ -59,61 +59,6 @@ def test_full_size_subset_and_twin_rows(fmt):
     assert d.max().item() <= 1 and (d != 0).float().mean().item() < 1e-3, ((d != 0).float().mean().item(), d.max())
 
 
-def test_dispatch_order_changes_nothing_but_the_schedule():
-    """``step(order=...)``: any permutation of the rows' dispatch order leaves every output and every byte of the
-    blobs as the natural order does; ``fold_first`` puts the rows that fold on the coming step first, padding last."""
-    HV, HK, D, m, rows = 8, 4, 128, 4, 24
-    fmt = (8, 'k', 128)
-    lay = SlotLayout(sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
-    gen = torch.Generator().manual_seed(9)
-    slots = torch.randperm(rows, generator=gen) + 1
-    slots[5] = 0                                                          # a padding row
-    idx = slots.to(torch.int32).to(DEV)
-    S0 = (torch.randn(rows, HV, D, D, generator=gen) * 0.4).to(DEV)
-    blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
-    views = [lay.views(b) for b in blobs]
-    live = idx > 0
-    for v in views:
-        lay.write(v, idx[live].long(), S0[live])
-        v['NPTR'][idx[live].long()] = (torch.arange(rows, device=DEV, dtype=torch.int32)[live] % m)[:, None]
-    for t in range(2 * m + 1):
-        q, k, vv, g, beta = (x.to(DEV) for x in gdn_token(gen, rows, HV, HK, D, D))
-        first = lay.fold_first(views[0], idx)
-        n = views[0]['NPTR'][idx.long().clamp_min(0), 0] & (m - 1)
-        want_first = (live & (n == m - 1)).sum().item()
-        assert sorted(first.tolist()) == list(range(rows))
-        assert set(first[:want_first].tolist()) == set(torch.nonzero(live & (n == m - 1)).flatten().tolist())
-        assert first[-1].item() == 5
-        order = first if t % 2 == 0 else torch.randperm(rows, generator=gen).to(torch.int32).to(DEV)
-        o0 = torch.full((rows, HV, D), 7.0, device=DEV)
-        o1 = torch.full((rows, HV, D), 7.0, device=DEV)
-        lay.step(views[0], idx, q, k, vv, o0, D ** -0.5, g=g, beta=beta, order=order)
-        lay.step(views[1], idx, q, k, vv, o1, D ** -0.5, g=g, beta=beta)
-        assert torch.equal(o0, o1), t
-        assert torch.equal(blobs[0], blobs[1]), t
-
-
-@pytest.mark.parametrize('rows', [1, 7, 256, 601])
-def test_fold_first_is_a_stable_three_class_order(rows):
-    """`sq_fold_first`: folding rows, then the other live rows, then padding rows, each class in its natural order
-    (more rows than the helper's workgroup has threads: several passes per class)."""
-    m = 8
-    lay = SlotLayout(sq.Quantizer(8, 'k', 128), 4, 2, 128, 128, m=m)
-    gen = torch.Generator().manual_seed(rows)
-    n_slots = rows + 3
-    views = lay.views(lay.alloc(n_slots, DEV))
-    views['NPTR'][:] = torch.randint(0, 4 * m, (n_slots, views['NPTR'].shape[1]), generator=gen).to(torch.int32).to(DEV)
-    idx = (torch.randperm(rows, generator=gen) + 1).to(torch.int32)
-    idx[torch.rand(rows, generator=gen) < 0.2] = 0
-    if rows > 3:
-        idx[2] = -1
-    got = lay.fold_first(views, idx.to(DEV)).cpu()
-    n = views['NPTR'][idx.long().clamp_min(0), 0].cpu() & (m - 1)
-    cls = torch.where(idx <= 0, 2, torch.where(n == m - 1, 0, 1))
-    want = torch.argsort(cls, stable=True).to(torch.int32)
-    assert torch.equal(got, want)
-
-
 def test_graph_replay_matches_eager():
     HV, HK, D, m, slots = 8, 4, 128, 4, 6
     fmt = (8, 'k', 64)
