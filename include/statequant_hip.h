@@ -141,7 +141,8 @@ typedef struct sq_mamba2_args {
 /* Store fp32 states in the packed format (fold.py:123-147 `pack_vk`; with idx, GCUR and NPTR given this is
  * slots.py:236-252 `SlotLayout.write`: the states go into sequences idx[b] and those sequences' buffers are emptied).
  * src [rows, hv, dv, dk] value-major fp32, row stride s_src in elements; codes / scales as in sq_state.
- * Uses lay.bits, axis_k, group, hv, dk, dv.  GCUR / NPTR may be NULL (left alone); gcur_per_head = 1 (GDN, Mamba2)
+ * Uses lay.bits, axis_k, group, hv, dk, dv.  GCUR / NPTR may be NULL (left alone); nptr_copies = counter copies per sequence that are zeroed (the slot
+ * layout keeps max(hv, 4), slots.py:13-15; 0 means hv); gcur_per_head = 1 (GDN, Mamba2)
  * or dk (KDA).  Rows with idx[b] <= 0 are skipped. */
 typedef struct sq_pack_args {
     sq_layout lay;
@@ -151,7 +152,7 @@ typedef struct sq_pack_args {
     void* S;            int64_t sS;
     void* SC;           int64_t sSC;
     float* GCUR;        int64_t sGC;     int32_t gcur_per_head;
-    int32_t* NPTR;      int64_t sN;
+    int32_t* NPTR;      int64_t sN;      int32_t nptr_copies;
 } sq_pack_args;
 
 /* The current state of sequences idx[b] as fp32 value-major [rows, hv, dv, dk] (row stride s_out in elements): the

@@ -302,6 +302,9 @@ int sq_pack_vk(const sq_pack_args* a, void* stream) {
     p.SC = static_cast<uint16_t*>(a->SC); p.sSC = uint32_t(a->sSC);
     p.GCUR = a->GCUR; p.sGC = uint32_t(a->sGC); p.gcur_per_head = a->gcur_per_head;
     p.NPTR = a->NPTR; p.sN = uint32_t(a->sN);
+    p.nptr_copies = a->nptr_copies > a->lay.hv ? a->nptr_copies : a->lay.hv;
+    if (a->NPTR && a->sN != 0 && int64_t(p.nptr_copies) > a->sN)
+        return fail(SQ_E_ARG, "%s: %d counter copies do not fit a counter stride of %lld", who, p.nptr_copies, (long long)a->sN);
     return finish(sq::dispatch_pack(p, static_cast<hipStream_t>(stream), true), who, a->lay);
 }
 

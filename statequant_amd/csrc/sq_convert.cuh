@@ -21,7 +21,11 @@ using RowTile = Tile<BITS, DK, 128, GROUP, QBUF, 16, AXV>;
 
 // Empty a sequence's buffer: this head's counter copy and running decay.
 __device__ __forceinline__ void reset_counters(const PackParams& p, uint32_t seq, uint32_t h, int lane) {
-    if (p.NPTR && lane == 0) *field(p.NPTR, seq, p.sN, h) = 0;
+    if (p.NPTR && lane == 0) {
+        *field(p.NPTR, seq, p.sN, h) = 0;
+        if (h + 1 == uint32_t(p.hv))                         // the last head also clears the copies no head owns
+            for (uint32_t e = p.hv; e < uint32_t(p.nptr_copies); ++e) *field(p.NPTR, seq, p.sN, e) = 0;
+    }
     if (p.GCUR)
         for (uint32_t e = lane; e < uint32_t(p.gcur_per_head); e += WAVE)
             *field(p.GCUR, seq, p.sGC, h * uint32_t(p.gcur_per_head) + e) = 0.0f;

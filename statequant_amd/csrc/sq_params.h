@@ -81,7 +81,7 @@ struct PackParams {
     uint8_t* S;        uint32_t sS;
     uint16_t* SC;      uint32_t sSC;
     float* GCUR;       uint32_t sGC;  int gcur_per_head;      // optional (null: leave)
-    int32_t* NPTR;     uint32_t sN;
+    int32_t* NPTR;     uint32_t sN;   int nptr_copies;        // counter copies per sequence (>= hv)
 };
 
 struct ReadParams : LayoutKey {

@@ -62,11 +62,11 @@ def config(environ=None):
     file, the window flag and its length)."""
     raw = _env(environ, ENV).strip()
     mode = raw.lower()
-    if mode in OFF:
-        return None
     _state.pop('gga', None)
     _state.pop('external', None)
     _state.pop('external_fn', None)
+    if mode in OFF:
+        return None
     if mode.startswith('external:'):
         source, _, name = raw[len('external:'):].rpartition(':')
         assert source and name, f'{ENV}=external:<file.py or module>:<function>, got {raw[len("external:"):]!r}'

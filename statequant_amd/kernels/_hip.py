@@ -78,7 +78,7 @@ class SqMamba2Args(C.Structure):
 class SqPackArgs(C.Structure):
     _fields_ = [('lay', SqLayout), ('rows', _i32), ('idx', _vp), ('src', _vp), ('s_src', _i64),
                 ('S', _vp), ('sS', _i64), ('SC', _vp), ('sSC', _i64),
-                ('GCUR', _vp), ('sGC', _i64), ('gcur_per_head', _i32), ('NPTR', _vp), ('sN', _i64)]
+                ('GCUR', _vp), ('sGC', _i64), ('gcur_per_head', _i32), ('NPTR', _vp), ('sN', _i64), ('nptr_copies', _i32)]
 
 
 class SqReadArgs(C.Structure):
@@ -197,7 +197,8 @@ def pack_into(lay, src, S, sS, SC, sSC, idx=None, GCUR=None, sGC=0, gcur_per_hea
     rows = src.shape[0]
     a = SqPackArgs(lay=lay, rows=rows, idx=ptr(idx), src=src.data_ptr(), s_src=src.stride(0) if rows else 0,
                    S=S.data_ptr(), sS=sS, SC=ptr(SC), sSC=sSC, GCUR=ptr(GCUR), sGC=sGC,
-                   gcur_per_head=gcur_per_head, NPTR=ptr(NPTR), sN=sN)
+                   gcur_per_head=gcur_per_head, NPTR=ptr(NPTR), sN=sN,
+                   nptr_copies=0 if NPTR is None else NPTR[0].numel())
     check(lib().sq_pack_vk(C.byref(a), current_stream(src.device)))
 
 

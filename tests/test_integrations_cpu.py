@@ -149,3 +149,275 @@ def test_gga_plan_file(tmp_path):
     assert P.gated_delta_net_state_shape(1, **QWEN) == (lay.nbytes,)
     cfg = P.configure({'STATEQUANT_VLLM': f'gga:{path}'})
     assert P.gga_settings()[1] is False and not P.layout(HV, 16, D, D).pw
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The patches themselves, on stand-in engine modules (no engine installed): the state calculators answer packed only
+# to the callers whose layers have a packed forward, the GDN base class refuses other subclasses, the patched
+# constructors attach the layout and refuse unsupported cache settings, and everything can be undone.
+# ---------------------------------------------------------------------------------------------------------------
+import types  # noqa: E402
+
+from statequant_amd.integrations import vllm_olmo  # noqa: E402
+
+
+def _fake_mamba_utils():
+    class MambaStateShapeCalculator:
+        @classmethod
+        def gated_delta_net_state_shape(cls, tp, nk, nv, dk, dv, conv_kernel_size, num_spec=0):
+            return ((2 * nk * dk + nv * dv) // tp, conv_kernel_size - 1), (nv // tp, dv, dk)
+
+        @classmethod
+        def kda_state_shape(cls, tp, num_heads, head_dim, num_k_heads=None, head_k_dim=None, conv_kernel_size=4,
+                            num_spec=0):
+            return (3 * num_heads * head_dim // tp, conv_kernel_size - 1), (num_heads // tp, head_dim, head_dim)
+
+        @classmethod
+        def mamba2_state_shape(cls, tp_world_size, intermediate_size, n_groups, num_heads, head_dim, state_size,
+                               conv_kernel, num_spec=0):
+            return ((intermediate_size + 2 * n_groups * state_size) // tp_world_size, conv_kernel - 1), \
+                (num_heads // tp_world_size, head_dim, state_size)
+
+    class MambaStateDtypeCalculator:
+        @classmethod
+        def gated_delta_net_state_dtype(cls, model_dtype, mamba_cache_dtype, mamba_ssm_cache_dtype='auto'):
+            return model_dtype, torch.bfloat16
+
+        @classmethod
+        def kda_state_dtype(cls, model_dtype, mamba_cache_dtype, mamba_ssm_cache_dtype='auto'):
+            return model_dtype, torch.float32
+
+        @classmethod
+        def mamba2_state_dtype(cls, model_dtype, mamba_cache_dtype, mamba_ssm_cache_dtype):
+            return model_dtype, torch.float32
+
+    return types.SimpleNamespace(MambaStateShapeCalculator=MambaStateShapeCalculator,
+                                 MambaStateDtypeCalculator=MambaStateDtypeCalculator)
+
+
+def _call_from(module_name, expr, **names):
+    """Evaluate ``expr`` in a function whose module is ``module_name`` (what the calculators look at: their caller)."""
+    g = dict(names, __name__=module_name, torch=torch)
+    exec(f'def hook():\n    return {expr}\n', g)
+    return g['hook']()
+
+
+def _vllm_config(spec=None, prefix_caching=False, mode='none', eager=True):
+    return types.SimpleNamespace(speculative_config=spec, model_config=types.SimpleNamespace(enforce_eager=eager),
+                                 cache_config=types.SimpleNamespace(enable_prefix_caching=prefix_caching,
+                                                                    mamba_cache_mode=mode, mamba_ssm_cache_dtype='auto'))
+
+
+def test_gdn_calculators_answer_packed_to_supported_callers_only():
+    P.configure({'STATEQUANT_VLLM': 'pace4'})
+    mu = _fake_mamba_utils()
+    P._patch_calculators(mu)
+    try:
+        shape = 'mu.MambaStateShapeCalculator.gated_delta_net_state_shape(1, 16, 32, 128, 128, 4)'
+        dtype = "mu.MambaStateDtypeCalculator.gated_delta_net_state_dtype(torch.bfloat16, 'auto')"
+        want = P.layout(32, 16, 128, 128).nbytes
+        for mod in P.PACKED_MODEL_MODULES + (P.PACKED_MODEL_MODULES[0] + '.sub',):
+            assert _call_from(mod, shape, mu=mu) == ((2 * 16 * 128 + 32 * 128, 3), (want,))
+            assert _call_from(mod, dtype, mu=mu) == (torch.bfloat16, torch.uint8)
+        # tensor parallel: each rank packs its own heads
+        tp2 = 'mu.MambaStateShapeCalculator.gated_delta_net_state_shape(2, 16, 32, 128, 128, 4)'
+        assert _call_from(P.PACKED_MODEL_MODULES[1], tp2, mu=mu)[1] == (P.layout(16, 8, 128, 128).nbytes,)
+        for mod in ('vllm.model_executor.models.minicpmv', 'vllm.model_executor.models.qwen3_next_mtp'):
+            with pytest.raises(NotImplementedError, match='stores packed GDN states only for'):
+                _call_from(mod, shape, mu=mu)
+            with pytest.raises(NotImplementedError):
+                _call_from(mod, dtype, mu=mu)
+        # a layer asking through its own method is recognised by its class, whatever module the call comes from
+        Layer = type('QwenGatedDeltaNetAttention', (), {'__module__': P.PACKED_LAYER[0]})
+        Sub = type('Derived', (Layer,), {'__module__': 'somewhere.else'})
+        Other = type('MiniGDN', (), {'__module__': 'vllm.model_executor.layers.mamba.gdn.other'})
+
+        def get_state_shape(self):
+            return mu.MambaStateShapeCalculator.gated_delta_net_state_shape(1, 16, 32, 128, 128, 4)
+        assert get_state_shape(Sub())[1] == (want,)
+        with pytest.raises(NotImplementedError, match='MiniGDN'):
+            get_state_shape(Other())
+        with pytest.raises(AssertionError, match='speculative'):
+            _call_from(P.PACKED_MODEL_MODULES[0],
+                       'mu.MambaStateShapeCalculator.gated_delta_net_state_shape(1, 16, 32, 128, 128, 4, 2)', mu=mu)
+    finally:
+        P.unpatch()
+    assert mu.MambaStateShapeCalculator.gated_delta_net_state_shape(1, 16, 32, 128, 128, 4)[1] == (32, 128, 128)
+
+
+def _fake_gdn_modules():
+    class GatedDeltaNetAttention:
+        def __init__(self, *a, **k):
+            self.base_built = True
+
+    def make(name):
+        def __init__(self, config, vllm_config, prefix='model.layers.1.linear_attn'):
+            GatedDeltaNetAttention.__init__(self)
+            self.prefix, self.tp_size = prefix, 2
+            self.num_v_heads, self.num_k_heads, self.head_k_dim, self.head_v_dim = 32, 16, 128, 128
+        return type(name, (GatedDeltaNetAttention,), {
+            '__init__': __init__, '_forward_core': lambda self, *a: 'stock',
+            '_warmup_prefill_kernels': lambda self, qkv, v_dim: self.get_state_dtype(),
+            'get_state_dtype': lambda self: (torch.bfloat16, torch.uint8)})
+    Q = types.SimpleNamespace(QwenGatedDeltaNetAttention=make('QwenGatedDeltaNetAttention'), logger=None)
+    O = types.SimpleNamespace(OlmoHybridGatedDeltaNetAttention=make('OlmoHybridGatedDeltaNetAttention'))
+    Other = type('OtherGDN', (GatedDeltaNetAttention,), {'__init__': lambda self: GatedDeltaNetAttention.__init__(self)})
+    return Q, O, types.SimpleNamespace(GatedDeltaNetAttention=GatedDeltaNetAttention), Other
+
+
+def test_gdn_layer_patch_attaches_layout_and_refuses_the_rest():
+    P.configure({'STATEQUANT_VLLM': 'int8k'})
+    Q, O, base, Other = _fake_gdn_modules()
+    cfg = types.SimpleNamespace(layer_types=['linear_attention'] * 4)
+    P._patch_layer(Q, O, base)
+    vllm_olmo.patch(P.layout, O)
+    try:
+        P._patch_layer(Q, O, base)                            # idempotent
+        layer = Q.QwenGatedDeltaNetAttention(cfg, _vllm_config())
+        assert layer.base_built and layer._sq_layout is P.layout(16, 8, 128, 128) and layer._sq_views is None
+        assert layer._sq_external is None and layer._sq_lk == {}
+        assert Q.QwenGatedDeltaNetAttention._forward_core is P._forward_core
+        # the prefill warm-up sees an fp32 state dtype, and the override is gone afterwards
+        assert layer._warmup_prefill_kernels(None, 0) == (torch.bfloat16, torch.float32)
+        assert layer.get_state_dtype() == (torch.bfloat16, torch.uint8)
+        olmo = O.OlmoHybridGatedDeltaNetAttention(cfg, _vllm_config())
+        assert olmo._sq_layout is layer._sq_layout and O.OlmoHybridGatedDeltaNetAttention._forward_core is vllm_olmo._forward_core
+        with pytest.raises(NotImplementedError, match='OtherGDN'):
+            Other()
+        for bad, msg in ((_vllm_config(spec=object()), 'speculative'), (_vllm_config(prefix_caching=True), 'prefix caching')):
+            with pytest.raises(AssertionError, match=msg):
+                Q.QwenGatedDeltaNetAttention(cfg, bad)
+            with pytest.raises(AssertionError, match=msg):
+                O.OlmoHybridGatedDeltaNetAttention(cfg, bad)
+        with pytest.raises(AssertionError):
+            Q.QwenGatedDeltaNetAttention(cfg, _vllm_config(mode='align'))
+    finally:
+        P.unpatch()
+        vllm_olmo.unpatch()
+    assert Q.QwenGatedDeltaNetAttention(cfg, _vllm_config())._forward_core() == 'stock'
+    assert not hasattr(Q.QwenGatedDeltaNetAttention(cfg, _vllm_config()), '_sq_layout')
+    Other()
+
+
+def test_external_quantizer_settings(tmp_path):
+    src = tmp_path / 'q.py'
+    src.write_text('def halve(S, layer):\n    return S * 0.5 + layer\n\nnot_callable = 3\n')
+    P.configure({'STATEQUANT_VLLM': f'external:{src}:halve', 'STATEQUANT_VLLM_EXTERNAL_DTYPE': 'bf16'})
+    assert P.layout(4, 2, 64, 64).state_dtype == torch.bfloat16
+    S = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).view(2, 3, 4, 5)           # value-major [P, HV, d_v, d_k]
+    got = P.apply_external(S, 2)
+    assert got.shape == S.shape and torch.equal(got, S * 0.5 + 2)
+    cfg = types.SimpleNamespace(layer_types=['linear_attention', 'full_attention', 'linear_attention'])
+    assert P.gdn_ordinal(cfg, 'model.layers.2.linear_attn') == 1 and P.gdn_ordinal(cfg, 'model.layers.0.x') == 0
+    with pytest.raises(AssertionError):
+        P.gdn_ordinal(cfg, 'model.layers.1.self_attn')
+    Q, O, base, _ = _fake_gdn_modules()
+    P._patch_layer(Q, O, base)
+    try:
+        with pytest.raises(AssertionError, match='no tensor parallelism'):           # the fake layers have tp_size 2
+            Q.QwenGatedDeltaNetAttention(cfg, _vllm_config(), prefix='model.layers.2.linear_attn')
+    finally:
+        P.unpatch()
+    P.configure({'STATEQUANT_VLLM': f'external:{src}:not_callable'})
+    with pytest.raises(AssertionError, match='not callable'):
+        P.external_fn()
+    P.configure({'STATEQUANT_VLLM': 'external:json:dumps'})                         # an importable module
+    import json
+    assert P.external_fn() is json.dumps
+    P.configure({'STATEQUANT_VLLM': 'off'})
+    assert P.external_fn() is None
+
+
+def test_kda_and_mamba2_patches_are_scoped_to_their_models():
+    cfg = P.configure({'STATEQUANT_VLLM': 'pace4'})
+    mu = _fake_mamba_utils()
+    vllm_kda._patch_calculators(cfg, mu)
+    vllm_mamba2._patch_calculators(cfg, mu)
+    try:
+        kda = 'mu.MambaStateShapeCalculator.kda_state_shape(1, 16, 128)'
+        assert _call_from('vllm.model_executor.models.bailing_moe_v3', kda, mu=mu)[1] == (246336,)
+        assert _call_from('vllm.model_executor.models.kimi_linear', kda, mu=mu)[1] == (16, 128, 128)  # stock answer
+        kd = "mu.MambaStateDtypeCalculator.kda_state_dtype(torch.bfloat16, 'auto')"
+        assert _call_from('vllm.model_executor.models.bailing_moe_v3', kd, mu=mu) == (torch.bfloat16, torch.uint8)
+        assert _call_from('elsewhere', kd, mu=mu) == (torch.bfloat16, torch.float32)
+        with pytest.raises(AssertionError, match='tensor parallel'):
+            _call_from('vllm.model_executor.models.bailing_moe_v3',
+                       'mu.MambaStateShapeCalculator.kda_state_shape(2, 16, 128)', mu=mu)
+        m2 = ('mu.MambaStateShapeCalculator.mamba2_state_shape(tp_world_size=1, intermediate_size=7680, n_groups=8, '
+              'num_heads=96, head_dim=80, state_size=128, conv_kernel=4)')
+        for mod in ('vllm.model_executor.layers.mamba.mamba_mixer2', 'vllm.model_executor.models.nemotron_h',
+                    'vllm.model_executor.models.falcon_h1'):
+            assert _call_from(mod, m2, mu=mu)[1] == (597376,)
+        assert _call_from('vllm.model_executor.models.plamo2', m2, mu=mu)[1] == (96, 80, 128)
+        md = "mu.MambaStateDtypeCalculator.mamba2_state_dtype(torch.bfloat16, 'auto', 'auto')"
+        assert _call_from('vllm.model_executor.models.zamba2', md, mu=mu) == (torch.bfloat16, torch.uint8)
+        assert _call_from('vllm.model_executor.models.plamo2', md, mu=mu) == (torch.bfloat16, torch.float32)
+    finally:
+        vllm_kda.unpatch()
+        vllm_mamba2.unpatch()
+    assert mu.MambaStateShapeCalculator.kda_state_shape(1, 16, 128)[1] == (16, 128, 128)
+
+
+def test_kda_and_mamba2_layer_patches():
+    cfg = P.configure({'STATEQUANT_VLLM': 'int8k'})
+    box = {'vc': _vllm_config()}
+
+    class Kimi:
+        def __init__(self, config, tp=1, spec=0):
+            self.tp_size, self.num_speculative_tokens, self.local_num_heads, self.head_dim = tp, spec, 16, 128
+
+        def _forward(self, *a):
+            return 'stock'
+    Mk = types.SimpleNamespace(BailingMoeV3KimiDeltaAttention=Kimi, get_current_vllm_config=lambda: box['vc'])
+
+    class Mixer:
+        def __init__(self, tp=1, replay=False):
+            self.tp_size, self.num_spec, self.use_replayssm = tp, 0, replay
+            self.num_heads, self.n_groups, self.ssm_state_size, self.head_dim = 96, 8, 128, 80
+
+        def _warmup_ssd_kernels(self, ps):
+            return self.get_state_dtype()
+
+        def get_state_dtype(self):
+            return (torch.bfloat16, torch.uint8)
+
+        def conv_ssm_forward(self, *a):
+            return 'stock'
+    Mm = types.SimpleNamespace(MambaMixer2=Mixer, get_current_vllm_config=lambda: box['vc'], logger=None)
+    vllm_kda._patch_layer(cfg, Mk)
+    vllm_mamba2._patch_layer(cfg, Mm)
+    try:
+        k = Kimi(None)
+        assert k._sq_layout is vllm_kda.layout(cfg, 16, 128) and Kimi._forward is vllm_kda._forward
+        with pytest.raises(AssertionError, match='tensor parallel'):
+            Kimi(None, tp=2)
+        with pytest.raises(AssertionError, match='MTP'):
+            Kimi(None, spec=1)
+        mx = Mixer()
+        assert mx._sq_layout is vllm_mamba2.layout(cfg, 96, 8, 128, 80) and Mixer.conv_ssm_forward is vllm_mamba2.conv_ssm_forward
+        assert mx._warmup_ssd_kernels(None) == (torch.bfloat16, torch.float32) and mx.get_state_dtype()[1] == torch.uint8
+        with pytest.raises(AssertionError, match='ReplaySSM'):
+            Mixer(replay=True)
+        with pytest.raises(AssertionError, match='tensor parallel'):
+            Mixer(tp=2)
+        box['vc'] = _vllm_config(prefix_caching=True)
+        with pytest.raises(AssertionError, match='prefix caching'):
+            Mixer()
+        with pytest.raises(AssertionError, match='prefix caching'):
+            Kimi(None)
+    finally:
+        vllm_kda.unpatch()
+        vllm_mamba2.unpatch()
+    box['vc'] = _vllm_config()
+    assert Kimi(None)._forward() == 'stock' and Mixer().conv_ssm_forward() == 'stock'
+
+
+def test_register_is_a_no_op_when_off(monkeypatch):
+    monkeypatch.delenv('STATEQUANT_VLLM', raising=False)
+    P.register()                                               # off: nothing imported, nothing patched
+    assert 'registered' not in P._state
+    monkeypatch.setenv('STATEQUANT_VLLM', 'pace4')
+    with pytest.raises(ImportError):                           # on, and no engine installed here
+        P.register()
+    P.unpatch()
+    P.configure({'STATEQUANT_VLLM': 'off'})
