@@ -459,6 +459,9 @@ def main():
                          '(sequences of unequal lengths, as a serving engine has them) instead of all slots folding '
                          'on the same step; a secondary figure, the headline is the lockstep configuration')
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--instances', default='', metavar='LIST',
+                    help='comma-separated exclusions handed to sq_debug_select, for same-machine comparisons of the '
+                         'kernel instances that can serve the workload: no-specialised, no-group')
     ap.add_argument('--cpu-budget', type=float, default=20.0)
     ap.add_argument('--op', default='step', choices=['step', 'write', 'read'],
                     help="step: the decode step (the headline); write / read: the prefill-side pack and read kernels "
@@ -476,6 +479,11 @@ def main():
     torch.cuda.set_device(dev)
     if a.calibrate_copy:
         return calibrate_copy(dev)
+    if a.instances:
+        from statequant_amd.kernels import _hip
+        off = {x.strip() for x in a.instances.split(',') if x.strip()}
+        assert off <= {'no-specialised', 'no-group'}, off
+        _hip.select_instances(no_specialised='no-specialised' in off, no_group_kernel='no-group' in off)
     m = a.m
     if a.slots:
         w = WORKLOADS[a.workload]
@@ -536,6 +544,7 @@ def main():
                    'steps_requested': requested[0], 'warmup_requested': requested[1], 'steps_timed': a.steps,
                    'folds_timed': a.steps // m if not a.mixed_fill else None,
                    'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
+                   'instances_excluded': a.instances or None,
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),
         'period_us': pstats, 'per_period_us': per_period_us,

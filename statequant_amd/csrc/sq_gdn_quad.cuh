@@ -90,6 +90,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
     using L = QuadLds<T, NB, GH, 2, 2>;
     constexpr int DK = T::DK, DV = T::DV, NW = Q::NW, NWH = Q::NWH, MM = T::MMAX, NE = Q::NE, NG = T::NG;
     constexpr int RQ = 1 % NW, RK = 3 % NW, RX = 2 % NW;          // which wavefront plays which shared role
+    constexpr bool DMA = SQ_QUAD_DMA != 0;                        // row blocks loaded straight into LDS
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     uint8_t* lds_kbr = lds + L::KBR;
     float* lds_xn = reinterpret_cast<float*>(lds + L::XN);
@@ -170,21 +171,28 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
     // fill count).
     {
         const uint32_t seq = slot, h = tid.h;
-        F.np = *field(p.st.NPTR, seq, p.st.sN, h);
         F.gcur = *field(p.st.GCUR, seq, p.st.sGC, h);
         const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
+        if constexpr (!DMA) F.np = *field(p.st.NPTR, seq, p.st.sN, h);
         SQ_MARK(3);                                               // counters issued
+        if constexpr (DMA) {
+            // the fill count, then the row blocks straight into their LDS image (sq_quad.cuh)
+            F.np = quad_dma_counter(field(p.st.NPTR, seq, p.st.sN, h));
+            quad_dma_blocks<Q, NB>(Sh + wh * NB * Q::BLK, my_codes, lane);
+        } else {
 #pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
+            for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-            for (int t = 0; t < Q::NLD; ++t)
-                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+                for (int t = 0; t < Q::NLD; ++t)
+                    F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     SQ_MARK(4);                                                   // row blocks issued
     const GdnAddr<T> A = gdn_addr<T>(p, tid, slot);
     void* const outp = advance(p.out, out_dt, A.obase);
     {
+        if constexpr (DMA) quad_dma_counter_wait<Q, NB>(F.np);      // before anything else is requested
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
@@ -291,11 +299,14 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
         lds_gbf[lane] = F.gbl;
         if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
     }
+    if constexpr (!DMA) {
 #pragma unroll
-    for (int bi = 0; bi < NB; ++bi)
+        for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-        for (int t = 0; t < Q::NLD; ++t)
-            *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+            for (int t = 0; t < Q::NLD; ++t)
+                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+    }
+    if constexpr (DMA) quad_dma_landed();
     const bool full = n == m - 1;
     SQ_MARK(6);                                                   // roles done, every load landed in LDS
     lds_barrier();

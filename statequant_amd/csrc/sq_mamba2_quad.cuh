@@ -112,13 +112,19 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
     uint8_t* const Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
     float* const gcp = field(p.st.GCUR, seq, p.st.sGC, h);
     int32_t* const np = field(p.st.NPTR, seq, p.st.sN, h);
-    F.np = *np;
+    constexpr bool DMA = SQ_QUAD_DMA != 0;                        // row blocks loaded straight into LDS (sq_quad.cuh)
     F.gcur = *gcp;
+    if constexpr (DMA) {
+        F.np = quad_dma_counter(np);
+        quad_dma_blocks<Q, NB>(Sh + wh * NB * Q::BLK, my_codes, lane);
+    } else {
+        F.np = *np;
 #pragma unroll
-    for (int bi = 0; bi < NB; ++bi)
+        for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-        for (int t = 0; t < Q::NLD; ++t)
-            F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+            for (int t = 0; t < Q::NLD; ++t)
+                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
+    }
     __builtin_amdgcn_sched_barrier(0);
     uint16_t* const SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
     uint8_t* const KBp = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
@@ -126,6 +132,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
     uint16_t* const KBSp = field(p.st.KBS, seq, p.st.sKBS, hk * um);
     uint16_t* const UBSp = field(p.st.UBS, seq, p.st.sUBS, h * um);
     float* const GBh = field(p.st.GB, seq, p.st.sGB, h * um);
+    if constexpr (DMA) quad_dma_counter_wait<Q, NB>(F.np);          // before anything else is requested
 #pragma unroll
     for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
@@ -221,11 +228,15 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
         lds_gbf[lane] = F.gbl;
         if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
     }
+    if constexpr (DMA) {
+        quad_dma_landed();
+    } else {
 #pragma unroll
-    for (int bi = 0; bi < NB; ++bi)
+        for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
-        for (int t = 0; t < Q::NLD; ++t)
-            *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+            for (int t = 0; t < Q::NLD; ++t)
+                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
+    }
     const bool full = n == m - 1;
     lds_barrier();
 

@@ -251,6 +251,54 @@ __device__ __forceinline__ float quad_block_pass(const uint8_t* blk, const v4i (
 }
 
 
+// ---------------------------------------------------------------------------------------------------------------
+// Row blocks loaded straight into their LDS image (global_load_lds_dwordx4: no pass through registers, no LDS store
+// instructions).  Such a load writes lane l's 16 bytes at (uniform LDS base) + 16 l, so the image's swizzle goes into
+// the global address instead: lane l fetches the chunk that belongs at position l of the 1 KB piece -- the lanes of a
+// row still cover the row's lines, in another order.
+//
+// The compiler books a load-to-LDS as touching both memories and forces every wait that follows it down to "nothing
+// outstanding", which would drain the row blocks before the fill counter (requested ahead of them) can be used.  So
+// the counter and the row blocks are requested in assembly, invisible to that bookkeeping, with the one wait in
+// between written by hand: loads complete in order, the counter is older than the N block loads, so it is here once
+// at most N loads are outstanding.  Nothing else may be requested between `quad_dma_counter` and
+// `quad_dma_counter_wait` (the compiler merges and reorders the loads it knows of; these it does not).  Every later
+// wait the compiler places for a younger load covers the block loads as well; `quad_dma_landed` states it.
+// ---------------------------------------------------------------------------------------------------------------
+#ifndef SQ_QUAD_DMA
+#define SQ_QUAD_DMA 1
+#endif
+
+__device__ __forceinline__ int quad_dma_counter(const int32_t* p) {
+    int v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+// NBLK row blocks of this wavefront: `src` their first byte in memory, `dst` their LDS image.
+template <class Q, int NBLK>
+__device__ __forceinline__ void quad_dma_blocks(const uint8_t* src, uint8_t* dst, int lane) {
+    const int pr = lane / Q::CPR, pc = lane % Q::CPR;
+#pragma unroll
+    for (int bi = 0; bi < NBLK; ++bi)
+#pragma unroll
+        for (int t = 0; t < Q::NLD; ++t) {
+            const int r = t * (1024 / Q::RB) + pr;
+            const int c = pc ^ ((r / Q::SWD) % Q::SWM);
+            const uint8_t* g = src + bi * Q::BLK + r * Q::RB + (c << 4);
+            const uint32_t at = uint32_t(reinterpret_cast<uintptr_t>(
+                (__attribute__((address_space(3))) uint8_t*)(dst + bi * Q::BLK + t * 1024)));
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+                         :: "v"(g), "s"(at) : "memory", "m0");
+        }
+}
+template <class Q, int NBLK>
+__device__ __forceinline__ void quad_dma_counter_wait(int& counter) {
+    constexpr int YOUNGER = NBLK * Q::NLD;
+    static_assert(YOUNGER < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(counter) : "n"(YOUNGER) : "memory");
+}
+__device__ __forceinline__ void quad_dma_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Raw buffered elements: four per lane.
 template <bool QBUF> struct Raw4;
 template <> struct Raw4<true> { uint32_t a; };
