@@ -106,3 +106,57 @@ def unpack_nib(codes, bits):
         return torch.where(raw < 0, -(raw & 0x7FFF), raw)
     c = codes.to(torch.int16)
     return torch.stack(((c & 15) - 8, ((c >> 4) & 15) - 8), -1).flatten(-2)
+
+
+class SlotSync:
+    """The re-sync protocol for a subset of the slots of a slot-addressed state: after every step the oracle's newest
+    buffer entry is compared with the slots' and replaced by it, after every fold the oracle's codes and scales
+    likewise, so that one rounding flip is counted once.  ``ref`` is an oracle over the slots ``sl`` (in that order,
+    built with ``auto_fold=False``); ``views`` the typed views of the blob."""
+
+    def __init__(self, views, sl, ref, bits, qbuf=True, exact_decay=True):
+        """exact_decay=False (Mamba2): the log decay is A x softplus(dt + bias) formed in the kernel, whose logf / expf
+        differ from torch's in the last bit, so the cumulative decays are compared to 5e-6 and taken over as well."""
+        self.V, self.sl, self.ref, self.bits, self.qbuf = views, sl.long(), ref, bits, qbuf
+        self.exact_decay = exact_decay
+        self.tal = Tally()
+
+    def _entry(self, i):
+        V, sl = self.V, self.sl
+        kb, ub = V['KB'][sl][:, :, i].float(), V['UB'][sl][:, :, i].float()
+        if self.qbuf:
+            kb, ub = kb * V['KBS'][sl][:, :, i, None].float(), ub * V['UBS'][sl][:, :, i, None].float()
+        return kb.flatten(0, 1).cpu(), ub.flatten(0, 1).cpu()
+
+    def after_step(self, got, want, i):
+        """``got`` / ``want``: the outputs of the subset's rows; ``i``: the buffer index this step appended at."""
+        ref, V, sl = self.ref, self.V, self.sl
+        self.tal.out(got, want)
+        kb, ub = self._entry(i)
+        self.tal.entries(kb, ref.K[:, i])
+        self.tal.entries(ub, ref.U[:, i])
+        gb = V['GB'][sl][:, :, i].flatten(0, 1).cpu()
+        if self.exact_decay:
+            assert torch.equal(gb, ref.G[:, i]), 'cumulative decays must be bit-equal'
+        else:
+            assert torch.allclose(gb, ref.G[:, i], rtol=5e-6, atol=1e-7)
+            ref.G[:, i] = gb
+            ref.gcur = gb.clone()                          # (the fold below, if due, resets it)
+        ref.K[:, i], ref.U[:, i] = kb, ub
+        if ref.n == ref.m:
+            ref.fold()
+            codes = V['S'][sl].cpu().reshape(ref.codes.shape)
+            scales = V['SC'][sl].cpu().reshape(ref.scales.shape)
+            self.tal.fold(codes, scales, ref, self.bits)
+            ref.adopt(codes, scales)
+        n = V['NPTR'][sl][:, 0].cpu()
+        assert (n == ref.n).all(), (n, ref.n)
+
+    def verdict(self, tag, o_bound=2e-5):
+        """The small tests' bounds: outputs 2e-5, codes at most 1e-4 off and never by more than one step."""
+        t = self.tal
+        print('\n' + t.report(tag))
+        assert t.worst_o < o_bound, t.worst_o
+        assert t.code_far == 0 and t.code_mism <= 1e-4 * max(t.code_n, 1), (t.code_mism, t.code_n)
+        assert t.buf_flips <= 1e-3 * t.buf_entries, (t.buf_flips, t.buf_entries)
+        assert t.folds >= 2

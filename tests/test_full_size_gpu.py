@@ -13,19 +13,13 @@ import torch
 import statequant_amd as sq
 from oracle import states as ST
 from statequant_amd.kernels import KDASlotLayout, Mamba2SlotLayout
-from tests._util import unpack_nib
+from tests._util import SlotSync
 from tests.test_gdn_gpu import check as check_gdn, run_decode as run_gdn
 from tests.test_kda_gpu import kda_token
 from tests.test_mamba2_gpu import m2_token, params
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
-
-
-def _codes_close(views, idx, rows, ref, bits):
-    codes = views['S'][idx[rows].long()].cpu().reshape(ref.codes.shape)
-    d = (unpack_nib(codes, bits).int() - unpack_nib(ref.codes, bits).int()).abs()
-    assert d.max().item() <= 1 and (d != 0).float().mean().item() < 1e-3, ((d != 0).float().mean().item(), d.max())
 
 
 def _twins_equal(views, idx, half, live=None, written=2):
@@ -52,21 +46,22 @@ def test_mamba2_full_size_subset_and_twin_rows():
     lay.write(views, idx[half:].long(), S_half.to(DEV))
     A, D, dtb = params(gen, H)
     rows = [0, 29, 63]
-    ref = ST.Mamba2Oracle(S_half[rows].reshape(-1, DV, DK), fmt, m=m, hv=H, hk=G, buffer_bits=8)
+    ref = ST.Mamba2Oracle(S_half[rows].reshape(-1, DV, DK), fmt, m=m, hv=H, hk=G, buffer_bits=8, auto_fold=False)
+    sync = SlotSync(views, idx[rows], ref, 8, exact_decay=False)
     two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
-    worst = 0.0
-    for t in range(m + 2):                                  # through one fold and two tokens beyond
+    steps = 2 * m + 2                                       # through two folds and two tokens beyond
+    for t in range(steps):
         x, dt, Bm, C = m2_token(gen, half, H, G, DK, DV)
         out = torch.full((slots, H, DV), 7.0, device=DEV)
         lay.step(views, idx, two(x), two(dt), two(Bm), two(C), out, A.to(DEV), D.to(DEV), dtb.to(DEV))
         got = out.cpu()
         assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
-        want = ref.step(x[rows], dt[rows], Bm[rows], C[rows], A, D, dtb, True, (0., float('inf'))).view(len(rows), H, DV)
-        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        i = ref.n
+        want = ref.step(x[rows], dt[rows], Bm[rows], C[rows], A, D, dtb, True, (0., float('inf')))
+        sync.after_step(got[rows].reshape(want.shape), want, i)
         assert torch.equal(views['NPTR'][idx.long(), :H].cpu(), torch.full((slots, H), (t + 1) % m, dtype=torch.int32))
-    assert worst < 5e-3, worst                 # no re-sync with the oracle here: a flipped buffer entry persists
-    _twins_equal(views, idx, half)
-    _codes_close(views, idx, rows, ref, 8)
+    sync.verdict('mamba2 full size')
+    _twins_equal(views, idx, half, written=steps % m)
 
 
 def test_kda_full_size_subset_and_twin_rows():
@@ -82,22 +77,23 @@ def test_kda_full_size_subset_and_twin_rows():
     lay.write(views, idx[:half].long(), S_half.to(DEV))
     lay.write(views, idx[half:].long(), S_half.to(DEV))
     rows = [0, 57, 127]
-    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8)
+    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8, auto_fold=False)
+    sync = SlotSync(views, idx[rows], ref, 4)
     two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
     flat = lambda x: x[rows].reshape(len(rows) * H, *x.shape[2:])          # noqa: E731
-    worst = 0.0
-    for t in range(m + 2):
+    steps = 2 * m + 2
+    for t in range(steps):
         q, k, v, g, beta = kda_token(gen, half, H, D, D)
         out = torch.full((slots, H, D), 7.0, device=DEV)
         lay.step(views, idx, two(q), two(k), two(v), two(g), two(beta), out)
         got = out.cpu()
         assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
-        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta)).view(len(rows), H, D)
-        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        i = ref.n
+        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta))
+        sync.after_step(got[rows].reshape(want.shape), want, i)
         assert torch.equal(views['NPTR'][idx.long(), :H].cpu(), torch.full((slots, H), (t + 1) % m, dtype=torch.int32))
-    assert worst < 5e-3, worst
-    _twins_equal(views, idx, half)
-    _codes_close(views, idx, rows, ref, 4)
+    sync.verdict('kda full size')
+    _twins_equal(views, idx, half, written=steps % m)
 
 
 def test_kda_ragged_variant_with_padding_rows():
@@ -125,25 +121,26 @@ def test_kda_ragged_variant_with_padding_rows():
     untouched[slot[slot > 0]] = False                                       # slot 0 and the slots no row points at
     before = blob[untouched.to(DEV)].clone()
     rows = [0, 57]
-    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8)
+    ref = ST.KDAOracle(S_half[rows].reshape(-1, D, D), fmt, m=m, hv=H, buffer_bits=8, auto_fold=False)
+    sync = SlotSync(views, idx[rows], ref, 4)
     two = lambda x: torch.cat([x, x]).to(DEV)              # noqa: E731
     flat = lambda x: x[rows].reshape(len(rows) * H, *x.shape[2:])          # noqa: E731
-    worst = 0.0
-    for t in range(m + 2):
+    steps = 2 * m + 2
+    for t in range(steps):
         q, k, v, g, beta = kda_token(gen, half, H, D, D)
         out = torch.full((nrows, H, D), 7.0, device=DEV)
         lay.step(views, idx, two(q), two(k), two(v), two(g), two(beta), out)
         got = out.cpu()
         assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
         assert torch.equal(got[:half][dead], torch.zeros(int(dead.sum()), H, D)), 'padding rows must give zeros'
-        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta)).view(len(rows), H, D)
-        worst = max(worst, ((got[rows] - want).abs().max() / want.abs().max()).item())
+        i = ref.n
+        want = ref.step(flat(q), flat(k), flat(v), flat(g), flat(beta))
+        sync.after_step(got[rows].reshape(want.shape), want, i)
         n_live = views['NPTR'][idx[:half][live].long(), :H].cpu()
         assert torch.equal(n_live, torch.full((int(live.sum()), H), (t + 1) % m, dtype=torch.int32))
-    assert worst < 5e-3, worst
+    sync.verdict('kda 20 heads, d 96, 40 % padding rows')
     assert torch.equal(blob[untouched.to(DEV)], before), 'a padding row wrote to a slot'
-    _twins_equal(views, idx, half, live=live.to(DEV))
-    _codes_close(views, idx, rows, ref, 4)
+    _twins_equal(views, idx, half, live=live.to(DEV), written=steps % m)
 
 
 @pytest.mark.parametrize('m,bb', [(8, 8), (8, 16)])

@@ -13,14 +13,17 @@ import torch
 import statequant_amd as sq
 from oracle import states as ST
 from statequant_amd.kernels import SlotLayout
-from tests._util import gdn_token, unpack_nib
+from tests._util import SlotSync, gdn_token
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
 
 
-@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 32)])
-def test_full_size_subset_and_twin_rows(fmt):
+@pytest.mark.parametrize('fmt,warm', [((8, 'k', 128), 0), ((4, 'k', 32), 0), ((8, 'k', 128), 64)])
+def test_full_size_subset_and_twin_rows(fmt, warm):
+    """warm = 0: states written from fp32 (``write``).  warm = 64: the benchmark's situation -- every slot starts at
+    zero and has been through 64 kernel steps (8 folds) before the comparison begins; the oracle then takes over the
+    slots' codes and scales (the buffers are empty at a multiple of m) and follows for two more fold periods."""
     HV, HK, D, m, slots = 32, 16, 128, 8, 256
     lay = SlotLayout(sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
     views = lay.views(lay.alloc(slots + 1, DEV))
@@ -28,35 +31,45 @@ def test_full_size_subset_and_twin_rows(fmt):
     half = slots // 2
     perm = (torch.randperm(slots, generator=gen) + 1)
     idx = perm.to(torch.int32).to(DEV)                                    # row r works on slot perm[r]
-    S_half = torch.randn(half, HV, D, D, generator=gen) * 0.3              # value-major; rows r, r + half share it
-    lay.write(views, idx[:half].long(), S_half.to(DEV))
-    lay.write(views, idx[half:].long(), S_half.to(DEV))
+    two = lambda x: torch.cat([x, x]).to(DEV)                             # noqa: E731
     check_rows = [0, 57, 127]                                             # rows checked against the oracle
-    ref = ST.GDNOracle(S_half[check_rows].reshape(-1, D, D), fmt, m=m, hv=HV, hk=HK, buffer_bits=8)
-    worst = 0.0
-    for t in range(m + 2):                                                # through one fold and two tokens beyond
+    sl = idx[check_rows]
+    if warm:
+        for t in range(warm):
+            q, k, v, g, beta = gdn_token(gen, half, HV, HK, D, D)
+            out = torch.empty(slots, HV, D, device=DEV)
+            lay.step(views, idx, two(q), two(k), two(v), out, D ** -0.5, g=two(g), beta=two(beta))
+        assert int(views['NPTR'][idx.long(), :HV].abs().max()) == 0 and torch.isfinite(out).all()
+        ref = ST.GDNOracle(torch.zeros(len(check_rows) * HV, D, D), fmt, m=m, hv=HV, hk=HK, buffer_bits=8, auto_fold=False)
+        ref.adopt(views['S'][sl.long()].cpu().reshape(ref.codes.shape), views['SC'][sl.long()].cpu().reshape(ref.scales.shape))
+        assert float(ref.S0.abs().max()) > 0.1                            # a state worth the name
+    else:
+        S_half = torch.randn(half, HV, D, D, generator=gen) * 0.3          # value-major; rows r, r + half share it
+        lay.write(views, idx[:half].long(), S_half.to(DEV))
+        lay.write(views, idx[half:].long(), S_half.to(DEV))
+        ref = ST.GDNOracle(S_half[check_rows].reshape(-1, D, D), fmt, m=m, hv=HV, hk=HK, buffer_bits=8, auto_fold=False)
+    sync = SlotSync(views, sl, ref, fmt[0])
+    steps = 2 * m + 2                                                     # through two folds and two tokens beyond
+    for t in range(steps):
         q, k, v, g, beta = gdn_token(gen, half, HV, HK, D, D)
-        two = lambda x: torch.cat([x, x]).to(DEV)                         # noqa: E731
         out = torch.full((slots, HV, D), 7.0, device=DEV)
         lay.step(views, idx, two(q), two(k), two(v), out, D ** -0.5, g=two(g), beta=two(beta))
         got = out.cpu()
         assert torch.equal(got[:half], got[half:]), f'twin rows differ at step {t}'
+        i = ref.n
         want = ref.step(q[check_rows].reshape(-1, D), k[check_rows].reshape(-1, D), v[check_rows].reshape(-1, D),
-                        g[check_rows].reshape(-1), beta[check_rows].reshape(-1), D ** -0.5).view(len(check_rows), HV, D)
-        worst = max(worst, ((got[check_rows] - want).abs().max() / want.abs().max()).item())
+                        g[check_rows].reshape(-1), beta[check_rows].reshape(-1), D ** -0.5)
+        sync.after_step(got[check_rows].reshape(want.shape), want, i)
         n = (t + 1) % m
         assert torch.equal(views['NPTR'][idx.long(), :HV].cpu(), torch.full((slots, HV), n, dtype=torch.int32))
-    assert worst < 5e-3, worst                 # no re-sync with the oracle here: a flipped buffer entry persists
+    sync.verdict(f'gdn {fmt} full size, {"after 64 kernel steps" if warm else "from written states"}')
     for f in ('S', 'SC', 'GCUR'):
         a, b = views[f][idx[:half].long()], views[f][idx[half:].long()]
         assert torch.equal(a, b), f
-    w = 2                                                                 # buffer slots written since the fold
+    w = steps % m                                                         # buffer slots written since the last fold
     for f in ('UB', 'KB', 'GB', 'UBS', 'KBS'):
         a, b = views[f][idx[:half].long()][:, :, :w], views[f][idx[half:].long()][:, :, :w]
         assert torch.equal(a, b), f
-    codes = views['S'][idx[check_rows].long()].cpu().reshape(ref.codes.shape)
-    d = (unpack_nib(codes, fmt[0]).int() - unpack_nib(ref.codes, fmt[0]).int()).abs()
-    assert d.max().item() <= 1 and (d != 0).float().mean().item() < 1e-3, ((d != 0).float().mean().item(), d.max())
 
 
 def test_graph_replay_matches_eager():
