@@ -59,7 +59,6 @@ __device__ __forceinline__ float vec_elem(const uint32_t (&w)[NE], int dt, int t
 // Everything a wavefront loads for one item, as issued loads (raw bits; nothing here waits for memory).
 template <class T, class Q>
 struct GdnLoads {
-    v4u cw[Q::NB][Q::NLD];                 // its row blocks
     uint16_t sc[Q::NB][T::NG];             // scales of rows (block bi, lane % 32)
     Raw4<T::QBUF> uraw[Q::UT], kraw[Q::KT];
     uint16_t kbs[Q::KT], ubs;
@@ -74,11 +73,13 @@ struct GdnLoads {
 // a, b and fp32 A_log, dt_bias.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift,
+void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
+                     uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride,
                      SQ_TL_PARAM const GdnParams p) {
     SQ_MARK(0);                                                   // entry
-    // the leading arguments (copies of fields of `p`) are what the slot index load needs: as separate scalar
-    // arguments they are preloaded into registers at wave launch, so that load goes out first thing
+    // the leading arguments (copies of fields of `p`) are what the slot index load, the fill counter and the row blocks
+    // need: as separate scalar arguments they are preloaded into registers at wave launch, so those requests go out
+    // without waiting for the argument block
     constexpr bool FIX = SPEC > 0;
     const int q_dt = FIX ? int(BF16) : p.q_dt, k_dt = FIX ? int(BF16) : p.k_dt, v_dt = FIX ? int(BF16) : p.v_dt;
     const int out_dt = FIX ? int(BF16) : p.out_dt;
@@ -90,7 +91,6 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
     using L = QuadLds<T, NB, GH, 2, 2>;
     constexpr int DK = T::DK, DV = T::DV, NW = Q::NW, NWH = Q::NWH, MM = T::MMAX, NE = Q::NE, NG = T::NG;
     constexpr int RQ = 1 % NW, RK = 3 % NW, RX = 2 % NW;          // which wavefront plays which shared role
-    constexpr bool DMA = SQ_QUAD_DMA != 0;                        // row blocks loaded straight into LDS
     __shared__ __attribute__((aligned(16))) uint8_t lds[L::BYTES];
     uint8_t* lds_kbr = lds + L::KBR;
     float* lds_xn = reinterpret_cast<float*>(lds + L::XN);
@@ -130,10 +130,10 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
     const int n32 = lane & 31, kb = lane >> 5;
     // the row of the head this lane finishes after the pass (NB = 2: the wavefront's halves take a block each)
     const int row = (wh * NB + (NB == 2 ? kb : 0)) * T::MR + n32;
-    const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);        // chunk `lane` of a 1 KB piece in the LDS image
 
-    // ---- issue every load: first the token's own operands (their addresses need the batch row only) ...
     GdnLoads<T, Q> F;
+    // ---- issue every load: first the token's own operands (their addresses need the batch row only: they go out
+    //      while the slot index is on its way, and being older than the row blocks they are back before them) ...
     {
         const uint32_t b = tid.b, h = tid.h;
         if constexpr (RQ == RK) {                                 // a single wavefront carries both vectors
@@ -165,40 +165,28 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
         return;
     }
     SQ_MARK(2);                                                   // slot known, the token's loads issued
-    // ... then the slot's side.  The counters and the row blocks go out first and by themselves: the scheduling
-    // barrier behind them keeps the address arithmetic of the other eight fields, and the first use of the fill count,
-    // from being scheduled in among them (the compiler had put half of the row-block loads behind the wait for the
-    // fill count).
-    {
-        const uint32_t seq = slot, h = tid.h;
-        F.gcur = *field(p.st.GCUR, seq, p.st.sGC, h);
-        const uint8_t* Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
-        if constexpr (!DMA) F.np = *field(p.st.NPTR, seq, p.st.sN, h);
-        SQ_MARK(3);                                               // counters issued
-        if constexpr (DMA) {
-            // the fill count, then the row blocks straight into their LDS image (sq_quad.cuh)
-            F.np = quad_dma_counter(field(p.st.NPTR, seq, p.st.sN, h));
-            quad_dma_blocks<Q, NB>(Sh + wh * NB * Q::BLK, my_codes, lane);
-        } else {
-#pragma unroll
-            for (int bi = 0; bi < NB; ++bi)
-#pragma unroll
-                for (int t = 0; t < Q::NLD; ++t)
-                    F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    SQ_MARK(4);                                                   // row blocks issued
+    // ... then the slot's big side, from the preloaded arguments alone: the row blocks, straight into their LDS image,
+    // and the fill counter (a scalar load; sq_quad.cuh) -- behind the row blocks, because the first wait for any
+    // scalar load, the argument block's included, waits for it as well ...
+    quad_dma_blocks<Q, NB>(field(codes, uint32_t(slot), codes_stride, uint32_t(tid.h) * (DV * T::ROW_BYTES)) + wh * NB * Q::BLK,
+                           my_codes, lane);
+    SQ_MARK(3);                                                   // row blocks issued
+    F.np = quad_dma_counter(field(counters, uint32_t(slot), counters_stride, uint32_t(tid.h)));
+    __builtin_amdgcn_sched_barrier(0);
+    SQ_MARK(4);                                                   // counter issued
+    // ... and the rest of the slot: running decay, scales, and -- once the fill counter is here -- the live part of
+    // the decode buffer
     const GdnAddr<T> A = gdn_addr<T>(p, tid, slot);
     void* const outp = advance(p.out, out_dt, A.obase);
+    F.gcur = *A.gcp;
     {
-        if constexpr (DMA) quad_dma_counter_wait<Q, NB>(F.np);      // before anything else is requested
 #pragma unroll
         for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
             for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(A.SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
         // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count,
         // requested ahead of the row blocks, is here by now
+        quad_dma_counter_wait(F.np);
         const uint32_t nfill = uint32_t(F.np & (m - 1));
         const uint32_t nl = nfill > 0 ? nfill : 1u;
         // buffered values of this wavefront's rows: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
@@ -299,14 +287,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
         lds_gbf[lane] = F.gbl;
         if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
     }
-    if constexpr (!DMA) {
-#pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
-#pragma unroll
-            for (int t = 0; t < Q::NLD; ++t)
-                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
-    }
-    if constexpr (DMA) quad_dma_landed();
+    quad_dma_landed();                                             // the row blocks are in LDS
     const bool full = n == m - 1;
     SQ_MARK(6);                                                   // roles done, every load landed in LDS
     lds_barrier();
@@ -548,10 +529,11 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
 #ifdef SQ_TIMELINE
     const SqTimelineBuf tl = sq_timeline_buffer();
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, tl.p, tl.cap, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
+                       tl.p, tl.cap, p);
 #else
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, p);
 #endif
     return int(hipGetLastError());
 }

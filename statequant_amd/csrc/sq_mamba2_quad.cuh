@@ -17,7 +17,6 @@ namespace sq {
 
 template <class T, class Q>
 struct Mamba2Loads {
-    v4u cw[Q::NB][Q::NLD];                 // its row blocks
     uint16_t sc[Q::NB][T::NG];             // scales of rows (block bi, lane % 32)
     Raw4<T::QBUF> uraw[Q::UT], kraw[Q::KT];
     uint16_t kbs[Q::KT], ubs;
@@ -30,7 +29,8 @@ struct Mamba2Loads {
 // dt_bias, head counts that are powers of two.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const Mamba2Params p) {
+void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
+                        uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, const Mamba2Params p) {
     constexpr bool FIX = SPEC > 0;
     const int x_dt = FIX ? int(BF16) : p.x_dt, B_dt = FIX ? int(BF16) : p.B_dt, C_dt = FIX ? int(BF16) : p.C_dt;
     const int out_dt = FIX ? int(BF16) : p.out_dt, dt_dt = FIX ? int(F32) : p.dt_dt, A_dt = FIX ? int(F32) : p.A_dt;
@@ -78,10 +78,10 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
     const int n32 = lane & 31, kb = lane >> 5;
     // the row of the head this lane finishes after the pass (NB = 2: the wavefront's halves take a block each)
     const int row = (wh * NB + (NB == 2 ? kb : 0)) * T::MR + n32;
-    const int swz0 = swz<Q>(lane / Q::CPR, lane % Q::CPR);        // chunk `lane` of a 1 KB piece in the LDS image
 
-    // ---- issue every load: first the token's own operands (their addresses need the batch row only) ----
     Mamba2Loads<T, Q> F;
+    // ---- issue every load: first the token's own operands (their addresses need the batch row only; being older
+    //      than the row blocks they are back before them) ...
     if constexpr (RQ == RK) {                                     // a single wavefront carries both vectors
         if (w == RQ) {
             load_vec<NE>(advance(p.C, C_dt, uint64_t(uint32_t(b)) * p.s_C + hk * DK), C_dt, lane, F.xr);
@@ -105,40 +105,30 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
         for (int r = wh * WAVE + lane; r < DV; r += NWH * WAVE) store_f(outp, out_dt, r, 0.0f);
         return;
     }
-    // ... and the slot's side
-    // the counters and the row blocks first and by themselves: the scheduling barrier behind them keeps the address
-    // arithmetic of the other fields, and the first use of the fill count, from being scheduled in among them
+    // ... then the slot's big side, from the preloaded leading arguments alone: the row blocks, straight into their
+    // LDS image, and the fill counter (a scalar load; sq_quad.cuh) behind them ...
+    quad_dma_blocks<Q, NB>(field(codes, uint32_t(slot), codes_stride, h * (DV * T::ROW_BYTES)) + wh * NB * Q::BLK, my_codes, lane);
+    F.np = quad_dma_counter(field(counters, uint32_t(slot), counters_stride, h));
+    __builtin_amdgcn_sched_barrier(0);
+    // ... and the rest of the slot
     const uint32_t seq = slot, um = m;
     uint8_t* const Sh = field(p.st.S, seq, p.st.sS, h * (DV * T::ROW_BYTES));
     float* const gcp = field(p.st.GCUR, seq, p.st.sGC, h);
     int32_t* const np = field(p.st.NPTR, seq, p.st.sN, h);
-    constexpr bool DMA = SQ_QUAD_DMA != 0;                        // row blocks loaded straight into LDS (sq_quad.cuh)
     F.gcur = *gcp;
-    if constexpr (DMA) {
-        F.np = quad_dma_counter(np);
-        quad_dma_blocks<Q, NB>(Sh + wh * NB * Q::BLK, my_codes, lane);
-    } else {
-        F.np = *np;
-#pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
-#pragma unroll
-            for (int t = 0; t < Q::NLD; ++t)
-                F.cw[bi][t] = stream_load(reinterpret_cast<const v4u*>(Sh + (wh * NB + bi) * Q::BLK + t * 1024 + lane * 16));
-    }
-    __builtin_amdgcn_sched_barrier(0);
     uint16_t* const SCh = field(p.st.SC, seq, p.st.sSC, h * T::SC_ELEMS);
     uint8_t* const KBp = p.st.KB + (uint64_t(seq) * p.st.sKB + hk * um * DK) * T::BE;
     uint8_t* const UBp = p.st.UB + (uint64_t(seq) * p.st.sUB + h * um * DV) * T::BE;
     uint16_t* const KBSp = field(p.st.KBS, seq, p.st.sKBS, hk * um);
     uint16_t* const UBSp = field(p.st.UBS, seq, p.st.sUBS, h * um);
     float* const GBh = field(p.st.GB, seq, p.st.sGB, h * um);
-    if constexpr (DMA) quad_dma_counter_wait<Q, NB>(F.np);          // before anything else is requested
 #pragma unroll
     for (int bi = 0; bi < NB; ++bi)
 #pragma unroll
         for (int g = 0; g < NG; ++g) F.sc[bi][g] = stream_load(SCh + uint32_t(((wh * NB + bi) * T::MR + n32) * NG + g));
     // the buffer, live slots only (the others repeat the last live one: no new memory traffic); the fill count,
     // requested ahead of the row blocks, is here by now
+    quad_dma_counter_wait(F.np);
     const uint32_t nfill = uint32_t(F.np & (m - 1));
     const uint32_t nl = nfill > 0 ? nfill : 1u;
     // buffered values of this wavefront's rows: lane (slot = lane / LU + SU t, rows 4 (lane % LU) ..)
@@ -228,15 +218,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
         lds_gbf[lane] = F.gbl;
         if constexpr (T::QBUF) lds_ubsf[lane] = f16_to_f32(F.ubs);
     }
-    if constexpr (DMA) {
-        quad_dma_landed();
-    } else {
-#pragma unroll
-        for (int bi = 0; bi < NB; ++bi)
-#pragma unroll
-            for (int t = 0; t < Q::NLD; ++t)
-                *reinterpret_cast<v4u*>(my_codes + bi * Q::BLK + t * 1024 + swz0) = F.cw[bi][t];
-    }
+    quad_dma_landed();                                             // the row blocks are in LDS
     const bool full = n == m - 1;
     lds_barrier();
 
@@ -449,7 +431,7 @@ int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     Mamba2Params p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p);
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, p);
     return int(hipGetLastError());
 }
 

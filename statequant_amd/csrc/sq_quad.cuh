@@ -258,21 +258,23 @@ __device__ __forceinline__ float quad_block_pass(const uint8_t* blk, const v4i (
 // row still cover the row's lines, in another order.
 //
 // The compiler books a load-to-LDS as touching both memories and forces every wait that follows it down to "nothing
-// outstanding", which would drain the row blocks before the fill counter (requested ahead of them) can be used.  So
-// the counter and the row blocks are requested in assembly, invisible to that bookkeeping, with the one wait in
-// between written by hand: loads complete in order, the counter is older than the N block loads, so it is here once
-// at most N loads are outstanding.  Nothing else may be requested between `quad_dma_counter` and
-// `quad_dma_counter_wait` (the compiler merges and reorders the loads it knows of; these it does not).  Every later
-// wait the compiler places for a younger load covers the block loads as well; `quad_dma_landed` states it.
+// outstanding", which would drain the row blocks before anything requested around them can be used.  So they are
+// requested in assembly, invisible to that bookkeeping.  Loads complete in order, so every wait the compiler places
+// for a load requested after them covers them as well; `quad_dma_landed` states it where the image is first read.
+//
+// The slot's fill counter decides which part of the decode buffer is requested, so it sits in front of those
+// requests.  It is fetched with a SCALAR load: scalar loads have a counter of their own, so waiting for it does not
+// wait for the row blocks requested behind it.  (The scalar cache is invalidated at every kernel start and the counter
+// was written by an earlier launch; within a launch a slot's counter is written by its own workgroup only, at the
+// end.)  The compiler would use a vector load here, because the same address is stored to later in the kernel.
 // ---------------------------------------------------------------------------------------------------------------
-#ifndef SQ_QUAD_DMA
-#define SQ_QUAD_DMA 1
-#endif
-
 __device__ __forceinline__ int quad_dma_counter(const int32_t* p) {
     int v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(v) : "s"(p) : "memory");
     return v;
+}
+__device__ __forceinline__ void quad_dma_counter_wait(int& counter) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(counter) :: "memory");
 }
 // NBLK row blocks of this wavefront: `src` their first byte in memory, `dst` their LDS image.  Every 1 KB piece gets
 // its own address pair and LDS base on purpose: the four pieces of a block behind one address with the instruction's
@@ -293,12 +295,6 @@ __device__ __forceinline__ void quad_dma_blocks(const uint8_t* src, uint8_t* dst
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
                          :: "v"(g), "s"(at) : "memory", "m0");
         }
-}
-template <class Q, int NBLK>
-__device__ __forceinline__ void quad_dma_counter_wait(int& counter) {
-    constexpr int YOUNGER = NBLK * Q::NLD;
-    static_assert(YOUNGER < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(counter) : "n"(YOUNGER) : "memory");
 }
 __device__ __forceinline__ void quad_dma_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
