@@ -461,7 +461,8 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--instances', default='', metavar='LIST',
                     help='comma-separated exclusions handed to sq_debug_select, for same-machine comparisons of the '
-                         'kernel instances that can serve the workload: no-specialised, no-group')
+                         'kernel instances that can serve the workload: no-specialised, no-group, '
+                         'lds-pad=<bytes> (unused dynamic LDS per workgroup: fewer resident workgroups)')
     ap.add_argument('--cpu-budget', type=float, default=20.0)
     ap.add_argument('--op', default='step', choices=['step', 'write', 'read'],
                     help="step: the decode step (the headline); write / read: the prefill-side pack and read kernels "
@@ -482,8 +483,9 @@ def main():
     if a.instances:
         from statequant_amd.kernels import _hip
         off = {x.strip() for x in a.instances.split(',') if x.strip()}
-        assert off <= {'no-specialised', 'no-group'}, off
-        _hip.select_instances(no_specialised='no-specialised' in off, no_group_kernel='no-group' in off)
+        pad = sum(int(x.split('=')[1]) for x in off if x.startswith('lds-pad='))
+        assert {x for x in off if not x.startswith('lds-pad=')} <= {'no-specialised', 'no-group'}, off
+        _hip.select_instances(no_specialised='no-specialised' in off, no_group_kernel='no-group' in off, lds_pad_bytes=pad)
     m = a.m
     if a.slots:
         w = WORKLOADS[a.workload]

@@ -217,9 +217,12 @@ const char* sq_last_error(void);
  * with the serving dtypes compiled in or the general one; a workgroup per key head or a wavefront per head; how many
  * value heads a workgroup takes).  Results do not depend on the choice up to the accumulation order of fp32 sums; the
  * twin tests and the profiling scripts use this to compare instances.  Non-zero no_specialised / no_group_kernel
- * exclude those instances, max_heads_per_workgroup <= 0 means no cap.  Process-wide, takes effect on the next call;
- * the library never reads the environment for it.  Pure host code. */
-void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup);
+ * exclude those instances, max_heads_per_workgroup <= 0 means no cap, lds_pad_bytes > 0 adds that much unused dynamic
+ * LDS to the workgroup-per-key-head launches (fewer resident workgroups per compute unit; static + dynamic must stay
+ * within 64 KB or the launch fails).  Process-wide, takes effect on the next call; the library reads no environment
+ * variable.  Pure host code. */
+void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup,
+                     int32_t lds_pad_bytes);
 
 /* 1 if a kernel is built for this layout (family: 0 GDN, 1 KDA, 2 Mamba2), else 0. Pure host code. */
 int sq_supported(int family, const sq_layout* lay);

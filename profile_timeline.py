@@ -32,8 +32,8 @@ from statequant_amd.kernels import _hip  # noqa: E402
 MARKS_KDA = ['entry', 'slot known, token loads issued', 'fill count here, every load issued',
              'vectors, scales, buffered values staged', 'keys and decays here, coefficients done', 'state pass done',
              'outputs stored', 'appended', 'folded (full buffer), counters advanced']
-MARKS = ['entry', 'item known (leading arguments here)', 'slot known, token loads issued', 'counters issued',
-         'row blocks issued', 'fill count here, buffer loads issued', 'roles done, all loads landed in LDS',
+MARKS = ['entry', 'item known (leading arguments here)', 'slot known, token loads issued', 'row blocks issued',
+         'fill counter issued', 'fill count here, buffer loads issued', 'roles done, all loads landed in LDS',
          'first barrier passed', 'state pass done', 'buffer dot products done', 'second barrier passed',
          'output stored', 'largest |u| known (barrier)', 'appended, counters advanced', 'fold done and stored']
 TICK_US = 0.01                                               # s_memrealtime counts at 100 MHz
@@ -88,6 +88,11 @@ def report(workload, step, t, nwg, fam, m=8):
     for k in range(last):
         lines.append(f'  {marks[k]:<38} -> {marks[k + 1]:<38} {d[:, :, k].mean():6.2f} {np.median(d[:, :, k]):6.2f} '
                      f'{np.percentile(d[:, :, k], 90):6.2f}')
+    first = T[:, 0, 0] < 1.0                                 # workgroups that the launch starts with
+    if first.any() and not first.all():
+        lines.append(f'mean of each interval, the {int(first.sum())} workgroups resident from the start / the others:')
+        lines.append('  from the start: ' + ' '.join(f'{d[first][:, :, k].mean():5.2f}' for k in range(last)))
+        lines.append('  the others:     ' + ' '.join(f'{d[~first][:, :, k].mean():5.2f}' for k in range(last)))
     if waves > 1:
         lines.append('mean of each interval by wavefront of the workgroup (1 and 3: q and k vectors; 0 and 2: gates; '
                      '2: key append):')
@@ -99,6 +104,10 @@ def report(workload, step, t, nwg, fam, m=8):
     lines.append('workgroups ending per 2 us:   ' + ' '.join(str(x) for x in np.histogram(en, edges)[0]))
     lines.append('resident workgroups at t us:  ' + ' '.join(f'{x:.0f}:{int(((st <= x) & (en > x)).sum())}'
                                                             for x in np.arange(1, T[:, :, :last + 1].max(), 2.0)))
+    if fam == 'gdn':                                         # when the row blocks are asked for and when they are all here
+        e1 = np.arange(0, T[:, :, :last + 1].max() + 1, 1.0)
+        lines.append('wavefronts asking for their row blocks per 1 us: ' + ' '.join(str(x) for x in np.histogram(T[:, :, 3], e1)[0]))
+        lines.append('wavefronts with every load landed per 1 us:      ' + ' '.join(str(x) for x in np.histogram(T[:, :, 6], e1)[0]))
     return lines
 
 

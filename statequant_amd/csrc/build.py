@@ -209,12 +209,14 @@ def generate():
          'namespace sq {',
          '// Which instance serves a call when several could (results do not depend on it): set through sq_debug_select,',
          '// never read from the environment.',
-         'static std::atomic<int> g_no_spec{0}, g_no_quad{0}, g_ghmax{64};',
-         'void select_instances(int no_spec, int no_quad, int ghmax) {',
+         'static std::atomic<int> g_no_spec{0}, g_no_quad{0}, g_ghmax{64}, g_lds_pad{0};',
+         'void select_instances(int no_spec, int no_quad, int ghmax, int lds_pad) {',
          '    g_no_spec.store(no_spec != 0);',
          '    g_no_quad.store(no_quad != 0);',
          '    g_ghmax.store(ghmax > 0 ? ghmax : 64);',
-         '}']
+         '    g_lds_pad.store(lds_pad > 0 ? lds_pad : 0);',
+         '}',
+         'int quad_lds_pad() { return g_lds_pad.load(std::memory_order_relaxed); }']
     for fam, rows in CASES.items():
         P = PARAMS[fam]
         d.append(f'template <class T, int SPEC> int launch_{fam}(const {P}&, hipStream_t);')

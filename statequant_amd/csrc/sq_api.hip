@@ -117,8 +117,9 @@ extern "C" {
 
 int sq_abi_version(void) { return SQ_ABI_VERSION; }
 
-void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup) {
-    sq::select_instances(no_specialised, no_group_kernel, max_heads_per_workgroup);
+void sq_debug_select(int32_t no_specialised, int32_t no_group_kernel, int32_t max_heads_per_workgroup,
+                     int32_t lds_pad_bytes) {
+    sq::select_instances(no_specialised, no_group_kernel, max_heads_per_workgroup, lds_pad_bytes);
 }
 
 const char* sq_strerror(int code) {

@@ -74,7 +74,7 @@ struct GdnLoads {
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
 void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
-                     uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride,
+                     uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, uint32_t start_ramp,
                      SQ_TL_PARAM const GdnParams p) {
     SQ_MARK(0);                                                   // entry
     // the leading arguments (copies of fields of `p`) are what the slot index load, the fill counter and the row blocks
@@ -168,6 +168,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
     // ... then the slot's big side, from the preloaded arguments alone: the row blocks, straight into their LDS image,
     // and the fill counter (a scalar load; sq_quad.cuh) -- behind the row blocks, because the first wait for any
     // scalar load, the argument block's included, waits for it as well ...
+    quad_start_wait<Q, WPE>(start_ramp);                  // the launch's first workgroups: spread over a ramp
     quad_dma_blocks<Q, NB>(field(codes, uint32_t(slot), codes_stride, uint32_t(tid.h) * (DV * T::ROW_BYTES)) + wh * NB * Q::BLK,
                            my_codes, lane);
     SQ_MARK(3);                                                   // row blocks issued
@@ -526,14 +527,16 @@ template <class T, int NB, int GH, int WPE, int SPEC>
 int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     GdnParams p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
+    const uint32_t grid = uint32_t(p.rows) * uint32_t(p.hv / GH);
+    const uint32_t stag = quad_start_ramp<Quad<T, NB, GH>, WPE>(grid);
 #ifdef SQ_TIMELINE
     const SqTimelineBuf tl = sq_timeline_buffer();
-    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
+    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag,
                        tl.p, tl.cap, p);
 #else
-    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, p);
+    hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag, p);
 #endif
     return int(hipGetLastError());
 }

@@ -30,7 +30,8 @@ struct Mamba2Loads {
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
 void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
-                        uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, const Mamba2Params p) {
+                        uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, uint32_t start_ramp,
+                        const Mamba2Params p) {
     constexpr bool FIX = SPEC > 0;
     const int x_dt = FIX ? int(BF16) : p.x_dt, B_dt = FIX ? int(BF16) : p.B_dt, C_dt = FIX ? int(BF16) : p.C_dt;
     const int out_dt = FIX ? int(BF16) : p.out_dt, dt_dt = FIX ? int(F32) : p.dt_dt, A_dt = FIX ? int(F32) : p.A_dt;
@@ -107,6 +108,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
     }
     // ... then the slot's big side, from the preloaded leading arguments alone: the row blocks, straight into their
     // LDS image, and the fill counter (a scalar load; sq_quad.cuh) behind them ...
+    quad_start_wait<Q, WPE>(start_ramp);                  // the launch's first workgroups: spread over a ramp
     quad_dma_blocks<Q, NB>(field(codes, uint32_t(slot), codes_stride, h * (DV * T::ROW_BYTES)) + wh * NB * Q::BLK, my_codes, lane);
     F.np = quad_dma_counter(field(counters, uint32_t(slot), counters_stride, h));
     __builtin_amdgcn_sched_barrier(0);
@@ -430,8 +432,10 @@ template <class T, int NB, int GH, int WPE, int SPEC>
 int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     Mamba2Params p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
-    hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(p.rows * (p.hv / GH)), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, p);
+    const uint32_t grid = uint32_t(p.rows) * uint32_t(p.hv / GH);
+    hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
+                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
+                       quad_start_ramp<Quad<T, NB, GH>, WPE>(grid), p);
     return int(hipGetLastError());
 }
 

@@ -178,6 +178,7 @@ int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
 int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
 int dispatch_gga(const GgaParams& p, int op, hipStream_t stream, bool run);      // op: 0 step, 1 store, 2 load
 // Diagnostic choice among the instances that can serve a step call (behind sq_debug_select of the C ABI).
-void select_instances(int no_spec, int no_quad, int ghmax);
+void select_instances(int no_spec, int no_quad, int ghmax, int lds_pad);
+int quad_lds_pad();                                       // unused dynamic LDS added to the workgroup kernels' launches
 
 }  // namespace sq

@@ -49,13 +49,31 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// Diagnostic switch: SQ_LDS_PAD=<bytes> in the environment adds that much unused dynamic LDS to every launch of the
-// workgroup kernels, so that a compute unit holds fewer workgroups (static + dynamic LDS must stay within 64 KB) --
-// for measuring how the step time depends on the number of resident workgroups.  Read once per process.
-inline int quad_lds_pad() {
-    static const int pad = getenv("SQ_LDS_PAD") ? atoi(getenv("SQ_LDS_PAD")) : 0;
-    return pad > 0 ? pad : 0;
+// The start of a launch.  Every compute unit takes as many workgroups as its LDS admits, all at once, so all of them
+// ask for their row blocks together, get them together, and compute together while memory idles until their
+// successors have started: the workgroups the launch starts with (blockIdx below the resident number) therefore hold
+// their row-block requests back by a ramp of blockIdx x `ramp` / 256 sleeps of 64 clocks, which spreads the first
+// round's requests over about the time memory needs to serve them.  Measured on one machine, int8 rows (four
+// workgroups per compute unit): 32.65 -> 32.08 us per launch with 32 (a stepped ramp of the same slope alike), 24:
+// 32.28, 40 and more: slower than none; the Mamba2 step 31.35 -> 31.15, sequences out of step 35.9 -> 35.5, 512 slots
+// 62.6 -> 61.9, 128 slots 19.1 -> 18.7.  With six smaller workgroups per compute unit (int4) no ramp helped, and a
+// launch of less than two rounds has nothing behind the first to gain from (64 slots: 11.38 -> 11.45), so the
+// launchers pass 0 for those.
+constexpr unsigned COMPUTE_UNITS = 256;                    // MI355X
+template <class Q, int WPE>
+inline uint32_t quad_start_ramp(uint32_t grid) {
+    constexpr uint32_t per_cu = WPE * 4 / Q::NW;           // resident workgroups per compute unit
+    return (per_cu <= 4 && grid >= 2 * COMPUTE_UNITS * per_cu) ? 32u : 0u;
 }
+template <class Q, int WPE>
+__device__ __forceinline__ void quad_start_wait(uint32_t ramp) {
+    if (ramp != 0 && blockIdx.x < COMPUTE_UNITS * (WPE * 4 / Q::NW))
+        for (uint32_t i = (blockIdx.x * ramp) >> 8; i > 0; --i) __builtin_amdgcn_s_sleep(1);
+}
+
+// Diagnostic: quad_lds_pad() (declared with the parameters, set through sq_debug_select) is that many bytes of unused
+// dynamic LDS added to every launch of the workgroup kernels, so that a compute unit holds fewer workgroups (static +
+// dynamic LDS must stay within 64 KB) -- for measuring how the step time depends on the number of resident workgroups.
 
 template <class T, int NB_, int GH_ = 1>
 struct Quad {

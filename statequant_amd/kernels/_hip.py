@@ -136,7 +136,7 @@ def lib():
             f.restype = C.c_int
             f.argtypes = [C.POINTER(SqGgaSlots), C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
         L.sq_debug_select.restype = None
-        L.sq_debug_select.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+        L.sq_debug_select.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
         L.sq_gga_supported.restype = C.c_int
         L.sq_gga_supported.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         if L.sq_abi_version() != ABI_VERSION:
@@ -212,10 +212,11 @@ def read_state(lay, T, strides, nptr_stride, idx, out, kda):
     check(lib().sq_read(C.byref(a), current_stream(out.device)))
 
 
-def select_instances(no_specialised=False, no_group_kernel=False, max_heads_per_workgroup=0):
+def select_instances(no_specialised=False, no_group_kernel=False, max_heads_per_workgroup=0, lds_pad_bytes=0):
     """``sq_debug_select``: which compiled instance serves a step call when several can (a diagnostic for twin tests
-    and profiles; results do not depend on it).  Call without arguments to restore the default choice."""
-    lib().sq_debug_select(int(no_specialised), int(no_group_kernel), int(max_heads_per_workgroup))
+    and profiles; results do not depend on it).  ``lds_pad_bytes`` adds unused dynamic LDS to the workgroup kernels'
+    launches (fewer resident workgroups).  Call without arguments to restore the default choice."""
+    lib().sq_debug_select(int(no_specialised), int(no_group_kernel), int(max_heads_per_workgroup), int(lds_pad_bytes))
 
 
 def require_gpu(t, what):
