@@ -528,7 +528,7 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
     GdnParams p = p0;
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     const uint32_t grid = uint32_t(p.rows) * uint32_t(p.hv / GH);
-    const uint32_t stag = quad_start_ramp<Quad<T, NB, GH>, WPE>(grid);
+    const uint32_t stag = quad_start_ramp<Quad<T, NB, GH>, WPE>(grid, 32);
 #ifdef SQ_TIMELINE
     const SqTimelineBuf tl = sq_timeline_buffer();
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),

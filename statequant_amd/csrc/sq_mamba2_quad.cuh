@@ -435,7 +435,7 @@ int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     const uint32_t grid = uint32_t(p.rows) * uint32_t(p.hv / GH);
     hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
                        quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
-                       quad_start_ramp<Quad<T, NB, GH>, WPE>(grid), p);
+                       quad_start_ramp<Quad<T, NB, GH>, WPE>(grid, 24), p);
     return int(hipGetLastError());
 }
 

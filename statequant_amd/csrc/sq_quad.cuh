@@ -55,15 +55,15 @@ __device__ __forceinline__ void static_for(F&& f) {
 // their row-block requests back by a ramp of blockIdx x `ramp` / 256 sleeps of 64 clocks, which spreads the first
 // round's requests over about the time memory needs to serve them.  Measured on one machine, int8 rows (four
 // workgroups per compute unit): 32.65 -> 32.08 us per launch with 32 (a stepped ramp of the same slope alike), 24:
-// 32.28, 40 and more: slower than none; the Mamba2 step 31.35 -> 31.15, sequences out of step 35.9 -> 35.5, 512 slots
-// 62.6 -> 61.9, 128 slots 19.1 -> 18.7.  With six smaller workgroups per compute unit (int4) no ramp helped, and a
-// launch of less than two rounds has nothing behind the first to gain from (64 slots: 11.38 -> 11.45), so the
-// launchers pass 0 for those.
+// 32.28, 40 and more: slower than none; the Mamba2 step 31.35 -> 31.15 (30.96 with 24, the slope its launcher
+// passes), sequences out of step 35.9 -> 35.5, 512 slots 62.6 -> 61.9, 128 slots 19.1 -> 18.7.  With six smaller
+// workgroups per compute unit (int4) no ramp helped, and a launch of less than two rounds has nothing behind the
+// first to gain from (64 slots: 11.38 -> 11.45), so those get 0.
 constexpr unsigned COMPUTE_UNITS = 256;                    // MI355X
 template <class Q, int WPE>
-inline uint32_t quad_start_ramp(uint32_t grid) {
+inline uint32_t quad_start_ramp(uint32_t grid, uint32_t slope) {
     constexpr uint32_t per_cu = WPE * 4 / Q::NW;           // resident workgroups per compute unit
-    return (per_cu <= 4 && grid >= 2 * COMPUTE_UNITS * per_cu) ? 32u : 0u;
+    return (per_cu <= 4 && grid >= 2 * COMPUTE_UNITS * per_cu) ? slope : 0u;
 }
 template <class Q, int WPE>
 __device__ __forceinline__ void quad_start_wait(uint32_t ramp) {
