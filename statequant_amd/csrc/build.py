@@ -301,16 +301,75 @@ def _unit_hash(src, seen=None):
     return h.hexdigest()
 
 
+_SREG = re.compile(r'\bs(\d+)\b|\bs\[(\d+):(\d+)\]')
+
+
+def lint_counter_loads(asm_text):
+    """The workgroup kernels fetch a slot's fill counter with a scalar load written in assembly and wait for it in a
+    second assembly statement further down (sq_quad.cuh: quad_dma_counter / quad_dma_counter_wait).  Between the two
+    the destination register holds nothing yet, and the compiler -- which believes the value is there -- must not have
+    read, copied or spilled it.  This walks the device assembly of a unit and returns one message per violation
+    (empty list: fine)."""
+    problems, pending, in_asm, func = [], None, False, '?'
+    for no, line in enumerate(asm_text.split('\n'), 1):
+        t = line.strip()
+        if t.endswith(':') and not t.startswith(('.', ';')):
+            func = t[:-1]
+        if t.startswith(';;#ASMSTART'):
+            in_asm = True
+            continue
+        if t.startswith(';;#ASMEND'):
+            in_asm = False
+            continue
+        if not t or t[0] in '.;' or t.endswith(':'):
+            continue
+        if t.startswith('s_endpgm') and pending is not None:    # a path that leaves before the wait never uses it
+            continue
+        if in_asm:
+            m = re.match(r's_load_dword s(\d+), ', t)
+            if m:
+                if pending is not None:
+                    problems.append(f'{func}: line {no}: a second counter load before the wait for s{pending}')
+                pending = int(m.group(1))
+                continue
+            if pending is not None and t.startswith('s_waitcnt') and 'lgkmcnt(0)' in t:
+                pending = None
+                continue
+        if pending is None:
+            continue
+        code = t.split(';')[0]
+        for m in _SREG.finditer(code):
+            lo, hi = (int(m.group(1)),) * 2 if m.group(1) else (int(m.group(2)), int(m.group(3)))
+            if lo <= pending <= hi:
+                problems.append(f'{func}: line {no}: `{code.strip()}` touches s{pending} before its load is waited for')
+                break
+    if pending is not None:
+        problems.append(f'{func}: counter load into s{pending} is never waited for')
+    return problems
+
+
 def _compile(src, force=False):
-    """Compile one unit unless its object is current (same sources, headers and flags as when it was built)."""
-    obj = os.path.join(OUT, os.path.splitext(os.path.basename(src))[0] + '.o')
+    """Compile one unit unless its object is current (same sources, headers and flags as when it was built).  Units of
+    the workgroup kernels keep their device assembly long enough for lint_counter_loads to read it."""
+    base = os.path.splitext(os.path.basename(src))[0]
+    obj = os.path.join(OUT, base + '.o')
     tag, want = obj + '.hash', _unit_hash(src)
     if not force and os.path.exists(obj) and os.path.exists(tag) and open(tag).read() == want:
         return obj
-    cmd = ['hipcc', *HIPCC_FLAGS, '-c', src, '-o', obj]
+    lint = base.startswith(tuple(f'inst_{fam}q_' for fam in QUAD_FAMILIES))
+    cmd = ['hipcc', *HIPCC_FLAGS, *(['--save-temps=obj'] if lint else []), '-c', src, '-o', obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode:
         raise RuntimeError(f'{" ".join(cmd)}\n{r.stdout}\n{r.stderr}')
+    if lint:
+        temps = [os.path.join(OUT, f) for f in os.listdir(OUT) if f.startswith(base + '-') or f.startswith(base + '.hip-')]
+        asm = [f for f in temps if f.endswith(f'{ARCH}.s')]
+        problems = lint_counter_loads(open(asm[0]).read()) if asm else [f'no device assembly kept for {src}']
+        for f in temps:
+            os.remove(f)
+        if problems:
+            os.remove(obj)
+            raise RuntimeError(f'{src}: hand-placed scalar wait violated\n  ' + '\n  '.join(problems))
     with open(tag, 'w') as f:
         f.write(want)
     return obj

@@ -285,6 +285,9 @@ __device__ __forceinline__ float quad_block_pass(const uint8_t* blk, const v4i (
 // wait for the row blocks requested behind it.  (The scalar cache is invalidated at every kernel start and the counter
 // was written by an earlier launch; within a launch a slot's counter is written by its own workgroup only, at the
 // end.)  The compiler would use a vector load here, because the same address is stored to later in the kernel.
+// Between the load and its wait the compiler believes the register holds the value; build.py reads the device
+// assembly of every unit of these kernels and refuses the build if anything touches that register in between
+// (lint_counter_loads).
 // ---------------------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int quad_dma_counter(const int32_t* p) {
     int v;

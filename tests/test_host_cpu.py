@@ -376,3 +376,23 @@ def test_gga_window_selects_dead_entries_away():
     assert torch.isfinite(left).all() and torch.isfinite(right).all()
     assert torch.equal(left[1, 0], torch.full((HV, D), 0.5)) and torch.equal(left[1, 1], torch.full((HV, D), 2.0))
     assert torch.equal(left[1, 2:], torch.zeros(2, HV, D)) and torch.equal(left[0], torch.zeros(m, HV, D))
+
+
+def test_build_lint_of_the_hand_placed_scalar_wait():
+    """build.py reads the device assembly of every workgroup-kernel unit and refuses a build in which the register of
+    the fill counter's scalar load (requested in one assembly statement, waited for in another) is touched in
+    between: here the checker itself, on assembly with and without such a violation."""
+    from statequant_amd.csrc.build import lint_counter_loads
+    good = '\n'.join(['_Zkernel:', '\ts_mov_b32 s3, 0', '\t;;#ASMSTART', '\ts_load_dword s14, s[8:9], 0x0', '\t;;#ASMEND',
+                      '\tv_mov_b32 v1, s15', '\ts_add_u32 s16, s12, s13', '\t;;#ASMSTART', '\ts_waitcnt lgkmcnt(0)',
+                      '\t;;#ASMEND', '\ts_and_b32 s14, s14, 7', '\ts_endpgm'])
+    assert lint_counter_loads(good) == []
+    copied = good.replace('v_mov_b32 v1, s15', 's_mov_b32 s20, s14')
+    assert len(lint_counter_loads(copied)) == 1 and 's_mov_b32 s20, s14' in lint_counter_loads(copied)[0]
+    in_range = good.replace('s_add_u32 s16, s12, s13', 's_load_dwordx4 s[12:15], s[0:1], 0x0')
+    assert len(lint_counter_loads(in_range)) == 1
+    no_wait = good.replace('\t;;#ASMSTART\n\ts_waitcnt lgkmcnt(0)\n\t;;#ASMEND\n', '')
+    assert any('never waited for' in m for m in lint_counter_loads(no_wait))
+    # a compiler-placed wait does not count: only the assembly statement's own does
+    compiler_wait = good.replace('\t;;#ASMSTART\n\ts_waitcnt lgkmcnt(0)\n\t;;#ASMEND\n', '\ts_waitcnt lgkmcnt(0)\n')
+    assert lint_counter_loads(compiler_wait) != []
