@@ -280,6 +280,18 @@ def test_many_slots_twin_rows_and_subset():
     assert not blob[0].any()
 
 
+def fp8_tie_moves(x):
+    """For vectors x [..., d] about to be FP8-encoded as the oracle does (scale = max |x| / 448): per element, by how
+    much its decoded value moves if the rounding goes the other way -- the FP8 step at that magnitude times the scale
+    -- where the scaled value lies within 2e-4 (fp32 rounding of a few ulp of the largest element) of the midpoint
+    between two FP8 numbers, else 0."""
+    s = (x.abs().amax(-1, keepdim=True) / 448.0).double()
+    v = (x.double() / torch.where(s > 0, s, torch.ones_like(s))).abs()
+    step = 2.0 ** (torch.floor(torch.log2(v.clamp_min(2.0 ** -6))) - 3)
+    near = ((v / step) % 1.0 - 0.5).abs() * step < 2e-4
+    return torch.where(near, step * s, torch.zeros_like(v)).float()
+
+
 def _random_gga_configs(n, seed=77):
     import random
     rng = random.Random(seed)
@@ -309,7 +321,13 @@ def test_random_configurations(cfg):
     live, li = idx[ok].to(DEV), idx[ok].long()
     pk.write(Vp, live, (torch.randn(B, HV, D, D, generator=g) * 0.3).transpose(-1, -2).to(DEV), layer=3)
     A_log, dtb = torch.randn(HV, generator=g) * 0.3, torch.randn(HV, generator=g) * 0.3
-    ora = G.GGAState(bits, w, B + 2, HV, HK, D, D, pw=pw, m=m)
+    tie_moves = []
+
+    def enc(x):
+        tie_moves.append(fp8_tie_moves(x))
+        return G.fp8_vec(x)
+
+    ora = G.GGAState(bits, w, B + 2, HV, HK, D, D, pw=pw, m=m, enc=enc)
     nonp = (bits != 16)[None, None, :, None]
     dt = torch.bfloat16 if cfg['bf16'] else torch.float32
     for t, (qq, kk, vv, a, b) in enumerate(tokens(cfg['steps'], B + 1, HV, HK, D, seed=cfg['seed'] + 1, dtype=dt)):
@@ -317,15 +335,28 @@ def test_random_configurations(cfg):
         if pw:
             P, V, n = pk.window(Vp, live)
             ora.P[li], ora.V[li], ora.n[li] = P.cpu(), V.cpu(), n.cpu().long()
+        V_before = ora.V[idx.long()].clone()                                      # [rows, m, HV, d_v]
+        tie_moves.clear()                                                         # the step's first encode: the queue
         op = torch.full((B + 1, HV, D), 7.0, device=DEV)
         pk.step(Vp, idx.to(DEV), *dev(qq, kk, vv), op, D ** -0.5, gate=tuple(dev(a, b, A_log, dtb)), layer=3)
         gl, beta = ora.gate(a, b, A_log, dtb)
         oe = ora.step(idx, qq, kk, vv, D ** -0.5, gl, beta)
         op = op.cpu()
         assert float(op[1].abs().max()) == 0.
-        assert ((op - oe).norm() / oe.norm()).item() < 1e-5, t
         Sp, Se = pk.stored(Vp, live, 3).cpu(), ora.O[li]
         assert ((Sp - Se).abs() > 1e-3 * Se.abs().amax()).float().mean().item() < 3e-3, t
+        # outputs: 1e-5 per (row, head), plus what an FP8 rounding tie can move: the read-out takes the queued left
+        # factors as the step re-encodes them, and where the value to encode lies within fp32 rounding of the midpoint
+        # between two FP8 numbers the kernel and the oracle may land on different sides (seen once in 2 000 steps of
+        # such configurations: a scaled value of 272.00004 between 256 and 288, the output of that head 1.6e-3 off)
+        err = (op - oe).norm(dim=-1) / oe.norm(dim=-1).clamp_min(1e-30)
+        slack = torch.zeros(B + 1, HV)
+        if pw:
+            qn = qq.float() * torch.rsqrt((qq.float() ** 2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+            qn = qn.repeat_interleave(HV // HK, 1)                                # [rows, HV, d_k]
+            move = tie_moves[0] * qn[:, None].abs()                               # [rows, m, HV, d_k]
+            slack = (move.sum(-1) * V_before.norm(dim=-1)).sum(1) / oe.norm(dim=-1).clamp_min(1e-30)
+        assert (err <= 1e-5 + 1.01 * slack).all(), (t, err, slack)
         if pw:
             P, V, n = pk.window(Vp, live)
             assert torch.equal(n.cpu().long(), ora.n[li]), t

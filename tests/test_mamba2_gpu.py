@@ -316,8 +316,8 @@ def _random_configs(n, seed=31, shapes=((128, 64), (128, 128), (64, 64))):
     while len(out) < n:
         fmt = rng.choice(fmts)
         DK, DV = rng.choice(list(shapes))
-        if fmt != 'bf16' and ((fmt[1] == 'k' and fmt[2] > DK) or (fmt[1] == 'v' and DV % fmt[2])):
-            continue
+        if fmt != 'bf16' and ((fmt[1] == 'k' and DK % fmt[2]) or (fmt[1] == 'v' and DV % fmt[2])):
+            continue                                         # Mamba2 groups must divide their axis (mamba2.py:73-78)
         G = rng.choice([1, 2, 3])
         out.append(dict(fmt=fmt, DK=DK, DV=DV, m=rng.choice([1, 2, 4, 8, 16]), bb=rng.choice([8, 16]), G=G,
                         H=G * rng.choice([1, 2, 7]), B=rng.choice([1, 3]), seed=rng.randrange(1000),
