@@ -115,6 +115,10 @@ __device__ __forceinline__ Divisor scale_divisor(float scale) {
     return v;
 }
 __device__ __forceinline__ float div_by(float x, const Divisor& v) { return div_rc(x, v.d, v.rc); }
+// The fp16-valued divisor back from its correctly rounded reciprocal: 1 / rc is within 2^-22 of it, and rounding to
+// fp16's grid (11 bits, subnormals included) removes that.  For paths that are rarely taken and would otherwise keep
+// the divisor in a register beside its reciprocal.
+__device__ __forceinline__ float divisor_of(float rc) { return float(_Float16(__builtin_amdgcn_rcpf(rc))); }
 
 // Quantizer scale: max(amax, 1e-8) / qmax -> fp16 (nearest even, subnormals kept) -> fp32, floored at 2^-24.  qmax is
 // 7 or 127 at every call (a constant there, so 1 / qmax is folded).
@@ -299,10 +303,38 @@ __device__ __forceinline__ RawRow<BITS> encode_row(const float (&c)[CPL]) {
 // the biased float, the bytes / nibbles are gathered with byte permutes.
 // CLAMP = false leaves the clamp out: for callers that know |a r| < qmax + 1/2 (a scale that is a NORMAL fp16
 // number lies within 2^-11 of absmax / qmax, so the largest quotient is qmax (1 + 2^-11) at most).
-template <int BITS, bool CLAMP = true>
-__device__ __forceinline__ RawRow<BITS> quantize_row(const float (&a)[CPL], float r) {
+// a r differs from the quotient a / d by the reciprocal's rounding, 2^-24 of it: where the quotient is within that
+// of a half-integer the code can come out one step from rint(a / d).  For values in general position that is one
+// code in 10^5; but a state that is a sum of a few products of low-precision numbers (the first fold after an empty
+// state: buffered vectors are bf16 or int8 x fp16) has quotients that are EXACTLY half-integers, thousands of them,
+// and those would go by the sign of the reciprocal's error instead of to even.  EXACT = true takes the IEEE quotient
+// first (div_rc with the divisor d: two more fmas and an addition per value), bit for bit the reference's
+// rint(div_rn(a, d)) (_fused_triton.py:472-486 there); the folds use it where the old state contributes nothing.
+template <int BITS, bool CLAMP = true, bool EXACT = false>
+__device__ __forceinline__ RawRow<BITS> quantize_row(const float (&a)[CPL], float r, float d = 0.0f) {
     constexpr float QMAX = float((1 << (BITS - 1)) - 1);
     constexpr float MAGIC = 12582912.0f + (BITS == 4 ? 8.0f : 0.0f);
+    if constexpr (EXACT) {
+        // the rarely taken exact path packs word by word, so that it needs fewer registers than the other one (it
+        // must not raise the allocation of kernels that run at their limit)
+        constexpr int PER = 32 / BITS;                       // codes per 32-bit word
+        uint32_t w[CPL / PER];
+#pragma unroll
+        for (int i = 0; i < CPL / PER; ++i) {
+            uint32_t acc = 0;
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                const float f = __builtin_amdgcn_fmed3f(div_rc(a[PER * i + e], d, r) + MAGIC, MAGIC - QMAX, MAGIC + QMAX);
+                acc |= (as_u32(f) & (BITS == 8 ? 0xFFu : 0xFu)) << (BITS * e);
+            }
+            w[i] = acc;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        RawRow<BITS> o;
+        if constexpr (BITS == 8) o.v = make_uint4(w[0], w[1], w[2], w[3]);
+        else o.v = make_uint2(w[0], w[1]);
+        return o;
+    }
     uint32_t u[CPL];
 #pragma unroll
     for (int t = 0; t < CPL; ++t) {

@@ -277,6 +277,12 @@ void gdn_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
     append_key<T>(kxe, ks, A.buf, n, int(h) == A.hk * gqa, l, kr);
     if (l.lane == 0) A.GBh[n] = gnew;
 
+    // ---- advance: here unless the buffer is full (then behind the fold, to zero), so that the running decay and
+    //      the count do not stay in registers across the fold ----
+    if (!full && l.lane == 0) {
+        *A.gcp = gnew;
+        *A.np = n + 1;
+    }
     // ---- fold ----
     if (full) {
         float uo[T::NOWN][T::MMAX];
@@ -298,12 +304,10 @@ void gdn_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
         wave_sync();
         if constexpr (T::AXV) fold_tile_v<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
         else fold_tile<T, false>(lds_k, lds_u, nullptr, expf(gnew), m, A.Sh, A.SCh, l);
-    }
-
-    // ---- advance ----
-    if (l.lane == 0) {
-        *A.gcp = full ? 0.0f : gnew;
-        *A.np = full ? 0 : n + 1;
+        if (l.lane == 0) {
+            *A.gcp = 0.0f;
+            *A.np = 0;
+        }
     }
 }
 

@@ -253,6 +253,15 @@ void kda_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
     }
 
     SQ_MARK(7);                                                   // appended
+    // the running decay: stored here unless the buffer is full (then it restarts at zero, stored behind the fold), so
+    // that it does not have to stay in registers across the fold
+    if (!full) {
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) {
+            const int e = l.lane + WAVE * t;
+            if (e < DK) gch[e] = gn[t];
+        }
+    }
     // ---- fold ----
     if (full) {
         float uo[T::NOWN][T::MMAX];
@@ -288,14 +297,14 @@ void kda_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
         wave_sync();
         if constexpr (T::AXV) fold_tile_v<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
         else fold_tile<T, true>(lds_k, lds_u, lds_c, 1.0f, m, Sh, SCh, l);
+#pragma unroll
+        for (int t = 0; t < T::NE; ++t) {
+            const int e = l.lane + WAVE * t;
+            if (e < DK) gch[e] = 0.0f;
+        }
     }
 
-    // ---- advance ----
-#pragma unroll
-    for (int t = 0; t < T::NE; ++t) {
-        const int e = l.lane + WAVE * t;
-        if (e < DK) gch[e] = full ? 0.0f : gn[t];
-    }
+    // ---- advance (the running decay of a full buffer is stored at the end of the fold) ----
     if (l.lane == 0) *np = full ? 0 : n + 1;
     SQ_MARK(8);                                                   // folded (a full buffer), counters advanced
 }

@@ -478,10 +478,19 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
     // number 1024 + byte by a byte permute (exponent byte 0x64 on top), and one v_mfma_f32_16x16x16_f16 against the
     // 16 x 16 identity hands every lane its own four numbers back as fp32 on top of the constant -1152 (exact).
     constexpr bool UNITS = T::BITS == 8 && T::NG == 1;
+    // An old scale at its floor is an empty group (or one too small to matter), and a decay of exactly 1 leaves the
+    // stored codes times their scale as they are: what is quantized then is a sum of a few products of low-precision
+    // numbers, whose quotients by the new scale are exact half-integers by the thousand -- the codes are taken as
+    // rint of the IEEE quotient there (quantize_row<.., EXACT>), which sends them to even as the reference's do.
+    const bool exact = __builtin_amdgcn_ballot_w64(s_old <= FP16_TINY || cmul == 1.0f) != 0;
     float unit = 1.0f;                                       // what one accumulator unit is worth
     if constexpr (UNITS) {
         typedef _Float16 v4h __attribute__((ext_vector_type(4)));
         unit = fmaxf(sm, 1e-30f);                            // a vanished old state: its term is below any scale
+        // exact mode: a power of two as the unit, so that scaling by it rounds nothing (the codes then count ratio
+        // = sm / unit each instead of 1)
+        const float ratio = exact ? sm / as_f32(as_u32(unit) & 0x7F800000u) : 1.0f;
+        if (exact) unit = as_f32(as_u32(unit) & 0x7F800000u);
         v4h ident;
 #pragma unroll
         for (int j = 0; j < 4; ++j) ident[j] = (n == 4 * q + j) ? _Float16(1.0f) : _Float16(0.0f);
@@ -493,6 +502,10 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
             h2.x = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);      // halves 1024 + byte 0, 1024 + byte 1
             h2.y = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);      // bytes 2, 3
             acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(ident, __builtin_bit_cast(v4h, h2), bias, 0, 0, 0);
+        }
+        if (exact) {
+#pragma unroll
+            for (int d = 0; d < NW32; ++d) acc[d] = acc[d] * ratio;
         }
     } else if constexpr (T::BITS == 8) {
 #pragma unroll
@@ -536,19 +549,21 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
     if constexpr (LPG >= 2) { const Pair pm = pair16(mx); mx = fmaxf(pm.lo, pm.hi); }
     if constexpr (LPG >= 4) { const Pair pm = pair32(mx); mx = fmaxf(pm.lo, pm.hi); }
     const float sc = fp16_scale(UNITS ? mx * unit : mx, T::QMAX);
-    const float rs = UNITS ? unit * scale_divisor(sc).rc : scale_divisor(sc).rc;        // sc is an fp16 value: the exact reciprocal
+    const Divisor dsc = scale_divisor(sc);                   // sc is an fp16 value: the correctly rounded reciprocal
+    const float rs = UNITS ? unit * dsc.rc : dsc.rc;         // (exact mode: unit is a power of two, both stay exact)
+    const float ds = UNITS ? dsc.d * __builtin_amdgcn_rcpf(unit) : dsc.d;
     if (q % LPG == 0) *sc_out = f32_to_f16(sc);
     // new codes, back into the LDS image.  A scale in fp16's normal range cannot push a quotient past qmax + 1/2, so
     // the clamp is only compiled into the path taken when some lane's scale is subnormal (or at its floor).
-    auto requantize = [&](auto clamp) {
-        constexpr bool CLAMP = decltype(clamp)::value;
+    auto requantize = [&](auto clamp, auto exactly) {
+        constexpr bool CLAMP = decltype(clamp)::value, EXACT = decltype(exactly)::value;
         if constexpr (NBY >= 16) {
 #pragma unroll
             for (int c = 0; c < CL / 16; ++c) {              // 16 columns per call
                 float a16[CPL];
 #pragma unroll
                 for (int e = 0; e < CPL; ++e) a16[e] = acc[4 * c + e / 4][e % 4];
-                const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP>(a16, rs);
+                const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP, EXACT>(a16, rs, ds);
                 if constexpr (T::BITS == 8) *reinterpret_cast<uint4*>(blk + (c == 0 ? at : at1)) = r.v;
                 else *reinterpret_cast<uint2*>(blk + at + 8 * c) = r.v;      // 16 columns = half a chunk
             }
@@ -556,12 +571,13 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
             float a16[CPL];
 #pragma unroll
             for (int e = 0; e < CPL; ++e) a16[e] = acc[e / 4][e % 4];
-            const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP>(a16, rs);
+            const RawRow<T::BITS> r = quantize_row<T::BITS, CLAMP, EXACT>(a16, rs, ds);
             *reinterpret_cast<uint2*>(blk + at) = r.v;
         }
     };
-    if (__builtin_amdgcn_ballot_w64(sc < 6.103515625e-05f) != 0) requantize(std::true_type{});
-    else requantize(std::false_type{});
+    if (exact) requantize(std::true_type{}, std::true_type{});
+    else if (__builtin_amdgcn_ballot_w64(sc < 6.103515625e-05f) != 0) requantize(std::true_type{}, std::false_type{});
+    else requantize(std::false_type{}, std::false_type{});
 }
 
 }  // namespace sq

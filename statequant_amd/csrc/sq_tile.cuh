@@ -891,6 +891,14 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
         uint16_t scr[T::NG];
 #pragma unroll
         for (int g = 0; g < T::NG; ++g) scr[g] = scn[g];
+        // an old scale at its floor (stored fp16 bits 0 or 1: an empty group) or a decay of exactly 1: what is
+        // quantized is a sum of a few low-precision products with exact half-integer quotients by the thousand --
+        // there the codes are rint of the IEEE quotient (quantize_row<.., EXACT>).  Decided here, while the old
+        // scales are in registers anyway.
+        bool cold = !COLVEC && cmul == 1.0f;
+#pragma unroll
+        for (int g = 0; g < T::NG; ++g) cold = cold || scr[g] <= 1;
+        const bool exact = __builtin_amdgcn_ballot_w64(cold) != 0;
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
@@ -955,14 +963,20 @@ __device__ __forceinline__ void fold_tile(float* lds_k, const float* lds_u, cons
             rs[g] = scale_divisor(sc).rc;
             if (kb == 0 && (!T::RAGV || row < T::DV)) sc_head[row * T::NG + g] = f32_to_f16(sc);
         }
+        auto requantize = [&](auto exactly) {                // two code paths, not a select between two results
 #pragma unroll
-        for (int cs = 0; cs < NCS; ++cs) {
-            float a16[CPL];
+            for (int cs = 0; cs < NCS; ++cs) {
+                float a16[CPL];
 #pragma unroll
-            for (int e = 0; e < CPL; ++e) a16[e] = acc[cs][e];
-            store_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES,
-                               quantize_row<T::BITS>(a16, rs[(cs * T::MK) / T::GROUP]));
-        }
+                for (int e = 0; e < CPL; ++e) a16[e] = acc[cs][e];
+                const int g = (cs * T::MK) / T::GROUP;
+                const float d = decltype(exactly)::value ? divisor_of(rs[g]) : 0.0f;
+                store_row<T::BITS>(blk + j * T::A_PITCH + (2 * cs + kb) * T::LANE_BYTES,
+                                   quantize_row<T::BITS, true, decltype(exactly)::value>(a16, rs[g], d));
+            }
+        };
+        if (exact) requantize(std::true_type{});
+        else requantize(std::false_type{});
         wave_sync();
         if (live) {
 #pragma unroll
@@ -1045,6 +1059,12 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         for (int cs = 0; cs < NCS; ++cs)
 #pragma unroll
             for (int hf = 0; hf < VH; ++hf) scr[cs][hf] = scn[cs][hf];
+        bool cold = !COLVEC && cmul == 1.0f;     // as in the key-axis fold: exact quotients where the old state is empty
+#pragma unroll
+        for (int cs = 0; cs < NCS; ++cs)
+#pragma unroll
+            for (int hf = 0; hf < VH; ++hf) cold = cold || scr[cs][hf] <= 1;
+        const bool exact = __builtin_amdgcn_ballot_w64(cold) != 0;
         if (live) {
 #pragma unroll
             for (int t = 0; t < NL; ++t)
@@ -1111,11 +1131,20 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
         }
         wave_sync();                                     // every lane has its codes: the block takes the new ones
         if (!last_phase) continue;
+        auto requantize = [&](auto exactly) {                // two code paths, not a select between two results
 #pragma unroll
         for (int cs = 0; cs < NCS; ++cs) {
 #pragma unroll
             for (int e = 0; e < CPL; ++e) {
-                const float f = __builtin_fmaf(acc[cs][e], rs[cs][VH > 1 ? e / 8 : 0], MAGIC);
+                const int hs = VH > 1 ? e / 8 : 0;
+                float f;
+                if constexpr (decltype(exactly)::value) {
+                    float d = divisor_of(rs[cs][hs]);        // anew for every element: the rare path must not hold
+                    asm volatile("" : "+v"(d));              // a second table of divisors in registers
+                    f = div_rc(acc[cs][e], d, rs[cs][hs]) + MAGIC;
+                } else {
+                    f = __builtin_fmaf(acc[cs][e], rs[cs][hs], MAGIC);
+                }
                 const uint32_t u = as_u32(__builtin_amdgcn_fmed3f(f, MAGIC - T::QMAX, MAGIC + T::QMAX));
                 const int row = 8 * (e / 4) + 4 * kb + (e % 4);
                 if constexpr (T::BITS == 8) {
@@ -1127,6 +1156,9 @@ __device__ __forceinline__ void fold_tile_v(float* lds_k, const float* lds_u, co
                 }
             }
         }
+        };
+        if (exact) requantize(std::true_type{});
+        else requantize(std::false_type{});
         wave_sync();
         if (live) {
 #pragma unroll

@@ -537,3 +537,29 @@ def test_random_configurations(cfg):
     assert tal.worst_o < 1e-4, tal.worst_o
     assert tal.buf_flips <= max(1, 1e-3 * tal.buf_entries), (tal.buf_flips, tal.buf_entries)
     assert tal.code_mism <= max(1, 1e-3 * tal.code_n) and tal.code_far == 0, (tal.code_mism, tal.code_far)
+
+
+@pytest.mark.parametrize('kernel', ['group', 'one-wavefront'])
+@pytest.mark.parametrize('fmt', [(8, 'k', 64), (8, 'k', 128), (4, 'k', 64), (4, 'k', 32), (8, 'v', 32), (4, 'v', 32)])
+@pytest.mark.parametrize('m', [1, 2])
+def test_first_fold_from_an_empty_state(fmt, m, kernel):
+    """The first fold after an empty state quantizes a sum of m products of low-precision numbers (bf16 buffer
+    entries): its quotients by the new scale are exact half-integers by the thousand (with m = 1, wherever the key's
+    largest entry has the significand 127/128), which rint(div_rn(.)) -- the reference's _rint_quot,
+    _fused_triton.py:472-486 there -- sends to even.  The kernels take the IEEE quotient where the old state
+    contributes nothing (an old scale at its floor); with the reciprocal shortcut of the other folds a third of a
+    percent of such a fold's codes would be one step off.  One fold: no code may differ (two for the sums' order)."""
+    from statequant_amd.kernels import _hip
+    if kernel == 'one-wavefront' and fmt[1] == 'v':
+        pytest.skip('value-axis groups run on the one-wavefront kernel either way')
+    _hip.select_instances(no_group_kernel=kernel == 'one-wavefront')
+    try:
+        worst = 0
+        for seed in range(6):
+            tal = run_decode(fmt, m, 16, B=2, HV=8, HK=2, D=128, T=m, seed=seed, S0_scale=0.0)
+            assert tal.folds == 1 and tal.code_far == 0 and tal.scale_mism == 0
+            worst = max(worst, tal.code_mism)
+        print(f'\n{fmt} m={m} {kernel}: at most {worst} of {tal.code_n} codes differ after the first fold (6 seeds)')
+        assert worst <= 2, worst
+    finally:
+        _hip.select_instances()
