@@ -47,8 +47,12 @@ class Tally:
         self.worst_deq = 0.0
         self.folds = 0
 
-    def out(self, o, ref):
-        self.worst_o = max(self.worst_o, ((o - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item())
+    def out(self, o, ref, floor=1e-30):
+        """Largest |o - ref| of the step relative to the largest |ref| -- or to ``floor``, the size the outputs
+        have by construction, where a step's outputs happen to be much smaller than that (an empty state and a k
+        nearly orthogonal to q leave o = (k.q) u with k.q the cancelled sum of d_k products: an absolute error of
+        1e-9 is then 1e-4 of an output of 1e-5)."""
+        self.worst_o = max(self.worst_o, ((o - ref).abs().max() / ref.abs().max().clamp_min(floor)).item())
 
     def entries(self, got, want):
         """Buffered vectors [..., d] as stored (dequantized).  A vector whose fp16 scale landed on the other side of a

