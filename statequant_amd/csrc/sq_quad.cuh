@@ -504,6 +504,7 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
             acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(ident, __builtin_bit_cast(v4h, h2), bias, 0, 0, 0);
         }
         if (exact) {
+            asm volatile("" ::: "memory");                   // a real branch: not 32 multiplications by 1 otherwise
 #pragma unroll
             for (int d = 0; d < NW32; ++d) acc[d] = acc[d] * ratio;
         }
