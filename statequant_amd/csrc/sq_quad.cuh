@@ -489,8 +489,9 @@ __device__ __forceinline__ void quad_fold_half(uint8_t* blk, int hf, const FoldK
         unit = fmaxf(sm, 1e-30f);                            // a vanished old state: its term is below any scale
         // exact mode: a power of two as the unit, so that scaling by it rounds nothing (the codes then count ratio
         // = sm / unit each instead of 1)
-        const float ratio = exact ? sm / as_f32(as_u32(unit) & 0x7F800000u) : 1.0f;
-        if (exact) unit = as_f32(as_u32(unit) & 0x7F800000u);
+        const float p2 = as_f32(as_u32(unit) & 0x7F800000u);
+        const float ratio = exact ? sm * __builtin_amdgcn_rcpf(p2) : 1.0f;     // the reciprocal of a power of two: exact
+        if (exact) unit = p2;
         v4h ident;
 #pragma unroll
         for (int j = 0; j < 4; ++j) ident[j] = (n == 4 * q + j) ? _Float16(1.0f) : _Float16(0.0f);
