@@ -564,3 +564,53 @@ def test_first_fold_from_an_empty_state(fmt, m, kernel):
         assert worst <= 2, worst
     finally:
         _hip.select_instances()
+
+
+@pytest.mark.parametrize('name', ['int4-k-g64', 'int8-k-g128', 'int8-v-g32', 'bf16'])
+@pytest.mark.parametrize('m,bb', [(8, 8), (2, 16), (1, 16)])
+def test_decode_in_a_freshly_allocated_slot(name, m, bb):
+    """A slot as `alloc` hands it out (slots.py:119-121 there: all bytes zero -- codes 0, scales 0, counters 0, which
+    is an empty state, though not the bytes `write` of a zero state leaves: those carry the scale floor 2^-24) decoded
+    from its first token, as a serving engine does with a sequence that starts in decode: outputs and, after every
+    fold, codes and scales against the oracle started from the zero state."""
+    fmt = {**FORMATS, **VALUE_AXIS, 'bf16': 'bf16'}[name]
+    lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=bb)
+    views = lay.views(lay.alloc(4, DEV))
+    slots = torch.tensor([2, 3])
+    idx = slots.to(torch.int32).to(DEV)
+    ref = ST.GDNOracle(torch.zeros(2 * HV, D, D), fmt, m=m, hv=HV, hk=HK, buffer_bits=bb, auto_fold=False)
+    gen = torch.Generator().manual_seed(4)
+    tal = Tally()
+    for t in range(2 * m + 1):
+        q, k, v, g, beta = gdn_token(gen, 2, HV, HK, D, D)
+        out = torch.empty(2, HV, D, device=DEV)
+        i = ref.n
+        lay.step(views, idx, q.to(DEV), k.to(DEV), v.to(DEV), out, D ** -0.5, g=g.to(DEV), beta=beta.to(DEV))
+        want = ref.step(q.reshape(-1, D), k.reshape(-1, D), v.reshape(-1, D), g.reshape(-1), beta.reshape(-1), D ** -0.5)
+        tal.out(out.cpu().reshape(-1, D), want, floor=1e-2 * D ** -0.5 * v.abs().max().item())
+        T = {f: views[f][slots.to(DEV)].flatten(0, 1) for f in ('KB', 'UB', 'KBS', 'UBS') if f in views}
+        kb = T['KB'].view(2 * HK, m, D)[:, i].float().cpu()                       # the oracle's: per key head
+        ub = T['UB'].view(2 * HV, m, D)[:, i].float().cpu()
+        if bb == 8:
+            kb = kb * T['KBS'].view(2 * HK, m)[:, i].float().cpu()[:, None]
+            ub = ub * T['UBS'].view(2 * HV, m)[:, i].float().cpu()[:, None]
+        tal.entries(kb, ref.K[:, i])
+        tal.entries(ub, ref.U[:, i])
+        ref.K[:, i], ref.U[:, i] = kb, ub
+        if ref.n == m:
+            ref.fold()
+            codes = views['S'][slots.to(DEV)].flatten(0, 1).cpu()
+            if fmt == 'bf16':
+                scales = ref.scales
+                tal.fold(codes, scales, ref, 16)
+            else:
+                scales = views['SC'][slots.to(DEV)].flatten(0, 1).cpu()
+                tal.fold(codes, scales, ref, fmt[0])
+            ref.adopt(codes, scales)
+    print('\n' + tal.report(f'fresh slot {name} m={m} buf{bb}'))
+    # (a group whose largest value differs in its last bit may get the neighbouring fp16 scale, and then other codes)
+    assert tal.folds == (2 * m + 1) // m and tal.worst_o < 2e-5 and tal.code_far == 0 and tal.scale_mism <= 2
+    assert tal.code_mism <= max(2, 1e-4 * tal.code_n) + tal.scale_mism * D
+    assert tal.buf_flips <= max(1, 1e-4 * tal.buf_entries)
+    assert views['NPTR'][slots.to(DEV), :HV].cpu().tolist() == [[(2 * m + 1) % m] * HV] * 2
+    assert not views['S'][0].any() and not views['S'][1].any()                   # the other slots: untouched
