@@ -614,3 +614,24 @@ def test_decode_in_a_freshly_allocated_slot(name, m, bb):
     assert tal.buf_flips <= max(1, 1e-4 * tal.buf_entries)
     assert views['NPTR'][slots.to(DEV), :HV].cpu().tolist() == [[(2 * m + 1) % m] * HV] * 2
     assert not views['S'][0].any() and not views['S'][1].any()                   # the other slots: untouched
+
+
+@pytest.mark.parametrize('fmt,m,bb', [((8, 'k', 128), 8, 8), ((4, 'v', 32), 4, 16)])
+def test_fp16_tokens_and_outputs(fmt, m, bb):
+    """fp16 q / k / v (dtype 2 of the C ABI; the reference upcasts any float dtype in the kernel,
+    _fused_triton.py:79-80) through both kernel kinds, and fp16 outputs of the slot op: the oracle's output rounded to
+    fp16, or its fp16 neighbour where the fp32 values differ in their last bits."""
+    check(run_decode(fmt, m, bb, dtype=torch.float16, T=2 * m + 1), f'gdn {fmt} fp16 tokens', 2 * m + 1, m)
+    lay = SlotLayout(quantizer(fmt), HV, HK, D, D, m=m, buffer_bits=bb)
+    views = lay.views(lay.alloc(4, DEV))
+    idx = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    ref = ST.GDNOracle(torch.zeros(2 * HV, D, D), fmt, m=m, hv=HV, hk=HK, buffer_bits=bb)
+    gen = torch.Generator().manual_seed(0)
+    for t in range(m + 2):
+        q, k, v, g, beta = gdn_token(gen, 2, HV, HK, D, D, torch.float16)
+        out = torch.empty(2, HV, D, device=DEV, dtype=torch.float16)
+        lay.step(views, idx, q.to(DEV), k.to(DEV), v.to(DEV), out, D ** -0.5, g=g.to(DEV), beta=beta.to(DEV))
+        want = ref.step(q.reshape(-1, D), k.reshape(-1, D), v.reshape(-1, D), g.reshape(-1), beta.reshape(-1), D ** -0.5)
+        got = out.float().cpu().reshape(-1, D)
+        assert ((got - want).abs() <= want.abs() * 2.0 ** -10 + 1e-7).all(), t      # within one fp16 step of the oracle
+        assert (got != want.half().float()).float().mean().item() < 1e-2, t       # and almost always its rounding

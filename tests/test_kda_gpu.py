@@ -342,3 +342,8 @@ def test_first_fold_from_an_empty_state(fmt, m):
         worst = max(worst, tal.code_mism)
     print(f'\nkda {fmt} m={m}: at most {worst} of {tal.code_n} codes differ after the first fold (6 seeds)')
     assert worst <= 2, worst
+
+
+def test_fp16_tokens():
+    """fp16 q / k / v (dtype 2 of the C ABI) through the KDA step."""
+    check(run_decode((4, 'k', 32), 8, 8, dtype=torch.float16, T=17), 'kda fp16 tokens', 17, 8)

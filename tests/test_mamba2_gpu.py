@@ -356,3 +356,9 @@ def test_first_fold_from_an_empty_state(fmt, m):
         worst = max(worst, tal.code_mism)
     print(f'\nmamba2 {fmt} m={m}: at most {worst} of {tal.code_n} codes differ after the first fold (6 seeds)')
     assert worst <= 2, worst
+
+
+def test_fp16_tokens():
+    """fp16 x / B / C (dtype 2 of the C ABI) through both Mamba2 kernel kinds."""
+    check(run_decode((8, 'k', 128), 8, 8, dtype=torch.float16, T=17), 'mamba2 fp16 tokens', 17, 8)
+    check(run_decode((8, 'v', 32), 4, 16, dtype=torch.float16, T=9), 'mamba2 value-axis fp16 tokens', 9, 4)
