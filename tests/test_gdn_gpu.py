@@ -635,3 +635,54 @@ def test_fp16_tokens_and_outputs(fmt, m, bb):
         got = out.float().cpu().reshape(-1, D)
         assert ((got - want).abs() <= want.abs() * 2.0 ** -10 + 1e-7).all(), t      # within one fp16 step of the oracle
         assert (got != want.half().float()).float().mean().item() < 1e-2, t       # and almost always its rounding
+
+
+@pytest.mark.parametrize('gd', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('bd', [torch.float32, torch.bfloat16, torch.float16])
+def test_gate_operand_dtypes(gd, bd):
+    """g and beta -- or the in-kernel gate's a, b, A_log, dt_bias -- in any of the three float dtypes, each with its
+    own dtype code in the C ABI (the reference's kernels upcast whatever they are given): the oracle on the same
+    rounded values, up to the first fold (later steps would need the re-sync of the other tests)."""
+    m = 4
+    lay = SlotLayout(quantizer((8, 'k', 128)), HV, HK, D, D, m=m, buffer_bits=8)
+    blob = lay.alloc(4, DEV)
+    views = lay.views(blob)
+    idx = torch.tensor([1, 0, 2], dtype=torch.int32, device=DEV)                  # row 1 is padding
+    live = [0, 2]
+    for gated in (False, True):
+        blob.zero_()
+        ref = ST.GDNOracle(torch.zeros(2 * HV, D, D), (8, 'k', 128), m=m, hv=HV, hk=HK, buffer_bits=8)
+        gen = torch.Generator().manual_seed(7)
+        A_log, dtb = (torch.randn(HV, generator=gen) * 0.3).to(gd), (torch.randn(HV, generator=gen) * 0.3).to(bd)
+        for t in range(m):
+            q, k, v, g, beta = gdn_token(gen, 3, HV, HK, D, D)
+            out = torch.full((3, HV, D), 7.0, device=DEV)
+            if gated:
+                a, b = (torch.randn(3, HV, generator=gen) * 0.5 - 2).to(gd), torch.randn(3, HV, generator=gen).to(bd)
+                lay.step(views, idx, q.to(DEV), k.to(DEV), v.to(DEV), out, D ** -0.5,
+                         gate=(a.to(DEV), b.to(DEV), A_log.to(DEV), dtb.to(DEV)))
+                g, beta = ST.gdn_gate(a.float(), b.float(), A_log.float(), dtb.float())
+            else:
+                g, beta = g.to(gd), beta.to(bd)
+                lay.step(views, idx, q.to(DEV), k.to(DEV), v.to(DEV), out, D ** -0.5, g=g.to(DEV), beta=beta.to(DEV))
+            want = ref.step(q[live].reshape(-1, D), k[live].reshape(-1, D), v[live].reshape(-1, D),
+                            g[live].float().reshape(-1), beta[live].float().reshape(-1), D ** -0.5)
+            assert float(out[1].abs().max()) == 0.
+            got = out[live].cpu().reshape(-1, D)
+            assert ((got - want).abs().max() / want.abs().max().clamp_min(1e-3)).item() < 2e-5, (gated, t)
+
+
+def test_empty_and_all_padding_batches():
+    """No rows at all (slots.py:140-141 there: returns `out`), and rows that are all padding: zero outputs, not a
+    byte of any slot touched."""
+    lay = SlotLayout(quantizer((8, 'k', 128)), HV, HK, D, D, m=4, buffer_bits=8)
+    blob = lay.alloc(4, DEV)
+    views = lay.views(blob)
+    e = lambda *s: torch.empty(*s, device=DEV)                  # noqa: E731
+    out = lay.step(views, torch.empty(0, dtype=torch.int32, device=DEV), e(0, HK, D), e(0, HK, D), e(0, HV, D), e(0, HV, D),
+                   D ** -0.5, g=e(0, HV), beta=e(0, HV))
+    assert out.shape[0] == 0
+    q, k, v, g, beta = (x.to(DEV) for x in gdn_token(torch.Generator().manual_seed(2), 3, HV, HK, D, D))
+    out = torch.full((3, HV, D), 7.0, device=DEV)
+    lay.step(views, torch.tensor([0, -1, 0], dtype=torch.int32, device=DEV), q, k, v, out, D ** -0.5, g=g, beta=beta)
+    assert float(out.abs().max()) == 0. and not blob.any()
