@@ -347,3 +347,22 @@ def test_first_fold_from_an_empty_state(fmt, m):
 def test_fp16_tokens():
     """fp16 q / k / v (dtype 2 of the C ABI) through the KDA step."""
     check(run_decode((4, 'k', 32), 8, 8, dtype=torch.float16, T=17), 'kda fp16 tokens', 17, 8)
+
+
+@pytest.mark.parametrize('gd,bd,od', [(torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.float16, torch.float16),
+                                      (torch.float16, torch.bfloat16, torch.bfloat16), (torch.float16, torch.float32, torch.float32)])
+def test_operand_and_output_dtypes(gd, bd, od):
+    """The per-channel log decay g, beta and the output in any of the three float dtypes (each has its own dtype code
+    in the C ABI): the oracle on the same rounded operands, its output rounded to the output's dtype or the neighbour
+    of that."""
+    B, H, D, m = 2, 4, 128, 4
+    ker = PackedKDAState(torch.zeros(B * H, D, D, device=DEV), quantizer((4, 'k', 32)), m=m, hv=H, buffer_bits=8, out_dtype=od)
+    ref = ST.KDAOracle(torch.zeros(B * H, D, D), (4, 'k', 32), m=m, hv=H, buffer_bits=8)
+    gen = torch.Generator().manual_seed(3)
+    ulp = {torch.float32: 2e-5, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[od]
+    for t in range(m):                                       # up to the first fold (later steps need the re-sync)
+        q, k, v, g, beta = kda_token(gen, B, H, D, D, torch.float32)
+        g, beta = g.to(gd), beta.to(bd)
+        o = ker.step(q.to(DEV), k.to(DEV), v.to(DEV), g.to(DEV), beta.to(DEV)).float().cpu().reshape(B * H, D)
+        r = ref.step(q, k, v, g.float(), beta.float())
+        assert ((o - r).abs() <= r.abs() * ulp + 1e-5 * r.abs().max()).all(), t

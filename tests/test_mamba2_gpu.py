@@ -362,3 +362,24 @@ def test_fp16_tokens():
     """fp16 x / B / C (dtype 2 of the C ABI) through both Mamba2 kernel kinds."""
     check(run_decode((8, 'k', 128), 8, 8, dtype=torch.float16, T=17), 'mamba2 fp16 tokens', 17, 8)
     check(run_decode((8, 'v', 32), 4, 16, dtype=torch.float16, T=9), 'mamba2 value-axis fp16 tokens', 9, 4)
+
+
+@pytest.mark.parametrize('sd,od', [(torch.float32, torch.float32), (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16),
+                                   (torch.float16, torch.float32)])
+def test_operand_and_output_dtypes(sd, od):
+    """dt, A, D, dt_bias in any of the three float dtypes and the output likewise (each has its own dtype code in the
+    C ABI): the oracle on the same rounded operands, its output rounded to the output's dtype or the neighbour."""
+    B, H, G, DK, DV, m = 2, 8, 2, 128, 64, 4
+    gen = torch.Generator().manual_seed(5)
+    A, Dp, dtb = (t.to(sd) for t in params(gen, H))
+    ker = PackedMamba2State(torch.zeros(B * H, DV, DK, device=DEV), quantizer((8, 'k', 128)), m=m, hv=H, hk=G, buffer_bits=8,
+                            out_dtype=od)
+    ref = ST.Mamba2Oracle(torch.zeros(B * H, DV, DK), (8, 'k', 128), m=m, hv=H, hk=G, buffer_bits=8)
+    ulp = {torch.float32: 2e-5, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[od]
+    for t in range(m):                                       # up to the first fold (later steps need the re-sync)
+        x, dt, Bm, C = m2_token(gen, B, H, G, DK, DV, torch.float32)
+        dt = dt.to(sd)
+        y = ker.step(x.to(DEV), dt.to(DEV), Bm.to(DEV), C.to(DEV), A.to(DEV), Dp.to(DEV), dtb.to(DEV), True,
+                     (0., float('inf'))).float().cpu().reshape(B * H, DV)
+        r = ref.step(x, dt.float(), Bm, C, A.float(), Dp.float(), dtb.float(), True, (0., float('inf')))
+        assert ((y - r).abs() <= r.abs() * ulp + 1e-5 * r.abs().max()).all(), t
