@@ -118,7 +118,9 @@ __device__ __forceinline__ float div_by(float x, const Divisor& v) { return div_
 // The fp16-valued divisor back from its correctly rounded reciprocal: 1 / rc is within 2^-22 of it, and rounding to
 // fp16's grid (11 bits, subnormals included) removes that.  For paths that are rarely taken and would otherwise keep
 // the divisor in a register beside its reciprocal.
-__device__ __forceinline__ float divisor_of(float rc) { return float(_Float16(__builtin_amdgcn_rcpf(rc))); }
+__device__ __forceinline__ float divisor_of(float rc) {
+    return fminf(float(_Float16(__builtin_amdgcn_rcpf(rc))), 3.0e38f);      // (an overflowed scale: as in scale_divisor)
+}
 
 // Quantizer scale: max(amax, 1e-8) / qmax -> fp16 (nearest even, subnormals kept) -> fp32, floored at 2^-24.  qmax is
 // 7 or 127 at every call (a constant there, so 1 / qmax is folded).
