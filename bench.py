@@ -455,9 +455,10 @@ def main():
                     help='number of sequences instead of the workload\'s own (the reference quotes batch 128 and 512)')
     ap.add_argument('--no-graph', action='store_true', help='launch eagerly instead of replaying a HIP graph')
     ap.add_argument('--mixed-fill', action='store_true',
-                    help='start slot s with s %% m tokens in its buffer, so that every step folds 1/m of the slots '
-                         '(sequences of unequal lengths, as a serving engine has them) instead of all slots folding '
-                         'on the same step; a secondary figure, the headline is the lockstep configuration')
+                    help='start the slots with 0 .. m - 1 tokens in their buffers, 1/m of them each, dealt at random over '
+                         'the batch rows, so that every step folds 1/m of the slots (sequences of unequal lengths, as '
+                         'a serving engine has them) instead of all slots folding on the same step; a secondary '
+                         'figure, the headline is the lockstep configuration')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--instances', default='', metavar='LIST',
                     help='comma-separated exclusions handed to sq_debug_select, for same-machine comparisons of the '
@@ -498,7 +499,8 @@ def main():
         return bench_convert(a, lay, views, idx, dev)
     inputs, extra = make_inputs(fam, lay, slots, layers, m, dev)
     if a.mixed_fill:
-        fill = (torch.arange(slots, device=dev, dtype=torch.int32) % m)[:, None]
+        gen = torch.Generator().manual_seed(2)
+        fill = (torch.arange(slots, dtype=torch.int32) % m)[torch.randperm(slots, generator=gen)].to(dev)[:, None]
         for V in views:
             V['NPTR'][idx.long()] = fill.expand(slots, V['NPTR'].shape[1])
     out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
