@@ -165,13 +165,15 @@ def make_inputs(fam, lay, slots, layers, m, device, seed=1):
     return out, extra
 
 
-def launch(fam, lay, views, idx, inp, extra, out):
+def launch(fam, lay, views, idx, inp, extra, out, order=None):
     if fam == 'gdn':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'])
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], out, lay.DK ** -0.5, g=inp['g'], beta=inp['beta'],
+                 order=order)
     elif fam == 'kda':
-        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out)
+        lay.step(views, idx, inp['q'], inp['k'], inp['v'], inp['g'], inp['beta'], out, order=order)
     else:
-        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'])
+        lay.step(views, idx, inp['x'], inp['dt'], inp['B'], inp['C'], out, extra['A'], extra['D'], extra['dt_bias'],
+                 order=order)
 
 
 def timed_periods(stream, run_period, warm_periods, periods):
@@ -459,6 +461,11 @@ def main():
                          'the batch rows, so that every step folds 1/m of the slots (sequences of unequal lengths, as '
                          'a serving engine has them) instead of all slots folding on the same step; a secondary '
                          'figure, the headline is the lockstep configuration')
+    ap.add_argument('--fold-order', action='store_true',
+                    help='dispatch every decode step in the order of `fold_order` (one small launch per step, inside '
+                         'the timed region, whose list serves the 24 layer launches): the rows that fold on the step '
+                         'spread evenly over the launch.  An addition to the reference\'s interface, for sequences '
+                         'out of step (--mixed-fill)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--instances', default='', metavar='LIST',
                     help='comma-separated exclusions handed to sq_debug_select, for same-machine comparisons of the '
@@ -505,10 +512,14 @@ def main():
             V['NPTR'][idx.long()] = fill.expand(slots, V['NPTR'].shape[1])
     out = torch.zeros(slots, hv, dv, device=dev, dtype=torch.bfloat16)
 
+    order = torch.zeros(slots, dtype=torch.int32, device=dev) if a.fold_order else None
+
     def period():                                           # m steps x layers launches
         for s in range(m):
+            if order is not None:                           # one list per decode step, from the first layer's counters
+                lay.fold_order(views[0], idx, out=order)
             for L in range(layers):
-                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out)
+                launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out, order)
 
     requested = (a.steps, a.warmup)
     a.steps = max(-(-a.steps // m), 1) * m                  # whole fold periods, so that any K times steps / m folds
@@ -548,6 +559,7 @@ def main():
                    'steps_requested': requested[0], 'warmup_requested': requested[1], 'steps_timed': a.steps,
                    'folds_timed': a.steps // m if not a.mixed_fill else None,
                    'fold_schedule': 'mixed (1/m of the slots per step)' if a.mixed_fill else 'lockstep',
+                   'dispatch_order': 'fold_order' if a.fold_order else 'batch order',
                    'instances_excluded': a.instances or None,
                    'state_bytes_per_slot_step': round(state_bytes_per_slot(bits, group, hv, dk, dv, m))},
         'hbm_gbs': round(achieved, 1),

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 5
+#define SQ_ABI_VERSION 6
 
 enum { SQ_F32 = 0, SQ_BF16 = 1, SQ_F16 = 2 };                /* dtype codes of float tensors */
 
@@ -99,6 +99,13 @@ typedef struct sq_gdn_args {
     const void* dt_bias; int32_t dt_bias_dtype;
     void* out;          int32_t out_dtype;
     float scale;
+    /* Optional dispatch order of the batch rows (NULL: the batch order): order[p] is the batch row that position p of
+     * the launch works on, a permutation of 0 .. rows-1.  Results do not depend on it.  No counterpart in the
+     * reference: a scheduling hint for batches whose sequences fill their buffers on different steps, where the rows
+     * that fold on this step keep their workgroups longer and their place in the launch decides when it ends (on the
+     * 256-slot int8 step: 37.5 us per launch in batch order, 32.8 with the order of sq_fold_order, 32.4 when all
+     * sequences fold together).  sq_fold_order() writes such a list from the counters. */
+    const int32_t* order;
 } sq_gdn_args;
 
 /* One KDA decode token per batch row (kda.py:192-205, 330-347): per-key-channel log decay g [rows, hv, dk];
@@ -115,6 +122,7 @@ typedef struct sq_kda_args {
     const void* beta;   int64_t s_beta;  int32_t beta_dtype;
     void* out;          int64_t s_out;   int32_t out_dtype;
     float scale;
+    const int32_t* order;   /* optional dispatch order of the rows, as in sq_gdn_args */
 } sq_kda_args;
 
 /* One Mamba2 / SSD decode token per batch row (mamba2.py:223-241, 377-396).
@@ -136,6 +144,7 @@ typedef struct sq_mamba2_args {
     int32_t dt_softplus;
     int32_t dt_clamp;   float dt_min, dt_max;
     void* out;          int64_t s_out;   int32_t out_dtype;
+    const int32_t* order;   /* optional dispatch order of the rows, as in sq_gdn_args */
 } sq_mamba2_args;
 
 /* Store fp32 states in the packed format (fold.py:123-147 `pack_vk`; with idx, GCUR and NPTR given this is
@@ -231,6 +240,15 @@ int sq_gdn_step(const sq_gdn_args* args, void* stream);
 int sq_kda_step(const sq_kda_args* args, void* stream);
 int sq_mamba2_step(const sq_mamba2_args* args, void* stream);
 int sq_pack_vk(const sq_pack_args* args, void* stream);
+/* order[0 .. rows) <- a dispatch order for the step calls' `order` (no counterpart in the reference): the rows whose
+ * buffer fills on the coming step (NPTR[idx[b] * sN] & (m-1) == m-1; idx == NULL: sequence b) dealt evenly over the
+ * eight ranges of rows that the step kernels give to the GPU's eight dies, and inside a range one after every few
+ * other rows of its first quarter; the other rows, padding rows (idx[b] <= 0) included, in batch order.  The identity
+ * when rows is not a multiple of 8 or below 64, when no row folds, or when more than every second row does.  NPTR and
+ * sN (in elements) as in sq_state; one small launch.  The counters of all layers of a model move together, so one
+ * list per decode step serves every layer. */
+int sq_fold_order(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m, int32_t rows, int32_t* order,
+                  void* stream);
 int sq_read(const sq_read_args* args, void* stream);
 int sq_gga_step(const sq_gga_args* args, void* stream);
 /* Fit + pack canonical fp32 states X [rows, hv, dk, dv] (key-major, contiguous) into slots idx[b]; their counters are

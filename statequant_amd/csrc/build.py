@@ -254,6 +254,11 @@ def generate():
                  f'&& p.kda == {k}) return run ? '
                  f'launch_read<{b}, {dk}, {g}, {tf(q)}, {tf(k)}, {tf(v)}>(p, stream) : 0;')
     d.append('    return -1;\n}')
+    d += ['int launch_fold_order(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,',
+          '                      hipStream_t stream) {',
+          '    hipLaunchKernelGGL((fold_order_kernel<FO_THREADS>), dim3(1), dim3(FO_THREADS), 0, stream, idx, NPTR, sN, m, rows, order);',
+          '    return int(hipGetLastError());',
+          '}']
     d.append('template <int DK, int DV> struct GgaTile;')
     d.append('template <class T> int launch_gga(const GgaParams&, int, hipStream_t);')
     d.append('int dispatch_gga(const GgaParams& p, int op, hipStream_t stream, bool run) {')

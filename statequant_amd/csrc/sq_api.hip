@@ -180,9 +180,11 @@ int sq_gdn_step(const sq_gdn_args* a, void* stream) {
     if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) ||
         !stride_ok(a->gate ? a->s_a : a->s_g) || !stride_ok(a->gate ? a->s_b : a->s_beta))
         return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
+    if (a->order && !aligned(a->order, 4)) return fail(SQ_E_ARG, "%s: misaligned order", who);
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
+    p.order = a->order;
     p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
     p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
     p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
@@ -223,9 +225,11 @@ int sq_kda_step(const sq_kda_args* a, void* stream) {
     if (!stride_ok(a->s_q) || !stride_ok(a->s_k) || !stride_ok(a->s_v) || !stride_ok(a->s_g) ||
         !stride_ok(a->s_beta) || !stride_ok(a->s_out))
         return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
+    if (a->order && !aligned(a->order, 4)) return fail(SQ_E_ARG, "%s: misaligned order", who);
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
+    p.order = a->order;
     p.q = a->q; p.s_q = uint32_t(a->s_q); p.q_dt = a->q_dtype;
     p.k = a->k; p.s_k = uint32_t(a->s_k); p.k_dt = a->k_dtype;
     p.v = a->v; p.s_v = uint32_t(a->s_v); p.v_dt = a->v_dtype;
@@ -251,9 +255,11 @@ int sq_mamba2_step(const sq_mamba2_args* a, void* stream) {
         return fail(SQ_E_ARG, "%s: bad dtype code", who);
     if (!stride_ok(a->s_x) || !stride_ok(a->s_dt) || !stride_ok(a->s_B) || !stride_ok(a->s_C) || !stride_ok(a->s_out))
         return fail(SQ_E_ARG, "%s: row strides must be in [0, 2^31)", who);
+    if (a->order && !aligned(a->order, 4)) return fail(SQ_E_ARG, "%s: misaligned order", who);
     p.rows = a->rows;
     set_rows(&p, a->rows);
     p.idx = a->idx;
+    p.order = a->order;
     p.x = a->x; p.s_x = uint32_t(a->s_x); p.x_dt = a->x_dtype;
     p.dt = a->dt; p.s_dt = uint32_t(a->s_dt); p.dt_dt = a->dt_dtype;
     p.B = a->B; p.s_B = uint32_t(a->s_B); p.B_dt = a->B_dtype;
@@ -307,6 +313,20 @@ int sq_pack_vk(const sq_pack_args* a, void* stream) {
     if (a->NPTR && a->sN != 0 && int64_t(p.nptr_copies) > a->sN)
         return fail(SQ_E_ARG, "%s: %d counter copies do not fit a counter stride of %lld", who, p.nptr_copies, (long long)a->sN);
     return finish(sq::dispatch_pack(p, static_cast<hipStream_t>(stream), true), who, a->lay);
+}
+
+int sq_fold_order(const int32_t* idx, const int32_t* NPTR, int64_t sN, int32_t m, int32_t rows, int32_t* order,
+                  void* stream) {
+    const char* who = "sq_fold_order";
+    if (rows < 0) return fail(SQ_E_ARG, "%s: rows %d", who, rows);
+    if (rows == 0) return SQ_OK;
+    if (!NPTR || !order || !aligned(NPTR, 4) || !aligned(order, 4) || (idx && !aligned(idx, 4)))
+        return fail(SQ_E_ARG, "%s: null or misaligned NPTR / order / idx", who);
+    if (m < 1 || (m & (m - 1))) return fail(SQ_E_ARG, "%s: m %d is not a power of two", who, m);
+    if (!stride_ok(sN)) return fail(SQ_E_ARG, "%s: counter stride must be in [0, 2^31)", who);
+    const int rc = sq::launch_fold_order(idx, NPTR, uint32_t(sN), m, rows, order, static_cast<hipStream_t>(stream));
+    if (rc != 0) return fail(SQ_E_LAUNCH, "%s: %s", who, hipGetErrorString(hipError_t(rc)));
+    return SQ_OK;
 }
 
 int sq_read(const sq_read_args* a, void* stream) {

@@ -298,4 +298,80 @@ int launch_read(const ReadParams& p, hipStream_t stream) {
     return int(hipGetLastError());
 }
 
+// A dispatch order for the step kernels (their `order` argument; no counterpart in the reference) for batches whose
+// sequences fill their buffers on different steps.  A row that folds on the coming step keeps its workgroups half
+// again as long as the others; where the batch order puts such rows decides when the launch ends: the step kernels
+// deal eight contiguous ranges of rows to the GPU's eight XCDs, which do not share work, so the folding rows should
+// be spread evenly over the ranges, and inside a range neither at the front (their writes then come in one burst)
+// nor in the last round of workgroups (they then end after everything else).  order[position] = batch row: every
+// range of R = rows / 8 positions gets F / 8 of the F folding rows (the first F % 8 ranges one more), one after
+// every s - 1 other rows from the start of the range, s = max(2, R / (4 f)) for a range with f of them -- its first
+// quarter (measured best on every kernel here: the one-wavefront kernels' folding tiles live three times as long as
+// the others and must start early; a first half costs them 20 %, the very front 1-2 % on all), more where more than
+// every eighth row folds; the other rows (padding rows among them) keep their order.  The identity for
+// rows % 8 != 0, fewer than 64 rows, no folding row, or more than every second row of a range folding.
+// One workgroup; ranks by ballots and a running count.
+constexpr int FO_THREADS = 256;
+template <int THREADS>                               // (a template only so that the header can hold it)
+__global__ __launch_bounds__(THREADS) void fold_order_kernel(const int32_t* idx, const int32_t* NPTR, uint32_t sN,
+                                                                int m, int rows, int32_t* order) {
+    constexpr int NWV = THREADS / WAVE;
+    __shared__ int wave_count[2][NWV];
+    const int tid = threadIdx.x, lane = tid % WAVE, wv = tid / WAVE;
+    auto folds = [&](int r) {
+        if (r >= rows) return false;
+        const int32_t slot = idx ? idx[r] : r;
+        if (idx && slot <= 0) return false;
+        return (NPTR[uint64_t(uint32_t(slot)) * sN] & (m - 1)) == m - 1;
+    };
+    int cnt = 0;
+    for (int r0 = 0; r0 < rows; r0 += THREADS) cnt += __popcll(__builtin_amdgcn_ballot_w64(folds(r0 + tid)));
+    if (lane == 0) wave_count[0][wv] = cnt;
+    __syncthreads();
+    int F = 0;
+    for (int w = 0; w < NWV; ++w) F += wave_count[0][w];
+    __syncthreads();
+    const int R = rows / 8, fq = F / 8, fr = F % 8;
+    if (rows % 8 != 0 || rows < 64 || F == 0 || 2 * ((F + 7) / 8) > R) {
+        for (int r = tid; r < rows; r += THREADS) order[r] = r;
+        return;
+    }
+    int base_f = 0, base_p = 0;
+    for (int r0 = 0; r0 < rows; r0 += THREADS) {
+        const int r = r0 + tid;
+        const bool f = folds(r), pl = r < rows && !f;
+        const unsigned long long bf = __builtin_amdgcn_ballot_w64(f), bp = __builtin_amdgcn_ballot_w64(pl);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        if (lane == 0) { wave_count[0][wv] = __popcll(bf); wave_count[1][wv] = __popcll(bp); }
+        __syncthreads();
+        int kf = base_f + __popcll(bf & below), kp = base_p + __popcll(bp & below);
+        for (int w = 0; w < NWV; ++w) {
+            if (w < wv) { kf += wave_count[0][w]; kp += wave_count[1][w]; }
+            base_f += wave_count[0][w];
+            base_p += wave_count[1][w];
+        }
+        __syncthreads();                             // the counts are rewritten on the next turn
+        if (f) {
+            const int c = kf % 8, j = kf / 8, fc = fq + (c < fr);
+            const int s = max(2, R / (4 * fc));
+            order[c * R + s * j + s - 1] = r;
+        } else if (pl) {
+            int t = kp, c = 0;
+            for (; c < 7; ++c) {
+                const int n = R - (fq + (c < fr));
+                if (t < n) break;
+                t -= n;
+            }
+            const int fc = fq + (c < fr);
+            int pos = t;
+            if (fc > 0) {
+                const int s = max(2, R / (4 * fc));
+                pos = t < (s - 1) * fc ? t + t / (s - 1) : t + fc;
+            }
+            order[c * R + pos] = r;
+        }
+    }
+}
+
+
 }  // namespace sq

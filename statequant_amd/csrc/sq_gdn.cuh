@@ -127,7 +127,7 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
 
 template <class T, int SPEC>
 __global__ __launch_bounds__(WAVE, 4)
-void gdn_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
+void gdn_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd,
                      int hv, int hv_shift, const GdnParams args) {
     GdnParams p = args;
     assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
@@ -150,7 +150,7 @@ void gdn_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
     constexpr int KT = KeyBuf<T>::KT;
     const bool own_key = !p.qk_per_key_head && gqa > 1;
     const LaneId l = lane_id<T>();
-    TileId tid = tile_id_lead<SPEC>(per_xcd, hv, hv_shift);          // from the leading arguments
+    TileId tid = tile_id_lead<SPEC>(order, per_xcd, hv, hv_shift);          // from the leading arguments
     const int32_t slot = idx ? idx[tid.b] : tid.b;               // scalar load: on its way while the inputs are issued
     tid.hk = p.gqa_shift >= 0 ? tid.h >> p.gqa_shift : tid.h / p.gqa;
     GdnFront<T> F;
@@ -313,7 +313,7 @@ void gdn_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
 
 template <class T, int SPEC>
 int launch_gdn(const GdnParams& p, hipStream_t stream) {
-    hipLaunchKernelGGL((gdn_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.per_xcd,
+    hipLaunchKernelGGL((gdn_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
                        p.hv, p.hv_shift, p);
     return int(hipGetLastError());
 }

@@ -73,7 +73,8 @@ struct GdnLoads {
 // a, b and fp32 A_log, dt_bias.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
+void gdn_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int hv, int hv_shift,
+                     const uint8_t* codes,
                      uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, uint32_t start_ramp,
                      SQ_TL_PARAM const GdnParams p) {
     SQ_MARK(0);                                                   // entry
@@ -122,6 +123,7 @@ void gdn_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int h
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
         tid.b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
         tid.h = (item - tid.b * ngrp) * GH + hl;
+        if (order) tid.b = order[tid.b];            // the caller's dispatch order: position -> batch row
         SQ_MARK(1);                                               // item known (the leading arguments are here)
         slot = idx ? idx[tid.b] : tid.b;
         tid.hk = (FIX || p.gqa_shift >= 0) ? tid.h >> p.gqa_shift : tid.h / p.gqa;
@@ -532,11 +534,11 @@ int launch_gdn_quad(const GdnParams& p0, hipStream_t stream) {
 #ifdef SQ_TIMELINE
     const SqTimelineBuf tl = sq_timeline_buffer();
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag,
+                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag,
                        tl.p, tl.cap, p);
 #else
     hipLaunchKernelGGL((gdn_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag, p);
+                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN, stag, p);
 #endif
     return int(hipGetLastError());
 }

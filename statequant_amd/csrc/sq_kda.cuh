@@ -22,7 +22,7 @@ __device__ __forceinline__ float kda_exp(float x) { return __builtin_amdgcn_exp2
 
 template <class T, int SPEC>
 __global__ __launch_bounds__(WAVE, 4)
-void kda_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
+void kda_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd,
                      int hv, int hv_shift, SQ_TL_PARAM const KdaParams args) {
     SQ_MARK(0);                                                   // entry
     KdaParams p = args;
@@ -43,7 +43,7 @@ void kda_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
     float* lds_c = reinterpret_cast<float*>(lds + L::FC);
 
     const LaneId l = lane_id<T>();
-    const TileId tid = tile_id_lead<SPEC>(per_xcd, hv, hv_shift);   // from the leading arguments
+    const TileId tid = tile_id_lead<SPEC>(order, per_xcd, hv, hv_shift);   // from the leading arguments
     const uint32_t b = tid.b, h = tid.h;
     const int m = p.m;
     const uint32_t um = m;
@@ -312,10 +312,10 @@ void kda_step_kernel(const int32_t* __restrict__ idx, int per_xcd,
 template <class T, int SPEC>
 int launch_kda(const KdaParams& p, hipStream_t stream) {
 #ifdef SQ_TIMELINE
-    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.per_xcd,
+    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
                        p.hv, p.hv_shift, sq_timeline_buffer().p, sq_timeline_buffer().cap, p);
 #else
-    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.per_xcd,
+    hipLaunchKernelGGL((kda_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
                        p.hv, p.hv_shift, p);
 #endif
     return int(hipGetLastError());

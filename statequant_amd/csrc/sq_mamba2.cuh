@@ -16,7 +16,7 @@ namespace sq {
 // is compiled at 234 without spills (asked for four the compiler gives up at 364, one wavefront per SIMD).
 template <class T, int SPEC>
 __global__ __launch_bounds__(WAVE, T::DK > 128 ? 2 : 4)
-void mamba2_step_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const Mamba2Params args) {
+void mamba2_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int hv, int hv_shift, const Mamba2Params args) {
     Mamba2Params p = args;
     assume_serving_case<SPEC>(p);                            // SPEC: see sq_params.h
     using L = LdsPlan<T, 1, 1>;
@@ -32,7 +32,7 @@ void mamba2_step_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
     float* lds_u = reinterpret_cast<float*>(lds + L::FU);
 
     const LaneId l = lane_id<T>();
-    const TileId tid = tile_id_lead<SPEC>(per_xcd, hv, hv_shift);   // from the leading arguments
+    const TileId tid = tile_id_lead<SPEC>(order, per_xcd, hv, hv_shift);   // from the leading arguments
     const uint32_t b = tid.b, h = tid.h, hk = p.gqa_shift >= 0 ? tid.h >> p.gqa_shift : tid.h / p.gqa;
     const int gqa = p.gqa;
     const int m = p.m;
@@ -215,7 +215,7 @@ void mamba2_step_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
 
 template <class T, int SPEC>
 int launch_mamba2(const Mamba2Params& p, hipStream_t stream) {
-    hipLaunchKernelGGL((mamba2_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.per_xcd,
+    hipLaunchKernelGGL((mamba2_step_kernel<T, SPEC>), dim3(p.rows * p.hv), dim3(WAVE), 0, stream, p.idx, p.order, p.per_xcd,
                        p.hv, p.hv_shift, p);
     return int(hipGetLastError());
 }

@@ -29,7 +29,8 @@ struct Mamba2Loads {
 // dt_bias, head counts that are powers of two.  SPEC = 0 reads all of it from the arguments.
 template <class T, int NB, int GH, int WPE, int SPEC>
 __global__ __launch_bounds__((Quad<T, NB, GH>::THREADS), WPE)
-void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, int hv_shift, const uint8_t* codes,
+void mamba2_quad_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd, int hv, int hv_shift,
+                     const uint8_t* codes,
                         uint32_t codes_stride, const int32_t* counters, uint32_t counters_stride, uint32_t start_ramp,
                         const Mamba2Params p) {
     constexpr bool FIX = SPEC > 0;
@@ -70,6 +71,7 @@ void mamba2_quad_kernel(const int32_t* __restrict__ idx, int per_xcd, int hv, in
         const int item = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
         b = (FIX || hv_shift >= 0) ? item >> (hv_shift - ilog2(GH)) : item / ngrp;
         grp = item - b * ngrp;
+        if (order) b = order[b];                    // the caller's dispatch order: position -> batch row
         slot = idx ? idx[b] : b;
     }
     const uint32_t h = grp * GH + hl;
@@ -434,7 +436,7 @@ int launch_mamba2_quad(const Mamba2Params& p0, hipStream_t stream) {
     p.per_xcd = (p.per_xcd % GH == 0) ? p.per_xcd / GH : 0;          // dealing over head groups
     const uint32_t grid = uint32_t(p.rows) * uint32_t(p.hv / GH);
     hipLaunchKernelGGL((mamba2_quad_kernel<T, NB, GH, WPE, SPEC>), dim3(grid), dim3(Quad<T, NB, GH>::THREADS),
-                       quad_lds_pad(), stream, p.idx, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
+                       quad_lds_pad(), stream, p.idx, p.order, p.per_xcd, p.hv, p.hv_shift, p.st.S, p.st.sS, p.st.NPTR, p.st.sN,
                        quad_start_ramp<Quad<T, NB, GH>, WPE>(grid, 24), p);
     return int(hipGetLastError());
 }

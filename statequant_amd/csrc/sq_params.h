@@ -33,6 +33,7 @@ struct GdnParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;                         // optional: the batch row of each position of the launch (null: natural)
     const void *q, *k, *v;
     uint32_t s_q, s_k, s_v;
     int q_dt, k_dt, v_dt;
@@ -50,6 +51,7 @@ struct KdaParams : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;
     const void *q, *k, *v, *g, *beta;
     uint32_t s_q, s_k, s_v, s_g, s_beta;
     int q_dt, k_dt, v_dt, g_dt, beta_dt;
@@ -63,6 +65,7 @@ struct Mamba2Params : LayoutKey {
     StatePtrs st;
     int rows;
     const int32_t* idx;
+    const int32_t* order;
     const void *x, *dt, *B, *C, *A, *D, *dt_bias;
     uint32_t s_x, s_dt, s_B, s_C;
     int x_dt, dt_dt, B_dt, C_dt, A_dt, D_dt, dt_bias_dt;
@@ -176,6 +179,8 @@ int dispatch_kda(const KdaParams& p, hipStream_t stream, bool run);
 int dispatch_mamba2(const Mamba2Params& p, hipStream_t stream, bool run);
 int dispatch_pack(const PackParams& p, hipStream_t stream, bool run);
 int dispatch_read(const ReadParams& p, hipStream_t stream, bool run);
+int launch_fold_order(const int32_t* idx, const int32_t* NPTR, uint32_t sN, int m, int rows, int32_t* order,
+                      hipStream_t stream);
 int dispatch_gga(const GgaParams& p, int op, hipStream_t stream, bool run);      // op: 0 step, 1 store, 2 load
 // Diagnostic choice among the instances that can serve a step call (behind sq_debug_select of the C ABI).
 void select_instances(int no_spec, int no_quad, int ghmax, int lds_pad);

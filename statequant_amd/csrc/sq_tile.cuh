@@ -133,7 +133,8 @@ __device__ __forceinline__ int row_of(const LaneId& l, int j) { return j * T::RG
 
 // Which (batch row, value head) a workgroup works on; the caller adds the key head.  Consecutive workgroup ids are
 // dealt round-robin to the 8 XCDs; with `per_xcd` set every XCD walks a contiguous range of tiles, so the heads of one
-// sequence (shared key buffer, neighbouring counters) meet in one L2.
+// sequence (shared key buffer, neighbouring counters) meet in one L2.  `order` (optional) names the batch row that each
+// position of this walk works on.
 // The arguments are the kernel's leading scalar arguments -- copies of those fields of the parameter struct.
 // Separate scalar arguments ahead of the struct are in registers when a wavefront starts, so the slot index load that
 // depends on the batch row need not wait for the argument block to be loaded.  SPEC > 0: the serving cases (a
@@ -142,12 +143,13 @@ struct TileId {
     int b, h, hk;
 };
 template <int SPEC>
-__device__ __forceinline__ TileId tile_id_lead(int per_xcd, int hv, int hv_shift) {
+__device__ __forceinline__ TileId tile_id_lead(const int32_t* order, int per_xcd, int hv, int hv_shift) {
     const int wg = blockIdx.x;
     const int tile = per_xcd ? (wg & 7) * per_xcd + (wg >> 3) : wg;
     TileId t;
     t.b = (SPEC > 0 || hv_shift >= 0) ? tile >> hv_shift : tile / hv;
     t.h = tile - t.b * hv;
+    if (order) t.b = order[t.b];                  // the caller's dispatch order: position -> batch row
     t.hk = t.h;
     return t;
 }

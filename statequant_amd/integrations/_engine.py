@@ -61,6 +61,37 @@ def slot_index(idx_all, rows):
     return idx
 
 
+def dispatch_order(ns, lay, views, slots, idx):
+    """The dispatch order of this forward pass's decode rows for ``step(..., order=)``, or None for the batch order.
+
+    Not in the reference.  A serving batch's sequences are at different points of their fold period; the rows that
+    fold on this token keep their workgroups longer, and ``fold_order`` places them where they do not decide when the
+    launch ends (a quarter to a sixth off the step time at 256 sequences).  The counters of all layers move together,
+    so the first patched layer of a pass computes the list (one small launch) and leaves it on the pass's forward
+    context, where the other layers find it.  Below 64 rows, or a row count that is no multiple of 8, ``fold_order``
+    would return the batch order: no launch then."""
+    rows = idx.shape[0]
+    if rows < 64 or rows % 8 or not hasattr(lay, 'fold_order'):           # (the mixed-width slot has no counters)
+        return None
+    ctx = ns.get_forward_context()
+    key = (slots.data_ptr(), rows, lay.m)
+    cached = getattr(ctx, '_sq_dispatch_order', None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    order = lay.fold_order(views, idx)
+    try:
+        ctx._sq_dispatch_order = (key, order)
+    except AttributeError:                                   # a context that takes no attributes: one list per layer
+        pass
+    return order
+
+
+def order_kw(ns, lay, views, slots, idx):
+    """``dispatch_order`` as keyword arguments of a ``step`` that may not know ``order`` (the mixed-width slot's)."""
+    order = dispatch_order(ns, lay, views, slots, idx)
+    return {} if order is None else {'order': order}
+
+
 def unit_stride_rows(x, rows):
     """The first ``rows`` rows of a 2-d activation with a unit inner stride (any row stride is fine for the kernels)."""
     x = x[:rows]

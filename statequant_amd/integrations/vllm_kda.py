@@ -180,7 +180,8 @@ def _forward(self, q_proj_states, k_proj_states, v_proj_states, g1, beta, core_a
         rows = E.decode_row_count(tokens, n_dec, n_pre)
         idx = E.slot_index(slots, rows)
         qd, kd, vd = (E.unit_stride_rows(x, rows).unflatten(1, (heads, d)) for x in (q, k, v))
-        lay.step(views, idx, qd, kd, vd, g1[:rows], beta[:rows], core_attn_out[0, :rows], self.head_dim ** -0.5)
+        lay.step(views, idx, qd, kd, vd, g1[:rows], beta[:rows], core_attn_out[0, :rows], self.head_dim ** -0.5,
+                 order=E.dispatch_order(M, lay, views, slots, idx))
 
     if n_pre > 0:
         span = tokens - n_dec

@@ -220,4 +220,4 @@ def conv_ssm_forward(self, projected_states, output):
         idx = E.slot_index(dslots[:, 0] if dslots.dim() == 2 else dslots, t_dec)
         lay.step(views, idx, x_d.view(t_dec, heads, hd), dt_d, B_d.view(t_dec, groups, n), C_d.view(t_dec, groups, n),
                  out_d.view(t_dec, heads, hd), self.A, self.D, self.dt_bias, dt_softplus=True,
-                 dt_limit=(0.0, float('inf')))
+                 dt_limit=(0.0, float('inf')), order=E.dispatch_order(M, lay, views, dslots, idx))

@@ -97,7 +97,7 @@ def _forward_core(self, mixed_qkv, b, a, core_attn_out):
         kw = lay.HK * lay.DK
         lay.step(views, idx, xd[:, :kw].unflatten(1, (lay.HK, lay.DK)), xd[:, kw:2 * kw].unflatten(1, (lay.HK, lay.DK)),
                  xd[:, 2 * kw:].unflatten(1, (lay.HV, lay.DV)), core_attn_out[:rows], self.head_k_dim ** -0.5,
-                 g=g[0, :rows], beta=beta[0, :rows])
+                 g=g[0, :rows], beta=beta[0, :rows], order=E.dispatch_order(O, lay, views, slots, idx))
 
     if n_pre > 0:
         q, k, v = self.rearrange_mixed_qkv(x[n_dec:])

@@ -395,7 +395,8 @@ def _forward_core(self, mixed_qkv, b, a, core_attn_out):
         k = xd[:, kw:2 * kw].unflatten(1, (lay.HK, lay.DK))
         v = xd[:, 2 * kw:].unflatten(1, (lay.HV, lay.DV))
         lay.step(views, idx, q, k, v, core_attn_out[:rows], self.head_k_dim ** -0.5,
-                 gate=(a[:rows], b[:rows], self.A_log, self.dt_bias), **self._sq_lk)
+                 gate=(a[:rows], b[:rows], self.A_log, self.dt_bias), **E.order_kw(Q, lay, views, slots, idx),
+                 **self._sq_lk)
         if self._sq_external is not None:
             _external_after_decode(self, views, idx)
 

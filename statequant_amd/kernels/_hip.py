@@ -13,14 +13,14 @@ import torch
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, 'libsqhip.so')
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 F32, BF16, F16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 FAMILY = {'gdn': 0, 'kda': 1, 'mamba2': 2}
 
 SYMBOLS = ('sq_abi_version', 'sq_strerror', 'sq_last_error', 'sq_supported', 'sq_gdn_step', 'sq_kda_step',
-           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_debug_select', 'sq_gga_step', 'sq_gga_store', 'sq_gga_load',
+           'sq_mamba2_step', 'sq_pack_vk', 'sq_read', 'sq_fold_order', 'sq_debug_select', 'sq_gga_step', 'sq_gga_store', 'sq_gga_load',
            'sq_gga_supported')
 E_UNSUPPORTED = -2
 
@@ -50,7 +50,7 @@ class SqGdnArgs(C.Structure):
                 ('b', _vp), ('s_b', _i64), ('b_dtype', _i32),
                 ('A_log', _vp), ('A_log_dtype', _i32),
                 ('dt_bias', _vp), ('dt_bias_dtype', _i32),
-                ('out', _vp), ('out_dtype', _i32), ('scale', _f32)]
+                ('out', _vp), ('out_dtype', _i32), ('scale', _f32), ('order', _vp)]
 
 
 class SqKdaArgs(C.Structure):
@@ -60,7 +60,7 @@ class SqKdaArgs(C.Structure):
                 ('v', _vp), ('s_v', _i64), ('v_dtype', _i32),
                 ('g', _vp), ('s_g', _i64), ('g_dtype', _i32),
                 ('beta', _vp), ('s_beta', _i64), ('beta_dtype', _i32),
-                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('scale', _f32)]
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('scale', _f32), ('order', _vp)]
 
 
 class SqMamba2Args(C.Structure):
@@ -72,7 +72,7 @@ class SqMamba2Args(C.Structure):
                 ('A', _vp), ('A_dtype', _i32), ('D', _vp), ('D_dtype', _i32),
                 ('dt_bias', _vp), ('dt_bias_dtype', _i32),
                 ('dt_softplus', _i32), ('dt_clamp', _i32), ('dt_min', _f32), ('dt_max', _f32),
-                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32)]
+                ('out', _vp), ('s_out', _i64), ('out_dtype', _i32), ('order', _vp)]
 
 
 class SqPackArgs(C.Structure):
@@ -135,6 +135,8 @@ def lib():
             f = getattr(L, name)
             f.restype = C.c_int
             f.argtypes = [C.POINTER(SqGgaSlots), C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]
+        L.sq_fold_order.restype = C.c_int
+        L.sq_fold_order.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
         L.sq_debug_select.restype = None
         L.sq_debug_select.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
         L.sq_gga_supported.restype = C.c_int
@@ -210,6 +212,31 @@ def read_state(lay, T, strides, nptr_stride, idx, out, kda):
     a = SqReadArgs(st=make_state(T, strides, nptr_stride), lay=lay, kda=int(kda), rows=rows, idx=ptr(idx),
                    out=out.data_ptr(), s_out=out.stride(0) if rows else 0)
     check(lib().sq_read(C.byref(a), current_stream(out.device)))
+
+
+def fold_order(NPTR, nptr_stride, m, idx, out=None):
+    """``sq_fold_order``: a dispatch order for the step calls' ``order`` argument (int32 [rows], on the device) from
+    the fill counters ``NPTR`` (per-sequence stride ``nptr_stride`` in elements) of the sequences ``idx`` (int32
+    [rows]; None: sequence b): the rows that fold on the coming step dealt evenly over the launch, the others in batch
+    order.  ``out``: where to write it (no allocation then: graph-capturable).  Results of a step never depend on
+    its order; with sequences out of step it shortens the launch.  No counterpart in the reference."""
+    rows = idx.shape[0] if idx is not None else NPTR.shape[0]
+    same_device('fold_order', NPTR, idx=idx, out=out)
+    assert NPTR.dtype == torch.int32 and (idx is None or (idx.dtype == torch.int32 and idx.is_contiguous()))
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int32, device=NPTR.device)
+    assert out.dtype == torch.int32 and out.is_contiguous() and out.shape[0] >= rows
+    check(lib().sq_fold_order(ptr(idx), NPTR.data_ptr(), nptr_stride, m, rows, out.data_ptr(),
+                              current_stream(NPTR.device)))
+    return out
+
+
+def check_order(order, rows, ref):
+    """The step wrappers' check of an ``order`` argument (None passes)."""
+    if order is not None:
+        assert order.dtype == torch.int32 and order.is_contiguous() and order.shape[0] >= rows
+        same_device('step', ref, order=order)
+    return ptr(order)
 
 
 def select_instances(no_specialised=False, no_group_kernel=False, max_heads_per_workgroup=0, lds_pad_bytes=0):

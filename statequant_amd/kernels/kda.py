@@ -61,7 +61,7 @@ def _common(st, fmt, hv, hk, dk, dv, m, buffer_bits):
     st.buffer_bits, st.qbuf = buffer_bits, buffer_bits == 8
 
 
-def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_stride):
+def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_stride, order=None):
     """One ``sq_kda_step`` call (replaces kda.py:192-205)."""
     for t in (q, k, v, g):
         assert t.stride(-1) == 1, 'unit inner stride'
@@ -75,7 +75,8 @@ def _launch(st, lay, rows, q, k, v, g, beta, out, scale, idx, T, strides, nptr_s
         v=v.data_ptr(), s_v=v.stride(0), v_dtype=_hip.dtype_code(v),
         g=g.data_ptr(), s_g=g.stride(0), g_dtype=_hip.dtype_code(g),
         beta=beta.data_ptr(), s_beta=beta.stride(0), beta_dtype=_hip.dtype_code(beta),
-        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out), scale=float(scale))
+        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out), scale=float(scale),
+        order=_hip.check_order(order, rows, T['S']))
     _hip.check(_hip.lib().sq_kda_step(ctypes.byref(a), _hip.current_stream(out.device)))
     return out
 
@@ -140,19 +141,20 @@ class KDASlotLayout(SlotLayout):
         return (f'KDASlotLayout({f}, heads={self.HV}, d_k={self.DK}, d_v={self.DV}, m={self.m}, '
                 f'buffer_bits={self.buffer_bits}, {self.nbytes} B/slot)')
 
-    def step(self, views, idx, q, k, v, g, beta, out, scale=None):
+    def step(self, views, idx, q, k, v, g, beta, out, scale=None, order=None):
         """One decode token for every batch row b on slot ``idx[b]`` (int32 [rows]; <= 0 = padding: output zeroed,
         nothing read or written) (kda.py:330-347).
 
         q, k [rows, H, d_k] raw, v [rows, H, d_v], g [rows, H, d_k] log decay, beta [rows, H] (after sigmoid): any
-        row stride, contiguous rows; out [rows, H, d_v] (row stride free).  One launch, no host syncs."""
+        row stride, contiguous rows; out [rows, H, d_v] (row stride free).  ``order``: optional dispatch order of the
+        rows (``fold_order``; not in the reference).  One launch, no host syncs."""
         rows = idx.shape[0]
         if rows == 0:
             return out
         assert idx.dtype == torch.int32 and idx.is_contiguous()
         T, strides, sN = slot_state(views)
         return _launch(self, self._layout_struct(), rows, q, k, v, g, beta, out,
-                       self.DK ** -0.5 if scale is None else scale, idx, T, strides, sN)
+                       self.DK ** -0.5 if scale is None else scale, idx, T, strides, sN, order)
 
     @torch.no_grad()
     def read(self, views, idx):

@@ -70,7 +70,8 @@ def _common(st, fmt, hv, hk, dk, dv, m, buffer_bits):
     st.buffer_bits, st.qbuf = buffer_bits, buffer_bits == 8
 
 
-def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx, T, strides, nptr_stride):
+def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx, T, strides, nptr_stride,
+            order=None):
     """One ``sq_mamba2_step`` call (replaces mamba2.py:223-241)."""
     assert x.stride(-1) == 1 and B.stride(-1) == 1 and C.stride(-1) == 1 and dt.stride(-1) == 1
     assert x.stride(-2) == st.DV and out.stride(-1) == 1 and out.stride(-2) == st.DV
@@ -89,7 +90,8 @@ def _launch(st, lay, rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limi
         D=_hip.ptr(D), D_dtype=_hip.dtype_code(D) if D is not None else 0,
         dt_bias=_hip.ptr(dt_bias), dt_bias_dtype=_hip.dtype_code(dt_bias) if dt_bias is not None else 0,
         dt_softplus=int(bool(dt_softplus)), dt_clamp=int(clamp), dt_min=lo, dt_max=hi,
-        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out))
+        out=out.data_ptr(), s_out=out.stride(0), out_dtype=_hip.dtype_code(out),
+        order=_hip.check_order(order, rows, T['S']))
     _hip.check(_hip.lib().sq_mamba2_step(ctypes.byref(a), _hip.current_stream(out.device)))
     return out
 
@@ -157,19 +159,20 @@ class Mamba2SlotLayout(SlotLayout):
                 f'm={self.m}, buffer_bits={self.buffer_bits}, {self.nbytes} B/slot)')
 
     def step(self, views, idx, x, dt, B, C, out, A, D=None, dt_bias=None, dt_softplus=True,
-             dt_limit=(0., float('inf'))):
+             dt_limit=(0., float('inf')), order=None):
         """One decode token for every batch row b on slot ``idx[b]`` (int32 [rows]; <= 0 = padding: output zeroed,
         nothing read or written) (mamba2.py:377-396).
 
         x [rows, H, d_v], dt [rows, H] (raw: + dt_bias, softplus, clamp in the kernel), B / C [rows, G, d_k]: any row
-        stride, contiguous rows; out [rows, H, d_v] (row stride free); A [H] (= -exp(A_log)), D, dt_bias [H] or None."""
+        stride, contiguous rows; out [rows, H, d_v] (row stride free); A [H] (= -exp(A_log)), D, dt_bias [H] or None.
+        ``order``: optional dispatch order of the rows (``fold_order``; not in the reference)."""
         rows = idx.shape[0]
         if rows == 0:
             return out
         assert idx.dtype == torch.int32 and idx.is_contiguous()
         T, strides, sN = slot_state(views)
         return _launch(self, self._layout_struct(), rows, x, dt, B, C, out, A, D, dt_bias, dt_softplus, dt_limit, idx,
-                       T, strides, sN)
+                       T, strides, sN, order)
 
 
 __all__ = ['PackedMamba2State', 'Mamba2SlotLayout', 'mamba2_recurrence']

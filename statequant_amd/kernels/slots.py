@@ -144,7 +144,17 @@ class SlotLayout:
         return torch.zeros(num_slots, self.nbytes, dtype=torch.uint8, device=device)
 
     # -- decode -----------------------------------------------------------------------------------------------
-    def step(self, views, idx, q, k, v, out, scale, *, g=None, beta=None, gate=None, fused='layout'):
+    def fold_order(self, views, idx, out=None):
+        """A dispatch order for ``step(..., order=)`` (int32 [B] on the device; not in the reference): the rows whose
+        buffer fills on the coming step spread evenly over the launch, the others in batch order.  For batches whose
+        sequences are at different points of their fold period (a serving engine's): a folding row keeps its
+        workgroups longer, and left where the batch order has them such rows end a launch late.  One small launch,
+        no host synchronization; with ``out`` given no allocation either.  The counters of all layers of a model
+        move together, so one list per decode step serves every layer."""
+        assert idx.dtype == torch.int32 and idx.is_contiguous()
+        return _hip.fold_order(views['NPTR'], slot_state(views)[2], self.m, idx, out)
+
+    def step(self, views, idx, q, k, v, out, scale, *, g=None, beta=None, gate=None, fused='layout', order=None):
         """One decode token for every batch row b, on slot ``idx[b]`` (int32 [B]; <= 0 = padding row)
         (slots.py:124-187).
 
@@ -153,6 +163,8 @@ class SlotLayout:
         out     [B, hv, d_v] contiguous; written (zeros on padding rows)
         g, beta [B, hv] log decay and (sigmoided) beta;  or ``gate=(a, b, A_log, dt_bias)``: formed in the kernel as
                 g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b)
+        order   optional int32 [B] dispatch order (``fold_order``; not in the reference): which batch row each position
+                of the launch works on.  Results do not depend on it
         One kernel launch on the current stream, no allocation, no host synchronization: graph-capturable.  Each
         row's buffer counter advances; rows whose buffer fills are folded and re-rounded in place.
         """
@@ -174,7 +186,8 @@ class SlotLayout:
             q=q.data_ptr(), s_q=q.stride(0), q_dtype=_hip.dtype_code(q),
             k=k.data_ptr(), s_k=k.stride(0), k_dtype=_hip.dtype_code(k),
             v=v.data_ptr(), s_v=v.stride(0), v_dtype=_hip.dtype_code(v), qk_per_key_head=1,
-            out=out.data_ptr(), out_dtype=_hip.dtype_code(out), scale=float(scale))
+            out=out.data_ptr(), out_dtype=_hip.dtype_code(out), scale=float(scale),
+            order=_hip.check_order(order, B, views['S']))
         if gate is not None:
             assert ga.stride(-1) == 1 and gb.stride(-1) == 1 and A_log.is_contiguous() and dt_bias.is_contiguous()
             a.gate = 1

@@ -149,8 +149,13 @@ def chunk_scan_mamba2(x, dt, A, B, C, chunk_size=None, D=None, z=None, dt_bias=N
 def engine_module(rec, context, **extra):
     """A namespace with the engine-module attributes the forwards use; ``context['md']`` is the dict the forward
     context hands out as ``attn_metadata``."""
+    def forward_context():                                   # one object per pass: a test starts a new pass by
+        fc = context.setdefault('fc', SimpleNamespace())     # dropping context['fc']
+        fc.attn_metadata = context.get('md')
+        return fc
+
     ns = SimpleNamespace(
-        get_forward_context=lambda: SimpleNamespace(attn_metadata=context.get('md')),
+        get_forward_context=forward_context,
         is_conv_state_dim_first=lambda: True,
         causal_conv1d_fn=rec.wrap('conv_varlen', conv_varlen),
         causal_conv1d_update=rec.wrap('conv_update', conv_update),

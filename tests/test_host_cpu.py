@@ -148,7 +148,7 @@ def test_library_exports_every_declared_symbol():
     L = _hip.lib()
     for name in declared:
         assert hasattr(L, name), name
-    assert L.sq_abi_version() == _hip.ABI_VERSION == 5
+    assert L.sq_abi_version() == _hip.ABI_VERSION == 6
     assert L.sq_strerror(0) == b'ok'
     lay = _hip.SqLayout(bits=8, axis_k=1, group=128, buffer_bits=8, m=8, hv=32, hk=16, dk=128, dv=128)
     assert L.sq_supported(0, ctypes.byref(lay)) == 1
@@ -158,6 +158,8 @@ def test_library_exports_every_declared_symbol():
     assert L.sq_gdn_step(None, None) == -1 and b'null args' in L.sq_last_error()
     a = _hip.SqGdnArgs(lay=_hip.SqLayout(bits=5, axis_k=1, group=32, buffer_bits=8, m=8, hv=4, hk=2, dk=64, dv=64))
     assert L.sq_gdn_step(ctypes.byref(a), None) == -2 and b'bits' in L.sq_last_error()
+    assert L.sq_fold_order(None, None, 0, 8, 64, None, None) == -1 and b'NPTR' in L.sq_last_error()
+    assert L.sq_fold_order(None, None, 0, 8, 0, None, None) == 0               # no rows: nothing to do
 
 
 def test_ctypes_structs_match_the_header():

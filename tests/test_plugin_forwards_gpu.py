@@ -357,3 +357,64 @@ def test_mamba2_conv_ssm_forward():
     assert book.worst < 1e-2, book.worst
     assert torch.equal(layer.kv_cache[1][0], null_before)
     print(f'[mamba2 {fmt}] max rel |y - y_oracle| over decode rows {book.worst:.2e}')
+
+
+def test_dispatch_order_is_made_once_per_forward_pass(monkeypatch):
+    """Two GDN layers of one model, 64 decode sequences out of step: the first layer of a pass makes the dispatch
+    order from the counters, the second finds it on the forward context; a new pass makes a new one; and the layers'
+    results are those of the same passes without any order, bit for bit."""
+    from statequant_amd.integrations import _engine as E
+    hk, hv, dk, dv, rows = 2, 4, 64, 64, 64
+    gen = torch.Generator().manual_seed(47)
+    lay = SlotLayout(sq.Quantizer(8, 'k', 64), hv, hk, dk, dv, m=M, buffer_bits=8)
+    rec, ctx = F.Recorder(), {}
+    ns = F.engine_module(rec, ctx)
+    vllm_plugin._state['Q'] = ns
+    C = 2 * hk * dk + hv * dv
+    r = lambda *s: torch.randn(*s, generator=gen).to(DEV)          # noqa: E731
+
+    def layers():
+        out = []
+        g2 = torch.Generator().manual_seed(48)
+        for L in range(2):
+            blob = lay.alloc(rows + 1, DEV)
+            V = lay.views(blob)
+            lay.write(V, torch.arange(1, rows + 1, device=DEV), (torch.randn(rows, hv, dv, dk, generator=g2) * 0.4).to(DEV))
+            V['NPTR'][1:] = (torch.arange(rows, device=DEV, dtype=torch.int32) % M)[:, None]
+            out.append(SimpleNamespace(
+                prefix=f'model.layers.{L}.linear_attn', activation='silu', head_k_dim=dk, head_v_dim=dv,
+                conv1d=SimpleNamespace(weight=torch.randn(C, 1, KC, generator=g2).to(DEV) * 0.5, bias=None),
+                A_log=torch.randn(hv, generator=g2).to(DEV) * 0.3 - 1.0, dt_bias=torch.randn(hv, generator=g2).to(DEV) * 0.3,
+                kv_cache=(torch.zeros(rows + 1, C, KC - 1, device=DEV), blob),
+                _sq_layout=lay, _sq_views=None, _sq_external=None, _sq_lk={},
+                chunk_gated_delta_rule=ns.chunk_gated_delta_rule,
+                _warmup_prefill_kernels=lambda *a: pytest.fail('warm-up on a step with metadata')))
+        return out
+
+    ordered, plain = layers(), layers()
+    calls, use = [], {'order': True}
+    real_fold_order, real_dispatch_order = SlotLayout.fold_order, E.dispatch_order
+    monkeypatch.setattr(SlotLayout, 'fold_order', lambda self, *a, **k: calls.append(1) or real_fold_order(self, *a, **k))
+    monkeypatch.setattr(E, 'dispatch_order', lambda *a, **k: real_dispatch_order(*a, **k) if use['order'] else None)
+    slots = list(range(1, rows + 1))
+    for step in range(M + 2):
+        md = F.gdn_metadata(slots, [], [], [], DEV)
+        x_in, a, b = r(rows, C), r(rows, hv) * 0.5 - 1, r(rows, hv)
+        outs = {}
+        for name, group in (('ordered', ordered), ('plain', plain)):
+            ctx.pop('fc', None)                              # a new forward pass
+            ctx['md'] = {layer.prefix: md for layer in group}
+            use['order'] = name == 'ordered'
+            before = len(calls)
+            outs[name] = []
+            for layer in group:
+                out = torch.full((rows, hv, dv), 7.0, device=DEV)
+                vllm_plugin._forward_core(layer, x_in, b, a, out)
+                outs[name].append(out)
+            assert len(calls) - before == (1 if name == 'ordered' else 0), (name, step)
+            assert hasattr(ctx['fc'], '_sq_dispatch_order') == (name == 'ordered')
+        for o1, o2, l1, l2 in zip(outs['ordered'], outs['plain'], ordered, plain):
+            assert torch.equal(o1, o2), step
+            assert torch.equal(l1.kv_cache[1], l2.kv_cache[1]), step
+    n = lay.views(ordered[0].kv_cache[1])['NPTR'][1:, 0].tolist()
+    assert len(set(n)) == M                                  # the sequences were out of step throughout
