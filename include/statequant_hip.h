@@ -103,7 +103,7 @@ typedef struct sq_gdn_args {
      * the launch works on, a permutation of 0 .. rows-1.  Results do not depend on it.  No counterpart in the
      * reference: a scheduling hint for batches whose sequences fill their buffers on different steps, where the rows
      * that fold on this step keep their workgroups longer and their place in the launch decides when it ends (on the
-     * 256-slot int8 step: 37.5 us per launch in batch order, 32.8 with the order of sq_fold_order, 32.4 when all
+     * 256-slot int8 step: 38.4 us per launch in batch order, 33.0 with the order of sq_fold_order, 32.2 when all
      * sequences fold together).  sq_fold_order() writes such a list from the counters. */
     const int32_t* order;
 } sq_gdn_args;
