@@ -237,3 +237,36 @@ def test_order_under_graph_replay():
             assert torch.equal(outs[0][L], outs[1][L]), (rep, L)
             assert torch.equal(blobs[0][L], blobs[1][L]), (rep, L)
     assert len(seen) > 1                                     # the order followed the counters from replay to replay
+
+
+@pytest.mark.parametrize('fmt', [(8, 'k', 128), (4, 'k', 64)])
+def test_full_size_batch_out_of_step(fmt):
+    """The benchmark's shape (256 sequences, 32 / 16 heads, d 128) with the fill levels dealt at random: stepped with
+    ``fold_order``'s list and in batch order, the two blobs and the outputs stay equal bit for bit through two fold
+    periods, and every sequence's counter advances by one per step."""
+    HV, HK, D, m, rows = 32, 16, 128, 8, 256
+    lay = SlotLayout(sq.Quantizer(*fmt), HV, HK, D, D, m=m, buffer_bits=8)
+    gen = torch.Generator().manual_seed(19)
+    idx = (torch.randperm(rows, generator=gen) + 1).to(torch.int32).to(DEV)
+    blobs = [lay.alloc(rows + 1, DEV) for _ in range(2)]
+    views = [lay.views(b) for b in blobs]
+    S0 = (torch.randn(rows, HV, D, D, generator=gen) * 0.3).to(DEV)
+    fill0 = torch.randint(0, m, (rows,), generator=gen).to(torch.int32).to(DEV)
+    for V in views:
+        lay.write(V, idx.long(), S0)
+        V['NPTR'][idx.long()] = fill0[:, None]
+    del S0
+    order = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    moved = 0
+    for t in range(2 * m + 1):
+        q, k, v, g, beta = (x.to(DEV) for x in gdn_token(gen, rows, HV, HK, D, D, dtype=torch.bfloat16))
+        outs = [torch.full((rows, HV, D), 3.0, device=DEV, dtype=torch.bfloat16) for _ in range(2)]
+        lay.step(views[0], idx, q, k, v, outs[0], D ** -0.5, g=g, beta=beta)
+        lay.fold_order(views[1], idx, out=order)
+        moved += int((order != torch.arange(rows, device=DEV, dtype=torch.int32)).any())
+        lay.step(views[1], idx, q, k, v, outs[1], D ** -0.5, g=g, beta=beta, order=order)
+        assert torch.equal(outs[0], outs[1]), t
+        assert torch.equal(blobs[0], blobs[1]), t
+        want = (fill0 + t + 1) % m
+        assert torch.equal(views[1]['NPTR'][idx.long(), 0], want), t
+    assert moved == 2 * m + 1                                # every step had rows to place
