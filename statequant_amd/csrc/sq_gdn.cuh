@@ -125,8 +125,10 @@ __device__ __forceinline__ void gdn_issue(const GdnParams& p, const GdnAddr<T>& 
     for (int t = 0; t < GdnFront<T>::KT; ++t) { const int i = l.rg + T::RG * t; f.gb[t] = a.GBh[i < nl ? i : nl - 1]; }
 }
 
+// Register target: four wavefronts per SIMD (what the tile's LDS admits), except the 128 x 128 int8 tile with
+// value-axis groups, which spills at 128 registers and is faster at three (136 registers: 45.6 -> 43.5 us per launch).
 template <class T, int SPEC>
-__global__ __launch_bounds__(WAVE, 4)
+__global__ __launch_bounds__(WAVE, (T::AXV && T::BITS == 8 && T::DK == 128 && T::DV == 128) ? 3 : 4)
 void gdn_step_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ order, int per_xcd,
                      int hv, int hv_shift, const GdnParams args) {
     GdnParams p = args;
