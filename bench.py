@@ -194,6 +194,39 @@ def timed_periods(stream, run_period, warm_periods, periods):
     return wall, [ev[i].elapsed_time(ev[i + 1]) for i in range(periods)]
 
 
+def out_of_step_figures(fam, lay, views, idx, inputs, extra, out, m, layers, slots, stream, dev, periods=16):
+    """Secondary figures of the default run: the same launches with the fill levels dealt at random over the batch
+    rows (--mixed-fill), in batch order and in the order of `fold_order` (its launch included); us per launch."""
+    gen = torch.Generator().manual_seed(2)
+    fill = (torch.arange(slots, dtype=torch.int32) % m)[torch.randperm(slots, generator=gen)].to(dev)[:, None]
+    order = torch.zeros(slots, dtype=torch.int32, device=dev)
+    res = {}
+    with torch.cuda.stream(stream):
+        for name, ordered in (('batch_order_us', False), ('fold_order_us', True)):
+            stream.synchronize()
+            for V in views:
+                V['NPTR'][idx.long()] = fill.expand(slots, V['NPTR'].shape[1])
+
+            def period():
+                for s in range(m):
+                    if ordered:
+                        lay.fold_order(views[0], idx, out=order)
+                    for L in range(layers):
+                        launch(fam, lay, views[L], idx, inputs[s * layers + L], extra, out, order if ordered else None)
+
+            period()
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                period()
+            _, per_ms = timed_periods(stream, graph.replay, 4, periods)
+            res[name] = round(sum(per_ms) * 1e3 / (periods * m * layers), 3)
+    res['what'] = ('sequences out of step: 1/m of the slots fold on every step, fill levels dealt at random over the '
+                   'rows (--mixed-fill); fold_order_us: dispatched in the order of sq_fold_order, one list per decode '
+                   'step, its launch inside the timed region (--fold-order)')
+    return res
+
+
 def period_stats(per_ms, launches_per_period):
     """Per-launch microseconds of every timed period and their min / median / mean."""
     us = sorted(x * 1e3 / launches_per_period for x in per_ms)
@@ -572,6 +605,8 @@ def main():
                                'frac': round(tot_gbs / HBM_PEAK_GBS, 4),
                                'counts': 'state + live buffer slots + append + counters + inputs + output'}},
     }
+    if use_graph and not a.mixed_fill and not a.fold_order and hasattr(lay, 'fold_order'):
+        res['out_of_step'] = out_of_step_figures(fam, lay, views, idx, inputs, extra, out, m, layers, slots, stream, dev)
     if not a.no_cpu_baseline:
         res['cpu_baseline'] = cpu_baseline(a.workload, m, a.cpu_budget)
         res['cpu_baseline_c1'] = cpu_baseline_c1()
