@@ -33,8 +33,9 @@ targets.
 
 Secondary figures: ``--workload`` (the other formats and families; ``gga4-pw8`` is the mixed-width GGA / STEP slot,
 which re-fits every head at every token), ``--slots N`` (other batch sizes), ``--op write |
-read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots)
-and ``--calibrate-copy`` (the known-size copy that the HBM counters are scaled by).
+read`` (the prefill-side kernels), ``--mixed-fill`` (sequences of unequal lengths: every step folds 1/m of the slots),
+``--fold-order`` (the step calls' optional dispatch order, for that case; the default run reports both as
+``out_of_step``) and ``--calibrate-copy`` (the known-size copy that the HBM counters are scaled by).
 """
 import argparse
 import json
